@@ -1,0 +1,153 @@
+/*
+ * C ABI of libstof_hip.so - the gfx950 (MI355X) implementation of STOF's hot path:
+ * block-masked multi-head attention driven by a full/partial/empty block LUT and
+ * the fused encoder operators (GEMM+bias+activation, GEMM+bias+residual+LayerNorm,
+ * bias+residual+LayerNorm).
+ *
+ * Conventions
+ *   - every pointer is a DEVICE pointer unless stated otherwise; the library never
+ *     allocates, frees or retains caller memory;
+ *   - all activations are IEEE fp16 (two bytes); accumulation and statistics are fp32;
+ *   - `stream` is a hipStream_t passed as void* (NULL = the null stream); launches
+ *     are asynchronous, nothing synchronises;
+ *   - every function returns 0 on success or a negative STOF_ERR_* code; no launch
+ *     is made when an argument check fails.  stof_status_string() names a code.
+ *
+ * Reference interfaces replaced (paths relative to the reference tree):
+ *   stof_block_attn_fwd        launch_block_attn_mask      src/ops/src/block_attn_mask.cpp:8-15,
+ *                                                           src/ops/src/block_attn_mask_cuda.cu:6026-6322
+ *   stof_pack_mask_bits        (the fp16 additive blocks built at src/util/masks.py:159-166,
+ *                               consumed at block_attn_mask_cuda.cu:3680-3698, and the fp16
+ *                               row_mask of launcher_rowwise_attn_mask, rowwise_attn_mask_cuda.cu:89-101)
+ *   stof_rowwise_attn_fwd      launcher_rowwise_attn_{full,sliding,mask}
+ *                                                           src/ops/src/rowwise_attn_full.cpp:8-12,
+ *                                                           rowwise_attn_sliding.cpp:8-12, rowwise_attn_mask.cpp:8-12
+ *   stof_bias_res_ln           batched_bias_layer_norm_fused_kernel
+ *                                                           src/triton_template/add_layernorm.py:19-107
+ *   stof_gemm_bias_act         the first product + bias + GELU of triton_matmul_batch_kernel
+ *                                                           src/triton_template/gemm_gemm.py:99-150
+ *                              and matmul + bias (+ F.gelu)  src/benchmk_end2end.py:80-81
+ *   stof_gemm_bias_res_ln      batch_matmul_bias_layernorm_kernel
+ *                                                           src/triton_template/gemm_add_layernorm.py:78-144
+ *                              and matmul + bias + residual + F.layer_norm, src/benchmk_end2end.py:73-76
+ */
+#ifndef STOF_ABI_H
+#define STOF_ABI_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define STOF_ABI_VERSION 1
+
+enum {
+  STOF_OK = 0,
+  STOF_ERR_NULL_POINTER = -1,   /* a required pointer is NULL */
+  STOF_ERR_BAD_SHAPE = -2,      /* a size is <= 0, not divisible as required, or too large */
+  STOF_ERR_UNSUPPORTED = -3,    /* head size / block size / activation not implemented */
+  STOF_ERR_MISALIGNED = -4,     /* pointer or stride breaks the 16-byte vector-access rule */
+  STOF_ERR_LAUNCH = -5,         /* hipGetLastError() reported a failure after the launch */
+  STOF_ERR_BAD_LUT = -6         /* inconsistent LUT description (host-visible part) */
+};
+
+/* activation selector of stof_gemm_bias_act */
+enum { STOF_ACT_NONE = 0, STOF_ACT_GELU_ERF = 1, STOF_ACT_GELU_TANH = 2, STOF_ACT_RELU = 3 };
+
+/* rowwise front-end selector of stof_rowwise_attn_fwd */
+enum { STOF_ROW_FULL = 0, STOF_ROW_SLIDING = 1, STOF_ROW_MASK = 2 };
+
+int stof_abi_version(void);
+const char* stof_status_string(int status);
+
+/*
+ * Block-masked multi-head attention, forward.
+ *   out[b,h,i,:] = sum_j softmax_j( scale * q[b,h,i,:].k[b,h,j,:]  over allowed j ) v[b,h,j,:]
+ * where the allowed (i,j) are described by the block LUT: key blocks listed in LOAD for
+ * query block i/block_m are visited in order; one that is next in the PART list uses the
+ * 64-bit row masks part_bitmask[slot*block_m + (i % block_m)] (bit j%block_n set = allowed),
+ * one that is next in the FULL list is unmasked, any other is skipped (the rule of
+ * block_attn_mask_cuda.cu:3675-3700).  Query rows without any allowed key produce zeros.
+ *
+ * Tensors are addressed as base + b*stride_b + h*stride_h + s*stride_s + d (strides in
+ * ELEMENTS, d contiguous), separately for q, k, v and out, so [B,H,S,D], [B,S,H,D] and
+ * slices of a packed [B,S,3*H*D] projection are all accepted without a copy.  out may
+ * alias q (the reference returns its result in q).
+ *
+ * LUT arrays are int32.  With lut_batch_stride == 0 the three row-pointer arrays have
+ * S/block_m + 1 entries and are shared by every (b,h) as in the reference; otherwise
+ * sample b uses row pointers at offset b*lut_batch_stride, whose values are absolute
+ * offsets into the (concatenated) column lists and bitmask slots.
+ *
+ * Supported: D == 64, block_m == block_n == 64, S % 64 == 0.  num_warps of the
+ * reference launcher has no counterpart: one wavefront owns one query block.
+ */
+int stof_block_attn_fwd(
+    const void* q, const void* k, const void* v, void* out,
+    const int32_t* full_row_ptr, const int32_t* full_col_idx,
+    const int32_t* part_row_ptr, const int32_t* part_col_idx, const uint64_t* part_bitmask,
+    const int32_t* load_row_ptr, const int32_t* load_col_idx,
+    int block_m, int block_n, float softmax_scale,
+    const int64_t q_strides[3], const int64_t k_strides[3],
+    const int64_t v_strides[3], const int64_t out_strides[3],
+    int batch_size, int seq_len, int head_num, int head_size,
+    int64_t lut_batch_stride, void* stream);
+
+/*
+ * Pack fp16 mask rows into bit rows: dst[r*(cols/64) + w] bit t = pred(src[r*ld + 64*w + t]).
+ * additive != 0: src holds additive masks (0 = keep, -10000 = drop), pred(x) = x > -5000;
+ * additive == 0: src holds 0/1 masks, pred(x) = x > 0 (the test of rowwise_attn_mask_cuda.cu:58).
+ * The stack of partial blocks [n,64,64] is packed with rows = n*64, cols = 64, ld = 64.
+ * cols % 64 == 0.  HBM-bound: 2*rows*cols bytes in, rows*cols/8 bytes out.
+ */
+int stof_pack_mask_bits(const void* src, uint64_t* dst, int64_t rows, int64_t cols, int64_t ld,
+                        int additive, void* stream);
+
+/*
+ * Row-wise attention front-ends (dense/causal, sliding window, element mask) with the
+ * reference's result layout out[B, S, H*D] (src/ops/package_op.py:11-48).
+ *   kind STOF_ROW_FULL:    keys j <= (is_causal ? i : S-1)
+ *   kind STOF_ROW_SLIDING: additionally j > i - bandwidth
+ *   kind STOF_ROW_MASK:    additionally bit j of mask_bits[i*(S/64) + j/64] set
+ * Unlike the reference kernels the softmax is max-subtracted (no overflow) and rows
+ * without an allowed key produce zeros.  q, k, v contiguous [B,H,S,D], D == 64, S % 64 == 0.
+ */
+int stof_rowwise_attn_fwd(
+    const void* q, const void* k, const void* v, void* out,
+    int kind, int is_causal, int bandwidth, const uint64_t* mask_bits,
+    int batch_size, int seq_len, int head_num, int head_size, void* stream);
+
+/*
+ * y[m,:] = LayerNorm(x[m,:] + bias[:] + residual[m,:]) * gamma + beta     (fp32 statistics)
+ * bias, residual, gamma, beta may be NULL (treated as 0, 0, 1, 0); mean/rstd (fp32 [M]) may
+ * be NULL.  N % 8 == 0, N <= 8192, rows are N contiguous elements at ld_* element pitch.
+ * HBM-bound: 2*M*N bytes per operand that is present.
+ */
+int stof_bias_res_ln(const void* x, const void* bias, const void* residual,
+                     const void* gamma, const void* beta, void* y,
+                     float* mean, float* rstd,
+                     int64_t M, int64_t N, float eps, void* stream);
+
+/*
+ * C[M,N] = act( A[M,K] @ W^T + bias[N] ) with W given as Wt[N,K] (K contiguous, the
+ * nn.Linear orientation).  A rows at pitch lda, C rows at pitch ldc (elements).
+ * K % 32 == 0, N % 8 == 0; M arbitrary.  bias may be NULL.
+ */
+int stof_gemm_bias_act(const void* A, const void* Wt, const void* bias, void* C,
+                       int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldc,
+                       int act, void* stream);
+
+/*
+ * C[M,N] = LayerNorm( A[M,K] @ W^T + bias[N] + residual[M,N] ) * gamma + beta, the whole
+ * row of N owned by one workgroup so the pre-normalisation values never reach HBM.
+ * N in {256, 512, 768, 1024}; K % 32 == 0.  bias / residual / gamma / beta may be NULL.
+ */
+int stof_gemm_bias_res_ln(const void* A, const void* Wt, const void* bias, const void* residual,
+                          const void* gamma, const void* beta, void* C,
+                          int64_t M, int64_t N, int64_t K, float eps, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* STOF_ABI_H */

@@ -1,0 +1,47 @@
+"""Build libstof_hip.so: every .hip file of this directory, compiled for gfx950 with hipcc
+and linked into one shared library placed next to the Python loader (stof/libstof_hip.so).
+
+Usage:  python csrc/build.py [--force]
+The library has a plain C ABI (include/stof_abi.h); it links against the HIP runtime only.
+"""
+import os
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(os.path.dirname(HERE))
+OUT = os.path.join(os.path.dirname(HERE), "stof", "libstof_hip.so")
+
+FLAGS = [
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
+    # packed-FP32 VALU forms are kept out of the generated code
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-I" + os.path.join(ROOT, "include"), "-I" + HERE,
+    "-Wno-unused-command-line-argument",
+]
+
+
+def sources():
+    return sorted(os.path.join(HERE, f) for f in os.listdir(HERE) if f.endswith(".hip"))
+
+
+def build(force=True, verbose=True):
+    srcs = sources()
+    deps = srcs + [os.path.join(HERE, "stof_common.h"), os.path.join(ROOT, "include", "stof_abi.h")]
+    if not force and os.path.exists(OUT) and all(os.path.getmtime(OUT) >= os.path.getmtime(d) for d in deps):
+        return OUT
+    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+    cmd = [hipcc] + FLAGS + srcs + ["-o", OUT]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    err = "\n".join(l for l in r.stderr.splitlines() if "packed-fp32-ops" not in l)
+    if r.returncode != 0:
+        raise RuntimeError("hipcc failed:\n" + err)
+    if verbose and err.strip():
+        print(err)
+    return OUT
+
+
+if __name__ == "__main__":
+    print(build(force=True))

@@ -1,0 +1,112 @@
+// bias + residual + LayerNorm for gfx950: y = LN(x + bias + residual) * gamma + beta.
+//
+// Replaces batched_bias_layer_norm_fused_kernel (src/triton_template/add_layernorm.py:19-84),
+// which walks each row three times from global memory.  Here one wavefront owns one row,
+// reads it once with 16-byte loads, keeps it in registers for the exact two-pass
+// mean / variance, and writes it once: the kernel moves the algorithmic minimum of bytes
+// and is bound by HBM bandwidth.
+#include "stof_common.h"
+
+namespace {
+
+struct LnParams {
+  const half_t* x; const half_t* bias; const half_t* res; const half_t* gamma; const half_t* beta;
+  half_t* y; float* mean; float* rstd;
+  int64_t M; int N; float eps; float inv_n;
+};
+
+__device__ __forceinline__ void load8(const half_t* p, float (&v)[8]) {
+  const half8_t h = *reinterpret_cast<const half8_t*>(p);
+#pragma unroll
+  for (int i = 0; i < 8; ++i) v[i] = (float)h[i];
+}
+
+// CH = 16-byte chunks per lane; the row has at most 64*CH chunks (N <= 512*CH).
+template <int CH>
+__global__ __launch_bounds__(256) void bias_res_ln_kernel(const LnParams p) {
+  const int lane = threadIdx.x & 63;
+  const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= p.M) return;
+  const int nchunk = p.N >> 3;
+  const half_t* xr = p.x + row * p.N;
+  const half_t* rr = p.res ? p.res + row * p.N : nullptr;
+
+  float v[CH][8];
+  float s = 0.f;
+#pragma unroll
+  for (int c = 0; c < CH; ++c) {
+    const int ch = lane + 64 * c;
+    if (ch < nchunk) {
+      load8(xr + 8 * ch, v[c]);
+      if (p.bias) { float t[8]; load8(p.bias + 8 * ch, t);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v[c][i] += t[i]; }
+      if (rr) { float t[8]; load8(rr + 8 * ch, t);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v[c][i] += t[i]; }
+#pragma unroll
+      for (int i = 0; i < 8; ++i) s += v[c][i];
+    } else {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) v[c][i] = 0.f;
+    }
+  }
+  const float mean = wave_sum(s) * p.inv_n;
+  float q = 0.f;
+#pragma unroll
+  for (int c = 0; c < CH; ++c)
+    if (lane + 64 * c < nchunk) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) { const float d = v[c][i] - mean; q += d * d; }
+    }
+  const float var = wave_sum(q) * p.inv_n;
+  const float rstd = 1.0f / sqrtf(var + p.eps);
+  if (lane == 0) {
+    if (p.mean) p.mean[row] = mean;
+    if (p.rstd) p.rstd[row] = rstd;
+  }
+  half_t* yr = p.y + row * p.N;
+#pragma unroll
+  for (int c = 0; c < CH; ++c) {
+    const int ch = lane + 64 * c;
+    if (ch < nchunk) {
+      float gm[8], bt[8];
+      if (p.gamma) load8(p.gamma + 8 * ch, gm);
+      if (p.beta) load8(p.beta + 8 * ch, bt);
+      half8_t o;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        float t = (v[c][i] - mean) * rstd;
+        if (p.gamma) t *= gm[i];
+        if (p.beta) t += bt[i];
+        o[i] = (half_t)t;
+      }
+      *reinterpret_cast<half8_t*>(yr + 8 * ch) = o;
+    }
+  }
+}
+
+}  // namespace
+
+extern "C" int stof_bias_res_ln(const void* x, const void* bias, const void* residual,
+                                const void* gamma, const void* beta, void* y,
+                                float* mean, float* rstd,
+                                int64_t M, int64_t N, float eps, void* stream) {
+  if (!x || !y) return STOF_ERR_NULL_POINTER;
+  if (M <= 0 || N <= 0 || N % 8 != 0 || N > 8192 || M > ((int64_t)1 << 31)) return STOF_ERR_BAD_SHAPE;
+  if (!stof_aligned16(x) || !stof_aligned16(y) || !stof_aligned16(bias) || !stof_aligned16(residual) ||
+      !stof_aligned16(gamma) || !stof_aligned16(beta))
+    return STOF_ERR_MISALIGNED;
+  LnParams p;
+  p.x = (const half_t*)x; p.bias = (const half_t*)bias; p.res = (const half_t*)residual;
+  p.gamma = (const half_t*)gamma; p.beta = (const half_t*)beta; p.y = (half_t*)y;
+  p.mean = mean; p.rstd = rstd; p.M = M; p.N = (int)N; p.eps = eps; p.inv_n = 1.0f / (float)N;
+  const dim3 grid((unsigned)((M + 3) / 4)), block(256);
+  hipStream_t st = (hipStream_t)stream;
+  if (N <= 512) hipLaunchKernelGGL(bias_res_ln_kernel<1>, grid, block, 0, st, p);
+  else if (N <= 1024) hipLaunchKernelGGL(bias_res_ln_kernel<2>, grid, block, 0, st, p);
+  else if (N <= 2048) hipLaunchKernelGGL(bias_res_ln_kernel<4>, grid, block, 0, st, p);
+  else if (N <= 4096) hipLaunchKernelGGL(bias_res_ln_kernel<8>, grid, block, 0, st, p);
+  else hipLaunchKernelGGL(bias_res_ln_kernel<16>, grid, block, 0, st, p);
+  return stof_check_launch();
+}

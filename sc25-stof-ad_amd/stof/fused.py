@@ -1,0 +1,156 @@
+"""Fused encoder operators on the HIP library.
+
+Reference-named entry points (same signatures as ``src/triton_template``):
+
+* ``triton_matmul_bias_layernorm(A, B, bias, eps=1e-5)``      gemm_add_layernorm.py:126-144
+* ``triton_matmul_batch(a, b, d, bias)``                      gemm_gemm.py:158-174
+* ``triton_batched_bias_layernorm(x, bias, weight, bias_ln, eps=1e-5)``  add_layernorm.py:86-107
+
+and the explicit forms the encoder layer uses:
+
+* ``gemm_bias_act(x, Wt, bias, act)``                          act(x @ Wt^T + bias)
+* ``gemm_bias_residual_layernorm(x, Wt, bias, residual, gamma, beta, eps)``
+* ``bias_residual_layernorm(x, bias, residual, gamma, beta, eps)``
+
+Weights are consumed in the ``[N, K]`` (nn.Linear) orientation, K contiguous, which is what
+the MFMA B operand wants; ``pack_weight`` converts a reference-style ``[K, N]`` matrix once.
+Nothing here falls back to PyTorch math: a missing library or unsupported shape raises.
+"""
+import torch
+
+from . import _lib
+from ._lib import StofError, check
+
+ACT = {"none": 0, "gelu": 1, "gelu_erf": 1, "gelu_tanh": 2, "relu": 3}
+_PACK_ATTR = "_stof_packed_nk"
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _require(cond, msg):
+    if not cond:
+        raise StofError(msg)
+
+
+def _f16c(name, t, allow_none=False):
+    if t is None:
+        _require(allow_none, f"{name} is required")
+        return None
+    _require(t.is_cuda and t.dtype == torch.float16, f"{name} must be a CUDA float16 tensor")
+    return t.contiguous()
+
+
+def _p(t):
+    return None if t is None else t.data_ptr()
+
+
+def pack_weight(W):
+    """Reference-style ``[K, N]`` weight -> ``[N, K]`` contiguous, converted once per tensor
+    object and content version (the copy is kept on the tensor)."""
+    cached = getattr(W, _PACK_ATTR, None)
+    if cached is not None and cached[0] == W._version:
+        return cached[1]
+    Wt = W.t().contiguous()
+    try:
+        setattr(W, _PACK_ATTR, (W._version, Wt))
+    except AttributeError:
+        pass
+    return Wt
+
+
+def bias_residual_layernorm(x, bias, residual, gamma, beta, eps=1e-5, return_stats=False):
+    """LN(x + bias + residual) * gamma + beta over the last dim; any operand but x may be None."""
+    x = _f16c("x", x)
+    N = x.shape[-1]
+    M = x.numel() // N
+    bias = _f16c("bias", bias, True); residual = _f16c("residual", residual, True)
+    gamma = _f16c("gamma", gamma, True); beta = _f16c("beta", beta, True)
+    for name, t in (("bias", bias), ("gamma", gamma), ("beta", beta)):
+        _require(t is None or t.numel() == N, f"{name} must have {N} elements")
+    _require(residual is None or residual.shape == x.shape, "residual must have x's shape")
+    y = torch.empty_like(x)
+    mean = rstd = None
+    if return_stats:
+        mean = torch.empty(M, dtype=torch.float32, device=x.device)
+        rstd = torch.empty(M, dtype=torch.float32, device=x.device)
+    check(_lib.lib().stof_bias_res_ln(x.data_ptr(), _p(bias), _p(residual), _p(gamma), _p(beta),
+                                      y.data_ptr(), _p(mean), _p(rstd), M, N, float(eps), _stream()),
+          "stof_bias_res_ln")
+    return (y, mean, rstd) if return_stats else y
+
+
+def triton_batched_bias_layernorm(x, bias, weight, bias_ln, eps=1e-5):
+    """src/triton_template/add_layernorm.py:86-107: LN(x + bias) * weight + bias_ln, x [B,S,hidden]."""
+    return bias_residual_layernorm(x, bias, None, weight, bias_ln, eps)
+
+
+def gemm_bias_act(x, Wt, bias=None, act="none", out=None):
+    """act(x @ Wt^T + bias): x [..., K] (rows may be strided), Wt [N, K], bias [N]."""
+    _require(act in ACT, f"unknown activation {act!r}")
+    _require(x.is_cuda and x.dtype == torch.float16, "x must be a CUDA float16 tensor")
+    Wt = _f16c("Wt", Wt); bias = _f16c("bias", bias, True)
+    K = x.shape[-1]
+    N = Wt.shape[0]
+    _require(Wt.dim() == 2 and Wt.shape[1] == K, f"Wt must be [N, {K}]")
+    _require(bias is None or bias.numel() == N, f"bias must have {N} elements")
+    x2 = x.reshape(-1, K)
+    if x2.stride(1) != 1:
+        x2 = x2.contiguous()
+    M = x2.shape[0]
+    if out is None:
+        out = torch.empty(x.shape[:-1] + (N,), dtype=torch.float16, device=x.device)
+    o2 = out.view(-1, N)
+    _require(o2.shape[0] == M and o2.stride(1) == 1, "out must be [..., N] with contiguous rows")
+    check(_lib.lib().stof_gemm_bias_act(x2.data_ptr(), Wt.data_ptr(), _p(bias), o2.data_ptr(),
+                                        M, N, K, x2.stride(0), o2.stride(0), ACT[act], _stream()),
+          "stof_gemm_bias_act")
+    return out
+
+
+def gemm_bias_residual_layernorm(x, Wt, bias, residual, gamma, beta, eps=1e-5, out=None):
+    """LN(x @ Wt^T + bias + residual) * gamma + beta with the row owned by one workgroup."""
+    x = _f16c("x", x); Wt = _f16c("Wt", Wt)
+    bias = _f16c("bias", bias, True); residual = _f16c("residual", residual, True)
+    gamma = _f16c("gamma", gamma, True); beta = _f16c("beta", beta, True)
+    K = x.shape[-1]
+    N = Wt.shape[0]
+    M = x.numel() // K
+    _require(Wt.dim() == 2 and Wt.shape[1] == K, f"Wt must be [N, {K}]")
+    _require(residual is None or residual.numel() == M * N, "residual must be [..., N] matching x's rows")
+    if out is None:
+        out = torch.empty(x.shape[:-1] + (N,), dtype=torch.float16, device=x.device)
+    check(_lib.lib().stof_gemm_bias_res_ln(x.data_ptr(), Wt.data_ptr(), _p(bias), _p(residual),
+                                           _p(gamma), _p(beta), out.data_ptr(), M, N, K, float(eps), _stream()),
+          "stof_gemm_bias_res_ln")
+    return out
+
+
+def triton_matmul_bias_layernorm(A, B, bias, eps=1e-5):
+    """src/triton_template/gemm_add_layernorm.py:126-144: LayerNorm WITHOUT gamma/beta of
+    ``A[b,M,K] @ B[b,K,N] + bias``.
+
+    ``B`` is the reference's per-batch weight, always an ``expand`` of one ``[K,N]`` matrix at
+    its call sites (src/tuning_STOF_cost.py:59-60); a batch of distinct matrices is rejected.
+    ``bias`` of N elements is a bias; of shape ``[b,M,N]`` it is the caller's
+    ``bias + residual`` (same call sites) and is added element-wise - the evident intent,
+    where the reference kernel reads only its first N elements.
+    """
+    _require(A.dim() == 3 and B.dim() == 3 and A.shape[2] == B.shape[1], "A [b,M,K], B [b,K,N] expected")
+    _require(B.stride(0) == 0 or B.shape[0] == 1, "B must be one weight matrix expanded over the batch")
+    N = B.shape[2]
+    Wt = pack_weight(B[0])
+    if bias.numel() == N:
+        return gemm_bias_residual_layernorm(A, Wt, bias.reshape(N), None, None, None, eps)
+    _require(bias.shape == A.shape[:2] + (N,), "bias must have N elements or shape [b,M,N]")
+    return gemm_bias_residual_layernorm(A, Wt, None, bias, None, None, eps)
+
+
+def triton_matmul_batch(a, b, d, bias):
+    """src/triton_template/gemm_gemm.py:158-174: gelu_tanh(a @ b + bias) @ d, a [B,M,K],
+    b [K,N], d [N,H]; the intermediate is fp16 (gemm_gemm.py:152).  Two launches of the GEMM
+    kernel; the intermediate stays in fp16 as in the reference."""
+    _require(a.dim() == 3 and b.dim() == 2 and d.dim() == 2, "a [B,M,K], b [K,N], d [N,H] expected")
+    t = gemm_bias_act(a, pack_weight(b), bias.reshape(-1)[: b.shape[1]], "gelu_tanh")
+    return gemm_bias_act(t, pack_weight(d), None, "none")

@@ -1,0 +1,198 @@
+"""Mask specification and the mask -> block-LUT compiler (host side, PyTorch).
+
+Same call signatures and return values as the reference's ``src/util/masks.py``:
+five dense-mask generators (``:10-122``) and ``get_sparse_storage`` (``:125-184``),
+which classifies every (query block, key block) tile of ``Mask[0]`` as full,
+partial or empty and returns three CSR-like int32 lists plus the additive fp16
+blocks of the partial tiles.  Outputs are bit-identical to the reference's; the
+implementation is not a loop translation: every generator is a closed-form index
+predicate evaluated once on the mask's device, and the classifier is a single
+blocked reduction, so the compile step costs a handful of tensor ops where the
+reference runs (S/bm)*(S/bn) ``torch.all`` calls.
+
+Extensions that the reference lacks (its LUT is shared by the whole batch):
+``get_sparse_storage_batched`` builds one LUT per sample and concatenates them
+with absolute offsets, so that B == 1 degenerates to the reference format.
+"""
+import random
+
+import torch
+
+NEG_MASK = -10000.0
+
+
+def _grid(seq_len, device):
+    i = torch.arange(seq_len, device=device)[:, None]
+    j = torch.arange(seq_len, device=device)[None, :]
+    return i, j
+
+
+def _finish(attr_mask, allowed, is_causal):
+    """Broadcast one [S,S] bool pattern over the batch in attr_mask's dtype and
+    apply the reference's causal trim, which reaches the LAST batch entry only
+    (its loop variable is used after the loop: src/util/masks.py:28-30)."""
+    out = allowed.to(attr_mask.dtype).unsqueeze(0).repeat(attr_mask.shape[0], 1, 1)
+    if is_causal:
+        s = attr_mask.shape[1]
+        i, j = _grid(s, attr_mask.device)
+        out[-1] = out[-1] * (j <= i).to(attr_mask.dtype)
+    return out
+
+
+def generate_causal_mask(attr_mask):
+    """src/util/masks.py:10-14: lower-triangular ones; float32 on the CPU whatever
+    attr_mask's dtype and device are, exactly as the reference returns it."""
+    seq_len = attr_mask.shape[1]
+    tri = torch.tril(torch.ones(seq_len, seq_len))
+    return tri.unsqueeze(0).repeat(attr_mask.shape[0], 1, 1)
+
+
+def generate_sliding_mask(attr_mask, bandwidth=1, is_cauasl=False):
+    """src/util/masks.py:17-32: 1 where |i-j| <= bandwidth."""
+    i, j = _grid(attr_mask.shape[1], attr_mask.device)
+    return _finish(attr_mask, (i - j).abs() <= bandwidth, is_cauasl)
+
+
+def generate_dilated_mask(attr_mask, bandwidth=1, dilation_rate=1, is_cauasl=False):
+    """src/util/masks.py:35-52: 1 at columns i-bw-d + t*(d+1), t >= 0, that lie in
+    [0, min(S, i+bw+d+1))."""
+    s = attr_mask.shape[1]
+    i, j = _grid(s, attr_mask.device)
+    w = bandwidth + dilation_rate
+    off = j - (i - w)
+    allowed = (off >= 0) & (off % (dilation_rate + 1) == 0) & (j < torch.clamp(i + w + 1, max=s))
+    return _finish(attr_mask, allowed, is_cauasl)
+
+
+def generate_longformer_mask(attr_mask, globalwidth=1, bandwidth=1, is_cauasl=False):
+    """src/util/masks.py:55-81: global rows/columns [0,g) and [S/2, S/2+g) plus the band."""
+    s = attr_mask.shape[1]
+    i, j = _grid(s, attr_mask.device)
+    lo, hi = int(s / 2), int(s / 2 + globalwidth)
+    glob = (i < globalwidth) | (j < globalwidth) | ((i >= lo) & (i < hi)) | ((j >= lo) & (j < hi))
+    return _finish(attr_mask, glob | ((i - j).abs() <= bandwidth), is_cauasl)
+
+
+def generate_bigbird_mask(attr_mask, globalwidth=1, bandwidth=1, fill_rate=0.2, is_cauasl=False):
+    """src/util/masks.py:86-122: global + band + random points.
+
+    The random points come from the stdlib generator seeded with 0 and consumed in
+    the reference's order (per batch, per 32-row block: one ``choice`` for the
+    column block, then ``randint(0,32)`` for x and y of each of
+    ``int(1024*fill_rate)`` points), so the mask is reproducible bit for bit.
+    """
+    b, s = attr_mask.shape[0], attr_mask.shape[1]
+    i, j = _grid(s, attr_mask.device)
+    base = (i < globalwidth) | (j < globalwidth) | ((i - j).abs() <= bandwidth)
+    out = base.to(attr_mask.dtype).unsqueeze(0).repeat(b, 1, 1)
+    npts = int(1024 * fill_rate)
+    random.seed(0)
+    nblk = int(s / 32)
+    bb, xx, yy = [], [], []
+    for batch in range(b):
+        for blk in range(nblk - 1):
+            sx = blk * 32
+            if blk == 0:
+                sy = sx + 32 * random.choice([1, 0])
+            elif blk == nblk - 2:
+                sy = sx + 32 * random.choice([-1, 0])
+            else:
+                sy = sx + 32 * random.choice([-1, 0, 1])
+            for _ in range(npts):
+                xx.append(sx + random.randint(0, 32))
+                yy.append(sy + random.randint(0, 32))
+                bb.append(batch)
+    if bb:
+        dev = attr_mask.device
+        out[torch.tensor(bb, device=dev), torch.tensor(xx, device=dev), torch.tensor(yy, device=dev)] = 1
+    if is_cauasl:
+        out[-1] = out[-1] * (j <= i).to(attr_mask.dtype)
+    return out
+
+
+def _classify(m2d, bm, bn):
+    """[S,S] -> (blocks [nQ,nK,bm,bn], full [nQ,nK] bool, part [nQ,nK] bool)."""
+    n = m2d.shape[-1]
+    if m2d.shape[-2] != n or n % bm or n % bn:
+        raise ValueError(f"mask must be square with seq_len divisible by the block sizes; "
+                         f"got {tuple(m2d.shape)} for blocks {bm}x{bn}")
+    blocks = m2d.reshape(n // bm, bm, n // bn, bn).permute(0, 2, 1, 3)
+    full = (blocks == 1).all(-1).all(-1)
+    empty = (blocks == 0).all(-1).all(-1)
+    return blocks, full, ~full & ~empty
+
+
+def _csr(flag):
+    """[nQ,nK] bool -> (row_ptr int32 [nQ+1], col_idx int32 [nnz]) in row-major order."""
+    counts = flag.sum(1)
+    row_ptr = torch.zeros(flag.shape[0] + 1, dtype=torch.int64, device=flag.device)
+    row_ptr[1:] = torch.cumsum(counts, 0)
+    col_idx = flag.nonzero()[:, 1]
+    return row_ptr.to(torch.int32), col_idx.to(torch.int32)
+
+
+def get_sparse_storage(Mask, block_size_m, block_size_n):
+    """src/util/masks.py:125-184.  Mask [B,S,S] of 0/1 (any float dtype, any device).
+
+    Returns ``(nnz, full_row_ptr, full_col_idx, part_row_ptr, part_col_idx,
+    part_block_mask, load_row_ptr, load_col_idx)`` on Mask's device: ``nnz`` is the
+    percentage of non-zeros of the WHOLE tensor over S*S (:137), the LUT describes
+    batch 0 only (:147), partial tiles carry ``-10000 * (1 - block.half())`` (:160)
+    and an LUT without partial tiles carries one dummy block of ones (:179-180).
+    """
+    n = Mask.shape[-1]
+    nnz = torch.count_nonzero(Mask) / (n * n) * 100
+    blocks, full, part = _classify(Mask[0], block_size_m, block_size_n)
+    full_row_ptr, full_col_idx = _csr(full)
+    part_row_ptr, part_col_idx = _csr(part)
+    load_row_ptr, load_col_idx = _csr(full | part)
+    if int(part_row_ptr[-1]) == 0:
+        part_block_mask = torch.ones(1, block_size_m, block_size_n, dtype=torch.float16, device=Mask.device)
+    else:
+        part_block_mask = (NEG_MASK * (1.0 - blocks[part].to(torch.float16))).contiguous()
+    return (nnz, full_row_ptr, full_col_idx, part_row_ptr, part_col_idx,
+            part_block_mask, load_row_ptr, load_col_idx)
+
+
+def get_sparse_storage_batched(Mask, block_size_m, block_size_n):
+    """One LUT per sample.  Row pointers have shape [B, nQ+1] and hold ABSOLUTE
+    offsets into the concatenated column lists / partial-block stack, so sample b's
+    query block r owns entries ``row_ptr[b,r] .. row_ptr[b,r+1]``; with B == 1 the
+    arrays equal get_sparse_storage's (row pointers gain a leading dim of 1).
+    The reference has no counterpart: its kernel shares one LUT over the batch.
+    """
+    B, n = Mask.shape[0], Mask.shape[-1]
+    nnz = torch.count_nonzero(Mask) / (n * n) * 100
+    outs = {k: [] for k in ("frp", "fci", "prp", "pci", "pbm", "lrp", "lci")}
+    fo = po = lo = 0
+    for b in range(B):
+        blocks, full, part = _classify(Mask[b], block_size_m, block_size_n)
+        frp, fci = _csr(full); prp, pci = _csr(part); lrp, lci = _csr(full | part)
+        outs["frp"].append(frp + fo); outs["fci"].append(fci)
+        outs["prp"].append(prp + po); outs["pci"].append(pci)
+        outs["lrp"].append(lrp + lo); outs["lci"].append(lci)
+        if pci.numel():
+            outs["pbm"].append((NEG_MASK * (1.0 - blocks[part].to(torch.float16))))
+        fo += fci.numel(); po += pci.numel(); lo += lci.numel()
+    if po == 0:
+        pbm = torch.ones(1, block_size_m, block_size_n, dtype=torch.float16, device=Mask.device)
+    else:
+        pbm = torch.cat(outs["pbm"], 0).contiguous()
+    st = lambda k: torch.stack(outs[k], 0).contiguous()
+    ct = lambda k: torch.cat(outs[k], 0).contiguous()
+    return (nnz, st("frp"), ct("fci"), st("prp"), ct("pci"), pbm, st("lrp"), ct("lci"))
+
+
+def expand_sparse_storage(lut, n, block_size_m, block_size_n):
+    """LUT -> dense [n,n] float32 0/1 mask (full -> 1, partial -> additive block == 0).
+    The inverse of get_sparse_storage on 0/1 masks; used to validate a LUT."""
+    _, frp, fci, prp, pci, pbm, _, _ = lut
+    nq, nk = n // block_size_m, n // block_size_n
+    dev = frp.device
+    out = torch.zeros(nq, nk, block_size_m, block_size_n, dtype=torch.float32, device=dev)
+    rows_f = torch.repeat_interleave(torch.arange(nq, device=dev), (frp[1:] - frp[:-1]).long())
+    out[rows_f, fci.long()] = 1
+    if int(prp[-1]) > 0:
+        rows_p = torch.repeat_interleave(torch.arange(nq, device=dev), (prp[1:] - prp[:-1]).long())
+        out[rows_p, pci.long()] = (pbm.float() == 0).float()
+    return out.permute(0, 2, 1, 3).reshape(n, n)

@@ -1,0 +1,222 @@
+"""Attention operators: the reference's ``src/ops/package_op.py`` API on the HIP library.
+
+``block_attn_mask_op`` and the three ``rowwise_attn_*_op`` keep the reference's call
+signatures, tensor layouts and return conventions (src/ops/package_op.py:10-74):
+
+* block op: q, k, v ``[B,H,S,D]`` fp16, the seven LUT tensors of ``get_sparse_storage``,
+  ``BLOCK_M, BLOCK_N, num_warps``; the result overwrites ``q`` and ``q`` is returned;
+* row-wise ops: a new zero-initialised ``[B, S, H*D]`` tensor is returned.
+
+``block_attn`` is the functional form underneath (separate output, strided inputs, output
+layout choice, optional per-sample LUT).  Everything runs in libstof_hip.so; there is no
+PyTorch fallback - a missing library or an unsupported configuration raises ``StofError``.
+"""
+import math
+
+import torch
+from torch.autograd import Function
+
+from . import _lib
+from ._lib import StofError, check, strides3
+
+__all__ = ["block_attn", "block_attn_mask_op", "rowwise_attn_full_op", "rowwise_attn_sliding_op",
+           "rowwise_attn_mask_op", "pack_mask_bits", "StofError"]
+
+_BITS_ATTR = "_stof_packed_bits"
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _ptr(t):
+    return t.data_ptr() if t is not None and t.numel() > 0 else None
+
+
+def _require(cond, msg):
+    if not cond:
+        raise StofError(msg)
+
+
+def pack_mask_bits(src, additive):
+    """fp16 ``[..., rows, cols]`` mask -> uint64-as-int64 ``[..., rows, cols/64]`` bit rows.
+    additive=True: 0 keeps / -10000 drops (the LUT's partial blocks);
+    additive=False: value > 0 keeps (the row-wise op's ``row_mask``)."""
+    _require(src.is_cuda and src.dtype == torch.float16, "mask must be a CUDA fp16 tensor")
+    src = src.contiguous()
+    cols = src.shape[-1]
+    _require(cols % 64 == 0, f"mask columns ({cols}) must be a multiple of 64")
+    rows = src.numel() // cols
+    dst = torch.empty(src.shape[:-1] + (cols // 64,), dtype=torch.int64, device=src.device)
+    check(_lib.lib().stof_pack_mask_bits(src.data_ptr(), dst.data_ptr(), rows, cols, cols,
+                                         1 if additive else 0, _stream()), "stof_pack_mask_bits")
+    return dst
+
+
+def _packed_partial_bits(part_block_mask):
+    """Bit rows of the LUT's partial blocks, packed once per tensor object and content
+    version and kept on the tensor itself."""
+    cached = getattr(part_block_mask, _BITS_ATTR, None)
+    if cached is not None and cached[0] == part_block_mask._version:
+        return cached[1]
+    pbm = part_block_mask
+    _require(pbm.dim() == 3, "part_block_mask must be [n_part, BLOCK_M, BLOCK_N]")
+    # The kernel applies element masks as bits; additive values other than 0 / -10000
+    # (or the all-ones dummy block of an LUT without partial tiles) cannot be represented.
+    ok = ((pbm == 0) | (pbm == -10000.0)).all() | ((pbm == 1).all() & (pbm.shape[0] == 1))
+    _require(bool(ok), "part_block_mask must hold only 0 and -10000 (get_sparse_storage's encoding)")
+    bits = pack_mask_bits(pbm, additive=True)
+    try:
+        setattr(part_block_mask, _BITS_ATTR, (part_block_mask._version, bits))
+    except AttributeError:
+        pass
+    return bits
+
+
+def _check_i32(name, t, device):
+    _require(t.dtype == torch.int32, f"{name} must be int32, got {t.dtype}")
+    _require(t.device == device, f"{name} is on {t.device}, expected {device}")
+    return t.contiguous()
+
+
+def block_attn(q, k, v, lut, block_m=64, block_n=64, out=None, out_layout="bhsd", softmax_scale=None):
+    """Block-masked attention.  q, k, v: fp16 views ``[B,H,S,D]`` with unit stride in D (any
+    other strides).  ``lut`` = (full_row_ptr, full_col_idx, part_row_ptr, part_col_idx,
+    part_block_mask, load_row_ptr, load_col_idx) as returned by ``get_sparse_storage`` (the
+    leading ``nnz`` dropped) or by ``get_sparse_storage_batched`` (2-D row pointers: one LUT
+    per sample).  Returns ``out``: ``[B,H,S,D]`` (``out_layout='bhsd'``) or ``[B,S,H*D]``
+    (``'bshd'``); ``out`` may be ``q`` itself.
+    """
+    frp, fci, prp, pci, pbm, lrp, lci = lut
+    _require(q.is_cuda, "q must be a CUDA tensor (this path has no CPU implementation)")
+    for name, t in (("q", q), ("k", k), ("v", v)):
+        _require(t.dtype == torch.float16, f"{name} must be float16, got {t.dtype}")
+        _require(t.dim() == 4 and t.stride(3) == 1, f"{name} must be [B,H,S,D] with contiguous D")
+        _require(t.device == q.device, f"{name} is on a different device than q")
+    _require(k.shape == q.shape and v.shape == q.shape, "q, k, v must have the same shape")
+    B, H, S, D = q.shape
+    dev = q.device
+    frp = _check_i32("full_row_ptr", frp, dev); fci = _check_i32("full_col_idx", fci, dev)
+    prp = _check_i32("part_row_ptr", prp, dev); pci = _check_i32("part_col_idx", pci, dev)
+    lrp = _check_i32("load_row_ptr", lrp, dev); lci = _check_i32("load_col_idx", lci, dev)
+    _require(pbm.dtype == torch.float16 and pbm.device == dev, "part_block_mask must be fp16 on q's device")
+    _require(S % block_m == 0 and S % block_n == 0, f"seq_len {S} not divisible by block {block_m}x{block_n}")
+    nq = S // block_m
+    if lrp.dim() == 2:
+        _require(lrp.shape == (B, nq + 1) and frp.shape == lrp.shape and prp.shape == lrp.shape,
+                 f"per-sample row pointers must be [{B}, {nq + 1}]")
+        lut_bs = nq + 1
+    else:
+        _require(lrp.numel() == nq + 1 and frp.numel() == nq + 1 and prp.numel() == nq + 1,
+                 f"row pointers must have {nq + 1} entries for seq_len {S}, block_m {block_m}")
+        lut_bs = 0
+    bits = _packed_partial_bits(pbm)
+    if out is None:
+        if out_layout == "bhsd":
+            out = torch.empty((B, H, S, D), dtype=torch.float16, device=dev)
+        else:
+            out = torch.empty((B, S, H * D), dtype=torch.float16, device=dev)
+    if out_layout == "bhsd":
+        _require(out.shape == (B, H, S, D) and out.stride(3) == 1, "out must be [B,H,S,D] with contiguous D")
+        ostr = strides3(out)
+    elif out_layout == "bshd":
+        _require(out.shape == (B, S, H * D) and out.stride(2) == 1, "out must be [B,S,H*D] with contiguous last dim")
+        ostr = (_lib.c_int64 * 3)(out.stride(0), D, out.stride(1))
+    else:
+        raise StofError(f"unknown out_layout {out_layout!r}")
+    _require(out.dtype == torch.float16 and out.device == dev, "out must be fp16 on q's device")
+    scale = softmax_scale if softmax_scale is not None else 1.0 / math.sqrt(D)
+    check(_lib.lib().stof_block_attn_fwd(
+        q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(),
+        _ptr(frp), _ptr(fci), _ptr(prp), _ptr(pci), _ptr(bits), _ptr(lrp), _ptr(lci),
+        block_m, block_n, scale,
+        strides3(q), strides3(k), strides3(v), ostr,
+        B, S, H, D, lut_bs, _stream()), "stof_block_attn_fwd")
+    return out
+
+
+class Block_Attn_Mask(Function):
+    """src/ops/package_op.py:50-68: the result is written into ``q`` and ``q`` is returned.
+    A non-contiguous ``q`` also receives the result (the reference silently returns it
+    unchanged in that case)."""
+
+    @staticmethod
+    def forward(ctx, q, k, v,
+                full_row_ptr, full_col_idx,
+                part_row_ptr, part_col_idx, part_block_mask,
+                load_row_ptr, load_col_idx,
+                BLOCK_M, BLOCK_N, num_warps):
+        lut = (full_row_ptr, full_col_idx, part_row_ptr, part_col_idx, part_block_mask,
+               load_row_ptr, load_col_idx)
+        if k.stride(-1) != 1:
+            k = k.contiguous()
+        if v.stride(-1) != 1:
+            v = v.contiguous()
+        if q.stride(-1) == 1:
+            block_attn(q, k, v, lut, BLOCK_M, BLOCK_N, out=q)
+        else:
+            q.copy_(block_attn(q.contiguous(), k, v, lut, BLOCK_M, BLOCK_N))
+        ctx.mark_non_differentiable(q)
+        return q
+
+
+def _rowwise(kind, q, k, v, is_causal, bandwidth, row_mask):
+    _require(q.is_cuda, "q must be a CUDA tensor (this path has no CPU implementation)")
+    for name, t in (("q", q), ("k", k), ("v", v)):
+        _require(t.dtype == torch.float16, f"{name} must be float16, got {t.dtype}")
+    q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
+    B, H, S, D = q.shape
+    result = torch.zeros((B, S, H * D), device=q.device, dtype=q.dtype)
+    bits = None
+    if kind == 2:
+        _require(row_mask.shape[-2:] == (S, S), f"row_mask must be [{S},{S}]")
+        cached = getattr(row_mask, _BITS_ATTR, None)
+        if cached is not None and cached[0] == row_mask._version:
+            bits = cached[1]
+        else:
+            bits = pack_mask_bits(row_mask.to(torch.float16).reshape(S, S), additive=False)
+            try:
+                setattr(row_mask, _BITS_ATTR, (row_mask._version, bits))
+            except AttributeError:
+                pass
+    check(_lib.lib().stof_rowwise_attn_fwd(
+        q.data_ptr(), k.data_ptr(), v.data_ptr(), result.data_ptr(),
+        kind, 1 if is_causal else 0, int(bandwidth), _ptr(bits),
+        B, S, H, D, _stream()), "stof_rowwise_attn_fwd")
+    return result
+
+
+class RowWise_Attn_Full(Function):
+    """src/ops/package_op.py:11-22."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, is_causal=False):
+        result = _rowwise(0, q, k, v, is_causal, 0, None)
+        ctx.mark_non_differentiable(result)
+        return result
+
+
+class RowWise_Attn_Sliding(Function):
+    """src/ops/package_op.py:24-35."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, is_causal, bandwidth):
+        result = _rowwise(1, q, k, v, is_causal, bandwidth, None)
+        ctx.mark_non_differentiable(result)
+        return result
+
+
+class RowWise_Attn_Mask(Function):
+    """src/ops/package_op.py:37-48."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, is_causal, row_mask):
+        result = _rowwise(2, q, k, v, is_causal, 0, row_mask)
+        ctx.mark_non_differentiable(result)
+        return result
+
+
+rowwise_attn_full_op = RowWise_Attn_Full.apply
+rowwise_attn_sliding_op = RowWise_Attn_Sliding.apply
+rowwise_attn_mask_op = RowWise_Attn_Mask.apply
+block_attn_mask_op = Block_Attn_Mask.apply

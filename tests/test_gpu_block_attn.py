@@ -1,0 +1,184 @@
+"""GPU parity of the block-masked attention kernel, through the Python operator API and
+the C ABI underneath, against the CPU oracle on the same seeded inputs.
+
+Tolerance (fp16 kernel vs fp32 oracle on the same fp16-rounded inputs):
+    |got - want| <= 2e-3 + 1e-2 * |want|        (max-abs 2e-3, rel 1e-2)
+Rows without any allowed key are defined as zero on both sides.
+"""
+import numpy as np
+import pytest
+import torch
+
+from oracle import attention as oa
+from oracle import masks as om
+from stof import configs, masks as pm
+from stof.ops import block_attn, block_attn_mask_op, StofError
+
+pytestmark = pytest.mark.gpu
+ATOL, RTOL = 2e-3, 1e-2
+
+
+def _close(got, want, what=""):
+    got = got.float().cpu(); want = want.float().cpu()
+    err = (got - want).abs()
+    bad = err > ATOL + RTOL * want.abs()
+    assert not bool(bad.any()), f"{what}: {int(bad.sum())} elements out of tolerance, max abs err {float(err.max()):.3e}"
+    return float(err.max())
+
+
+def _inputs(b, h, s, seed, scale=1.0):
+    cfg = configs.AttnConfig("t", b, h, s)
+    return configs.qkv(cfg, seed=seed, dtype=torch.float16, device="cuda", scale=scale)
+
+
+def _run(q, k, v, mask2d, **kw):
+    lut = pm.get_sparse_storage(mask2d.float()[None].cuda(), 64, 64)[1:]
+    return block_attn(q, k, v, lut, 64, 64, **kw)
+
+
+def _oracle(q, k, v, mask):
+    return oa.dense_masked_attention(q.cpu().float(), k.cpu().float(), v.cpu().float(), mask.cpu())
+
+
+@pytest.mark.parametrize("name,b,h,s", [("C1", 1, 12, 512), ("C2", 8, 12, 1024), ("C5", 2, 4, 2048)])
+def test_config_shapes_vs_oracle(name, b, h, s):
+    print(f"case {name} b{b} h{h} s{s}", flush=True)
+    mask = configs.ATTN_MASKS[name](s)
+    q, k, v = _inputs(b, h, s, seed=0)
+    got = _run(q, k, v, mask)
+    torch.cuda.synchronize()
+    _close(got, _oracle(q, k, v, mask), name)
+
+
+def test_c4_full_size_subset_and_properties():
+    """C4 at its full shape: oracle on a subset of (batch, head) pairs, plus size-independent
+    properties on the whole output (rows of ones for V == 1, linearity in V)."""
+    print("case C4 full", flush=True)
+    cfg = configs.C4
+    mask = configs.mask_c4(cfg.seq)
+    q, k, v = configs.qkv(cfg, seed=0, device="cuda")
+    lut = pm.get_sparse_storage(mask.float()[None].cuda(), 64, 64)[1:]
+    assert lut[5][-1].item() == 946
+    got = block_attn(q, k, v, lut)
+    for (b, h) in [(0, 0), (1, 15), (0, 7)]:
+        want = _oracle(q[b:b + 1, h:h + 1], k[b:b + 1, h:h + 1], v[b:b + 1, h:h + 1], mask)
+        _close(got[b:b + 1, h:h + 1], want, f"C4 b{b} h{h}")
+    ones = block_attn(q, k, torch.ones_like(v), lut)
+    assert float((ones.float() - 1).abs().max()) <= 2e-3
+    v2 = torch.randn_like(v)
+    a = block_attn(q, k, v, lut).float(); b2 = block_attn(q, k, v2, lut).float()
+    ab = block_attn(q, k, (v.float() + v2.float()).half(), lut).float()
+    assert float((ab - (a + b2)).abs().max()) <= 1e-2   # fp16 rounding of v+v2 and of three outputs
+
+
+def test_in_place_op_returns_q_like_reference():
+    mask = configs.mask_c1(512)
+    q, k, v = _inputs(1, 12, 512, seed=1)
+    want = _oracle(q, k, v, mask)
+    lut = pm.get_sparse_storage(mask.float()[None].cuda(), 64, 64)
+    ret = block_attn_mask_op(q, k, v, *lut[1:], 64, 64, 4)
+    assert ret.data_ptr() == q.data_ptr()
+    _close(q, want, "in place")
+
+
+def test_non_contiguous_q_receives_result():
+    mask = configs.mask_c1(256)
+    q, k, v = _inputs(1, 4, 256, seed=2)
+    want = _oracle(q, k, v, mask)
+    qt = q.permute(0, 2, 1, 3).contiguous().permute(0, 2, 1, 3)     # [B,H,S,D] view, S/H swapped in memory
+    qd = torch.empty(1, 4, 256, 128, dtype=torch.float16, device="cuda")[..., ::2]  # D stride 2
+    qd.copy_(q)
+    lut = pm.get_sparse_storage(mask.float()[None].cuda(), 64, 64)
+    _close(block_attn_mask_op(qt, k, v, *lut[1:], 64, 64, 4), want, "strided q")
+    _close(block_attn_mask_op(qd, k, v, *lut[1:], 64, 64, 4), want, "q with D stride 2")
+
+
+def test_packed_qkv_views_and_bshd_output():
+    """q, k, v as slices of one [B,S,3*H*D] projection buffer; output written as [B,S,H*D]."""
+    B, H, S, D = 2, 6, 512, 64
+    g = torch.Generator().manual_seed(3)
+    packed = torch.randn(B, S, 3 * H * D, generator=g).half().cuda()
+    q, k, v = (packed[..., t * H * D:(t + 1) * H * D].view(B, S, H, D).permute(0, 2, 1, 3) for t in range(3))
+    mask = configs.mask_c5(S)
+    out = _run(q, k, v, mask, out_layout="bshd")
+    want = _oracle(q, k, v, mask).permute(0, 2, 1, 3).reshape(B, S, H * D)
+    assert out.shape == (B, S, H * D)
+    _close(out, want, "packed/bshd")
+
+
+def test_per_sample_lut_padding_mask():
+    """C3's mask at reduced batch: one LUT per sample (key padding x sliding window)."""
+    B, H, S = 4, 12, 512
+    mask, L = configs.mask_c3(batch=B, s=S, window=256, seed=0)
+    q, k, v = _inputs(B, H, S, seed=4)
+    lut = pm.get_sparse_storage_batched(mask.float().cuda(), 64, 64)[1:]
+    got = block_attn(q, k, v, lut)
+    _close(got, _oracle(q, k, v, mask), "per-sample LUT")
+
+
+def test_dead_rows_empty_blocks_and_masked_first_tile():
+    S = 256
+    mask = torch.ones(S, S)
+    mask[64:128, :] = 0                 # a query block with no LUT entry -> zeros
+    mask[3, :] = 0                      # a dead row inside a live block
+    mask[130, :64] = 0                  # row masked in its FIRST visited (partial) tile only
+    mask[131, :] = 0; mask[131, 255] = 1   # single allowed key, in the last tile
+    q, k, v = _inputs(2, 3, S, seed=5)
+    got = _run(q, k, v, mask)
+    assert bool((got[:, :, 64:128] == 0).all()) and bool((got[:, :, 3] == 0).all())
+    _close(got, _oracle(q, k, v, mask), "edge rows")
+    assert torch.allclose(got[:, :, 131].float(), v[:, :, 255].float(), atol=1e-3)
+
+
+@pytest.mark.parametrize("seed", [0, 1, 2, 3])
+def test_random_block_masks(seed):
+    """Random full / partial / empty tiling, random element masks inside partial tiles."""
+    rng = np.random.default_rng(seed)
+    S = 64 * int(rng.integers(2, 9))
+    n = S // 64
+    kind = rng.integers(0, 3, size=(n, n))
+    mask = torch.zeros(S, S)
+    for r in range(n):
+        for c in range(n):
+            if kind[r, c] == 1:
+                mask[r * 64:(r + 1) * 64, c * 64:(c + 1) * 64] = 1
+            elif kind[r, c] == 2:
+                dens = rng.choice([0.02, 0.5, 0.98])
+                mask[r * 64:(r + 1) * 64, c * 64:(c + 1) * 64] = torch.from_numpy(
+                    (rng.random((64, 64)) < dens).astype(np.float32))
+    B, H = int(rng.integers(1, 4)), int(rng.integers(1, 5))
+    print(f"seed {seed}: S {S} B {B} H {H}", flush=True)
+    q, k, v = _inputs(B, H, S, seed=10 + seed)
+    got = _run(q, k, v, mask)
+    _close(got, _oracle(q, k, v, mask), f"random seed {seed}")
+    # the oracle's restatement of the reference's block algorithm agrees as well
+    lut_np = om.get_sparse_storage(mask.numpy()[None], 64, 64)
+    blk = oa.block_attn_mask(q.cpu().float().numpy(), k.cpu().float().numpy(), v.cpu().float().numpy(), lut_np, 64, 64)
+    _close(got, torch.from_numpy(blk), f"random seed {seed} (block oracle)")
+
+
+def test_large_logits_no_overflow():
+    """|score| of several hundred: the max-subtracted softmax must stay finite."""
+    q, k, v = _inputs(1, 2, 256, seed=6, scale=6.0)
+    mask = configs.mask_c1(256)
+    got = _run(q, k, v, mask)
+    assert bool(torch.isfinite(got).all())
+    _close(got, _oracle(q, k, v, mask), "large logits")
+
+
+def test_error_paths_raise():
+    q, k, v = _inputs(1, 2, 128, seed=7)
+    lut = pm.get_sparse_storage(torch.ones(1, 128, 128).cuda(), 64, 64)[1:]
+    with pytest.raises(StofError):
+        block_attn(q.float(), k, v, lut)                       # wrong dtype
+    with pytest.raises(StofError):
+        block_attn(q, k, v, lut, 32, 32)                       # row pointers do not fit 32x32
+    lut32 = pm.get_sparse_storage(torch.ones(1, 128, 128).cuda(), 32, 32)[1:]
+    with pytest.raises(StofError):
+        block_attn(q, k, v, lut32, 32, 32)                     # unsupported block size
+    bad = list(lut); bad[5] = lut[5].long()
+    with pytest.raises(StofError):
+        block_attn(q, k, v, tuple(bad))                        # int64 row pointers
+    q96 = torch.randn(1, 2, 128, 96, device="cuda").half()
+    with pytest.raises(StofError):
+        block_attn(q96, q96, q96, lut)                         # head size 96
