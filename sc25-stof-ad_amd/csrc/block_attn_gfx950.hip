@@ -4,22 +4,26 @@
 // (src/ops/src/block_attn_mask_cuda.cu:269-6322) with one kernel designed around the
 // CDNA4 wavefront:
 //
-//  * one 64-lane wavefront (= one workgroup) owns one 64-row query block and walks the
-//    LUT's key blocks for it; there is no cross-wave sharing, hence no workgroup barrier
-//    that waits on another wave and no S/P/O traffic through LDS;
+//  * a workgroup of two 64-lane wavefronts owns one 64-row query block; each wave keeps 32
+//    queries in registers and both walk the LUT's key blocks, sharing the K and V tiles
+//    in LDS.  S, P and O never touch LDS;
+//  * K/V tiles travel HBM/L2 -> LDS with the asynchronous direct-to-LDS loads
+//    (global_load_lds_dwordx4), double buffered: the loads of block t+1 are issued before
+//    the math of block t, no VGPRs are used for staging and one barrier per block suffices;
 //  * scores are produced TRANSPOSED, S^T = K . Q^T, with v_mfma_f32_32x32x16_f16.  In the
-//    32x32 accumulator layout a lane then holds 32 keys of ONE query (lane & 31), so the
+//    32x32 accumulator layout a lane holds 32 keys of ONE query (lane & 31), so the
 //    online-softmax state (running max, running sum, rescale factor) is one scalar per
-//    lane, the row reduction is a register loop plus a single exchange with lane ^ 32,
-//    and the probabilities are already in the register layout the second product
-//    O^T = V^T . P^T wants for its B operand - P never leaves registers;
-//  * K is staged in LDS row-major (its contraction index d is contiguous in memory),
-//    V is staged TRANSPOSED (contraction index = key must be contiguous per lane): each
-//    lane gathers a 4-key x 8-channel patch with 16-byte loads and transposes it in
-//    registers with v_perm_b32 before 8-byte LDS writes;
+//    lane, the row reduction is a register loop plus one v_permlane32_swap, and the
+//    probabilities already sit in the register layout the second product
+//    O^T = V^T . P^T wants for its B operand;
+//  * V stays row-major in LDS; the A operand of the second product (key index contiguous
+//    per lane) is formed by the transposing LDS read ds_read_b64_tr_b16;
+//  * LDS tiles are unpadded (the DMA writes 1 KB contiguous per instruction); a 16-byte
+//    chunk XOR swizzle applied on the global-address side keeps both the 16-byte K
+//    fragment reads and the transposing V reads free of bank conflicts;
 //  * masks: full tiles run mask-free, partial tiles test one bit per element from a
 //    64-bit row mask (512 B per tile instead of the reference's 8 KB additive fp16 tile),
-//    empty tiles are never visited;
+//    empty tiles are never visited; the LUT row is fetched once into registers;
 //  * workgroup ids are remapped so that all query blocks of one (batch, head) run on one
 //    XCD (K/V stay in that XCD's L2) and long LUT rows start first.
 #include "stof_common.h"
@@ -29,13 +33,17 @@ namespace {
 constexpr int kD = 64;        // head size
 constexpr int kBM = 64;       // query rows per block
 constexpr int kBN = 64;       // keys per block
-constexpr int kLd = 72;       // LDS row pitch in halves: 64 + 8 pad (144 B) keeps the
-                              // 16-byte fragment reads of 16 consecutive rows on distinct banks
-constexpr float kMasked = -INFINITY;   // score given to a masked element
+constexpr int kTile = kBN * kD * 2;   // bytes of one K or V tile in LDS (8 KB, unpadded)
+constexpr float kMasked = -INFINITY;  // score given to a masked element
+
+typedef __attribute__((address_space(3))) unsigned char lds_byte;
+typedef short short4_t __attribute__((ext_vector_type(4)));
+typedef short short8_t __attribute__((ext_vector_type(8)));
+typedef __attribute__((address_space(3))) short4_t lds_short4;
+typedef __attribute__((address_space(1))) const void gptr_t;
 
 struct AttnParams {
   const half_t* q; const half_t* k; const half_t* v; half_t* out;
-  const int32_t* frp; const int32_t* fci;
   const int32_t* prp; const int32_t* pci; const uint64_t* pbits;
   const int32_t* lrp; const int32_t* lci;
   int64_t qs[3], ks[3], vs[3], os[3];
@@ -49,26 +57,30 @@ __device__ __forceinline__ floatx16 mfma32(half8_t a, half8_t b, floatx16 c) {
   return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
 }
 
-// LUT cursor of one query block: yields (key block, bitmask slot or -1) in LOAD order,
-// following the three-way rule of block_attn_mask_cuda.cu:3675-3700.
-struct LutCursor {
-  const int32_t* fci; const int32_t* pci; const int32_t* lci;
-  int t, t_end, f, f_end, pp, pp_end;
-  __device__ __forceinline__ bool next(int& col, int& slot) {
-    while (t < t_end) {
-      const int c = __builtin_amdgcn_readfirstlane(lci[t++]);
-      if (f < f_end && __builtin_amdgcn_readfirstlane(fci[f]) == c) { ++f; col = c; slot = -1; return true; }
-      if (pp < pp_end && __builtin_amdgcn_readfirstlane(pci[pp]) == c) { col = c; slot = pp++; return true; }
-    }
-    return false;
-  }
-};
+// max / sum of a value with its partner lane (lane ^ 32).  v_permlane32_swap(x, x) leaves
+// {own, partner} in some order in its two results for either half of the wave.
+__device__ __forceinline__ float pair_max(float x) {
+  const unsigned u = __builtin_bit_cast(unsigned, x);
+  const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  return fmaxf(__builtin_bit_cast(float, (unsigned)r[0]), __builtin_bit_cast(float, (unsigned)r[1]));
+}
+__device__ __forceinline__ float pair_sum(float x) {
+  const unsigned u = __builtin_bit_cast(unsigned, x);
+  const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  return __builtin_bit_cast(float, (unsigned)r[0]) + __builtin_bit_cast(float, (unsigned)r[1]);
+}
 
-__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void block_attn_fwd_kernel(const AttnParams p) {
-  __shared__ __attribute__((aligned(16))) half_t Ks[kBN * kLd];
-  __shared__ __attribute__((aligned(16))) half_t Vt[kD * kLd];
+// 16-byte-chunk swizzle of a tile row: chunk c of row r is stored at chunk position
+// c ^ swz(r).  swz is a bijection of row bits (1,2,3) onto chunk bits (2,0,1).
+__device__ __forceinline__ int swz(int row) { return (((row >> 1) & 1) << 2) | ((row >> 2) & 3); }
 
-  const int lane = threadIdx.x;
+__global__ __launch_bounds__(128) void block_attn_fwd_kernel(const AttnParams p) {
+  // [K buf 0][K buf 1][V buf 0][V buf 1]
+  __shared__ __attribute__((aligned(1024))) unsigned char smem[4 * kTile];
+  lds_byte* const lds = (lds_byte*)smem;
+
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
   const int j32 = lane & 31;
   const int g = lane >> 5;
 
@@ -82,185 +94,197 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
   const int b = bh / p.H;
   const int h = bh - b * p.H;
 
-  const half_t* qb = p.q + b * p.qs[0] + h * p.qs[1] + (int64_t)qi * kBM * p.qs[2];
+  const half_t* qb = p.q + b * p.qs[0] + h * p.qs[1] + ((int64_t)qi * kBM + 32 * wave) * p.qs[2];
   const half_t* kb = p.k + b * p.ks[0] + h * p.ks[1];
   const half_t* vb = p.v + b * p.vs[0] + h * p.vs[1];
-  half_t* ob = p.out + b * p.os[0] + h * p.os[1] + (int64_t)qi * kBM * p.os[2];
+  half_t* ob = p.out + b * p.os[0] + h * p.os[1] + ((int64_t)qi * kBM + 32 * wave) * p.os[2];
 
-  // Q^T as the B operand: lane (n = query j32 of tile nt, k-group g) holds 8 consecutive d.
-  half8_t qf[2][4];
-#pragma unroll
-  for (int nt = 0; nt < 2; ++nt)
-#pragma unroll
-    for (int ks = 0; ks < 4; ++ks)
-      qf[nt][ks] = *reinterpret_cast<const half8_t*>(qb + (int64_t)(32 * nt + j32) * p.qs[2] + 16 * ks + 8 * g);
-
+  // ---- LUT row -> registers: lane i holds entry i (key block, bitmask slot or -1).
+  // LOAD is the sorted union of FULL and PART (get_sparse_storage builds it so), hence an
+  // entry is partial iff its key block is in this row's PART list, otherwise full.
   const int64_t lo = (int64_t)b * p.lut_bs;
-  LutCursor cur;
-  cur.fci = p.fci; cur.pci = p.pci; cur.lci = p.lci;
-  cur.t = __builtin_amdgcn_readfirstlane(p.lrp[lo + qi]); cur.t_end = __builtin_amdgcn_readfirstlane(p.lrp[lo + qi + 1]);
-  cur.f = __builtin_amdgcn_readfirstlane(p.frp[lo + qi]); cur.f_end = __builtin_amdgcn_readfirstlane(p.frp[lo + qi + 1]);
-  cur.pp = __builtin_amdgcn_readfirstlane(p.prp[lo + qi]); cur.pp_end = __builtin_amdgcn_readfirstlane(p.prp[lo + qi + 1]);
+  const int t0 = __builtin_amdgcn_readfirstlane(p.lrp[lo + qi]);
+  const int n_ent = __builtin_amdgcn_readfirstlane(p.lrp[lo + qi + 1]) - t0;
+  const int p0 = __builtin_amdgcn_readfirstlane(p.prp[lo + qi]);
+  const int n_part = __builtin_amdgcn_readfirstlane(p.prp[lo + qi + 1]) - p0;
 
-  floatx16 oacc[2][2];   // [d tile][query tile]: O^T
+  // Q^T as the B operand: lane (n = query j32, k-group g) holds 8 consecutive d per k-step.
+  half8_t qf[4];
+#pragma unroll
+  for (int ks = 0; ks < 4; ++ks)
+    qf[ks] = *reinterpret_cast<const half8_t*>(qb + (int64_t)j32 * p.qs[2] + 16 * ks + 8 * g);
+
+  // ---- per-lane constants of the data movement
+  // DMA: instruction i of this wave fills tile rows 8*(4*wave+i) .. +7 (1 KB of LDS);
+  // lane l lands at (row 8*(4*wave+i) + l/8, chunk position l%8) and therefore fetches
+  // global chunk (l%8) ^ swz(row).
+  int k_src[4], v_src[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int row = 8 * (4 * wave + i) + (lane >> 3);
+    const int chunk = (lane & 7) ^ swz(row);
+    k_src[i] = row * (int)p.ks[2] + 8 * chunk;
+    v_src[i] = row * (int)p.vs[2] + 8 * chunk;
+  }
+  // K fragment (A operand of S^T): row = key 32*mt + j32, chunk 2*ks + g.
+  int k_rd[4];
+#pragma unroll
+  for (int ks = 0; ks < 4; ++ks) k_rd[ks] = j32 * 128 + (((2 * ks + g) ^ swz(j32)) << 4);
+  // V fragment (A operand of O^T) through the transposing read.  Within a 16-lane block,
+  // lane j supplies the address of key row (j >> 2) at channel offset 4*(j & 3) and receives
+  // the four keys of channel (block base + j).  Block = lane >> 4: k-group g = block >> 1,
+  // channel half = block & 1.  Keys of k-step (mt, s2), half hh: 32mt + 16s2 + 8hh + 4g + c.
+  int v_rd[2][2];
+  {
+    const int j = lane & 15, dh = (lane >> 4) & 1;
+#pragma unroll
+    for (int dt = 0; dt < 2; ++dt)
+#pragma unroll
+      for (int hh = 0; hh < 2; ++hh) {
+        const int row = 8 * hh + 4 * g + (j >> 2);
+        const int chunk = 4 * dt + 2 * dh + ((j >> 1) & 1);
+        v_rd[dt][hh] = row * 128 + ((chunk ^ swz(row)) << 4) + 8 * (j & 1);
+      }
+  }
+
+  floatx16 oacc[2];   // [d tile]: O^T for this wave's 32 queries
 #pragma unroll
   for (int i = 0; i < 2; ++i)
 #pragma unroll
-    for (int j = 0; j < 2; ++j)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) oacc[i][j][r] = 0.f;
-  float m_run[2] = {-INFINITY, -INFINITY};
-  float l_run[2] = {0.f, 0.f};
+    for (int r = 0; r < 16; ++r) oacc[i][r] = 0.f;
+  float m_run = -INFINITY;
+  float l_run = 0.f;
 
-  // staging lanes: 8 lanes cover one 128-byte row
-  const int dc = lane & 7;     // 16-byte chunk (8 channels) within a row
-  const int rq = lane >> 3;    // row (K) or key quad (V) handled by this lane, per round
+  auto issue_tile = [&](int col, int buf) {
+    const half_t* kt = kb + (int64_t)col * kBN * p.ks[2];
+    const half_t* vt = vb + (int64_t)col * kBN * p.vs[2];
+    lds_byte* kd = lds + buf * kTile + (4 * wave) * 1024;
+    lds_byte* vd = lds + (2 + buf) * kTile + (4 * wave) * 1024;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      __builtin_amdgcn_global_load_lds((gptr_t*)(kt + k_src[i]), (__attribute__((address_space(3))) void*)(kd + i * 1024), 16, 0, 0);
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      __builtin_amdgcn_global_load_lds((gptr_t*)(vt + v_src[i]), (__attribute__((address_space(3))) void*)(vd + i * 1024), 16, 0, 0);
+  };
 
-  int col, slot;
-  bool have = cur.next(col, slot);
-
-  while (have) {
-    // ---- K tile -> LDS (row-major); the V tile's loads stay in flight while S is computed
-    {
-      uint4 kr[8];
-      const half_t* kt = kb + (int64_t)col * kBN * p.ks[2] + 8 * dc;
-#pragma unroll
-      for (int t = 0; t < 8; ++t) kr[t] = *reinterpret_cast<const uint4*>(kt + (int64_t)(8 * t + rq) * p.ks[2]);
-#pragma unroll
-      for (int t = 0; t < 8; ++t) *reinterpret_cast<uint4*>(&Ks[(8 * t + rq) * kLd + 8 * dc]) = kr[t];
-    }
-    uint4 vr[2][4];
-    {
-      const half_t* vt = vb + (int64_t)col * kBN * p.vs[2] + 8 * dc;
-#pragma unroll
-      for (int t = 0; t < 2; ++t)
-#pragma unroll
-        for (int c4 = 0; c4 < 4; ++c4)
-          vr[t][c4] = *reinterpret_cast<const uint4*>(vt + (int64_t)(4 * (rq + 8 * t) + c4) * p.vs[2]);
-    }
-    __syncthreads();
-
-    // ---- S^T = K . Q^T : sacc[nt][mt][r] = S[query 32nt+j32][key 32mt + 8(r/4) + 4g + r%4]
-    floatx16 sacc[2][2];
-#pragma unroll
-    for (int i = 0; i < 2; ++i)
-#pragma unroll
-      for (int j = 0; j < 2; ++j)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) sacc[i][j][r] = 0.f;
-#pragma unroll
-    for (int ks = 0; ks < 4; ++ks)
-#pragma unroll
-      for (int mt = 0; mt < 2; ++mt) {
-        const half8_t a = *reinterpret_cast<const half8_t*>(&Ks[(32 * mt + j32) * kLd + 16 * ks + 8 * g]);
-#pragma unroll
-        for (int nt = 0; nt < 2; ++nt) sacc[nt][mt] = mfma32(a, qf[nt][ks], sacc[nt][mt]);
-      }
-
-    // ---- V tile -> LDS transposed.  This lane holds keys 4*qd .. 4*qd+3 (rows) x channels
-    // 8*dc .. 8*dc+7; it writes, for each channel, the 4 keys as one 8-byte word at the
-    // position the P.V A-operand read expects: key = 32mt + 16s + 8h + 4g' + c sits at
-    // 32mt + 16s + 8g' + 4h + c, i.e. the two low bits of the quad index are swapped.
-#pragma unroll
-    for (int t = 0; t < 2; ++t) {
-      const int qd = rq + 8 * t;
-      const int pq = (qd & ~3) | ((qd & 1) << 1) | ((qd >> 1) & 1);
-      const uint4 a0 = vr[t][0], a1 = vr[t][1], a2 = vr[t][2], a3 = vr[t][3];
-      const uint32_t v0[4] = {a0.x, a0.y, a0.z, a0.w};
-      const uint32_t v1[4] = {a1.x, a1.y, a1.z, a1.w};
-      const uint32_t v2[4] = {a2.x, a2.y, a2.z, a2.w};
-      const uint32_t v3[4] = {a3.x, a3.y, a3.z, a3.w};
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        uint2 ev, od;
-        ev.x = __builtin_amdgcn_perm(v1[j], v0[j], 0x05040100u);
-        ev.y = __builtin_amdgcn_perm(v3[j], v2[j], 0x05040100u);
-        od.x = __builtin_amdgcn_perm(v1[j], v0[j], 0x07060302u);
-        od.y = __builtin_amdgcn_perm(v3[j], v2[j], 0x07060302u);
-        *reinterpret_cast<uint2*>(&Vt[(8 * dc + 2 * j) * kLd + 4 * pq]) = ev;
-        *reinterpret_cast<uint2*>(&Vt[(8 * dc + 2 * j + 1) * kLd + 4 * pq]) = od;
-      }
+  for (int base = 0; base < n_ent; base += 64) {
+    const int n_here = min(64, n_ent - base);
+    int ent_col = 0, ent_slot = -1;
+    if (lane < n_here) ent_col = p.lci[t0 + base + lane];
+    for (int pb = 0; pb < n_part; pb += 64) {
+      const int np_here = min(64, n_part - pb);
+      int pc = -1;
+      if (lane < np_here) pc = p.pci[p0 + pb + lane];
+      for (int j = 0; j < np_here; ++j)
+        if (ent_col == __builtin_amdgcn_readlane(pc, j)) ent_slot = p0 + pb + j;
     }
 
-    const int cur_slot = slot;
-    const int cur_col = col;
-    (void)cur_col;
-    const bool have_next = cur.next(col, slot);
-    __syncthreads();
+    int buf = 0;
+    issue_tile(__builtin_amdgcn_readlane(ent_col, 0), 0);
+    for (int t = 0; t < n_here; ++t, buf ^= 1) {
+      const int slot = __builtin_amdgcn_readlane(ent_slot, t);
+      // all DMA issued so far (tile t) has landed for this wave; the barrier makes both
+      // waves' halves visible and also orders last iteration's reads of the other buffer
+      // before the loads that overwrite it.
+      // (the row mask of a partial tile is fetched first so that its latency hides behind
+      // the same wait and no register-returning load is pending across the DMA issue)
+      uint64_t bits = ~0ull;
+      if (slot >= 0) bits = p.pbits[(int64_t)slot * kBM + 32 * wave + j32];
+      __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0)
+      __syncthreads();
+      if (t + 1 < n_here) issue_tile(__builtin_amdgcn_readlane(ent_col, t + 1), buf ^ 1);
 
-    // ---- online softmax on S^T; one query per lane (and its partner lane ^ 32)
-    half8_t pf[2][2][2];   // [query tile][key tile][half]: B operand of O^T = V^T . P^T
+      const lds_byte* kt = lds + buf * kTile;
+      const lds_byte* vt = lds + (2 + buf) * kTile;
+
+      // ---- S^T = K . Q^T : sacc[mt][r] = S[query j32][key 32mt + 8(r/4) + 4g + r%4]
+      floatx16 sacc[2];
 #pragma unroll
-    for (int nt = 0; nt < 2; ++nt) {
-      if (cur_slot >= 0) {
-        const uint64_t bits = p.pbits[(int64_t)cur_slot * kBM + 32 * nt + j32];
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) sacc[i][r] = 0.f;
+#pragma unroll
+      for (int ks = 0; ks < 4; ++ks)
+#pragma unroll
+        for (int mt = 0; mt < 2; ++mt) {
+          const half8_t a = *reinterpret_cast<const __attribute__((address_space(3))) half8_t*>(kt + mt * 4096 + k_rd[ks]);
+          sacc[mt] = mfma32(a, qf[ks], sacc[mt]);
+        }
+
+      // ---- element mask of a partial tile
+      if (slot >= 0) {
 #pragma unroll
         for (int mt = 0; mt < 2; ++mt) {
           const uint32_t w = (uint32_t)(bits >> (32 * mt)) >> (4 * g);
 #pragma unroll
           for (int r = 0; r < 16; ++r)
-            if (!((w >> (8 * (r >> 2) + (r & 3))) & 1u)) sacc[nt][mt][r] = kMasked;
+            if (!((w >> (8 * (r >> 2) + (r & 3))) & 1u)) sacc[mt][r] = kMasked;
         }
       }
-      float mx = sacc[nt][0][0];
+
+      // ---- online softmax; one query per lane (shared with the partner lane ^ 32)
+      float mx = sacc[0][0];
 #pragma unroll
       for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) mx = fmaxf(mx, sacc[nt][mt][r]);
-      mx = fmaxf(mx, xchg32(mx));
-      const float m_new = fmaxf(m_run[nt], mx);
+        for (int r = 0; r < 16; ++r) mx = fmaxf(mx, sacc[mt][r]);
+      mx = pair_max(mx);
+      const float m_new = fmaxf(m_run, mx);
       // A row that has seen no allowed key yet has m_new == -inf: subtract 0 instead, so
       // that its probabilities are exp2(-inf) = 0 and no inf - inf appears.
       const float m_sub = (m_new == -INFINITY) ? 0.f : m_new;
-      const float alpha = __builtin_amdgcn_exp2f((m_run[nt] - m_sub) * p.c);
+      const float alpha = __builtin_amdgcn_exp2f((m_run - m_sub) * p.c);
       const float mc = m_sub * p.c;
       float lsum = 0.f;
+      half8_t pf[2][2];   // [key tile][half]: B operand of O^T = V^T . P^T
 #pragma unroll
       for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-          const float e = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[nt][mt][r], p.c, -mc));
+          const float e = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[mt][r], p.c, -mc));
           lsum += e;
-          pf[nt][mt][r >> 3][r & 7] = (half_t)e;
+          pf[mt][r >> 3][r & 7] = (half_t)e;
         }
-      l_run[nt] = l_run[nt] * alpha + lsum;   // per-lane partial sum; halves are added at the end
-      m_run[nt] = m_new;
+      l_run = l_run * alpha + lsum;   // per-lane partial sum; the two halves are added at the end
+      m_run = m_new;
+      if (__any(alpha != 1.0f)) {
 #pragma unroll
-      for (int dt = 0; dt < 2; ++dt)
+        for (int dt = 0; dt < 2; ++dt)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) oacc[dt][nt][r] *= alpha;
-    }
-
-    // ---- O^T += V^T . P^T
-#pragma unroll
-    for (int mt = 0; mt < 2; ++mt)
-#pragma unroll
-      for (int s2 = 0; s2 < 2; ++s2)
-#pragma unroll
-        for (int dt = 0; dt < 2; ++dt) {
-          const half8_t a = *reinterpret_cast<const half8_t*>(&Vt[(32 * dt + j32) * kLd + 32 * mt + 16 * s2 + 8 * g]);
-#pragma unroll
-          for (int nt = 0; nt < 2; ++nt) oacc[dt][nt] = mfma32(a, pf[nt][mt][s2], oacc[dt][nt]);
-        }
-    have = have_next;
-  }
-
-  // ---- normalise and store: oacc[dt][nt][r] = O[query 32nt+j32][d = 32dt + 8(r/4) + 4g + r%4]
-#pragma unroll
-  for (int nt = 0; nt < 2; ++nt) {
-    const float l = l_run[nt] + xchg32(l_run[nt]);
-    const float inv = (l > 0.f) ? 1.0f / l : 0.f;   // no allowed key at all: zeros
-    half_t* orow = ob + (int64_t)(32 * nt + j32) * p.os[2];
-#pragma unroll
-    for (int dt = 0; dt < 2; ++dt)
-#pragma unroll
-      for (int q4 = 0; q4 < 4; ++q4) {
-        half4_t o4;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) o4[e] = (half_t)(oacc[dt][nt][4 * q4 + e] * inv);
-        *reinterpret_cast<half4_t*>(orow + 32 * dt + 8 * q4 + 4 * g) = o4;
+          for (int r = 0; r < 16; ++r) oacc[dt][r] *= alpha;
       }
+
+      // ---- O^T += V^T . P^T
+#pragma unroll
+      for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+        for (int s2 = 0; s2 < 2; ++s2)
+#pragma unroll
+          for (int dt = 0; dt < 2; ++dt) {
+            const lds_byte* vp = vt + (32 * mt + 16 * s2) * 128;
+            const short4_t a0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4*)(vp + v_rd[dt][0]));
+            const short4_t a1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4*)(vp + v_rd[dt][1]));
+            const half8_t a = __builtin_bit_cast(half8_t, (short8_t)__builtin_shufflevector(a0, a1, 0, 1, 2, 3, 4, 5, 6, 7));
+            oacc[dt] = mfma32(a, pf[mt][s2], oacc[dt]);
+          }
+    }
+    __syncthreads();   // the next chunk's first loads overwrite buffer 0
   }
+
+  // ---- normalise and store: oacc[dt][r] = O[query j32][d = 32dt + 8(r/4) + 4g + r%4]
+  const float l = pair_sum(l_run);
+  const float inv = (l > 0.f) ? 1.0f / l : 0.f;   // no allowed key at all: zeros
+  half_t* orow = ob + (int64_t)j32 * p.os[2];
+#pragma unroll
+  for (int dt = 0; dt < 2; ++dt)
+#pragma unroll
+    for (int q4 = 0; q4 < 4; ++q4) {
+      half4_t o4;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) o4[e] = (half_t)(oacc[dt][4 * q4 + e] * inv);
+      *reinterpret_cast<half4_t*>(orow + 32 * dt + 8 * q4 + 4 * g) = o4;
+    }
 }
 
 // dst[r*(cols/64)+w] bit t = pred(src[r*ld + 64w + t]); one wavefront per 64-element word.
@@ -282,7 +306,9 @@ __global__ __launch_bounds__(256) void pack_mask_bits_kernel(const half_t* __res
   }
 }
 
-bool strides_ok(const int64_t s[3]) { return (s[0] % 8 == 0) && (s[1] % 8 == 0) && (s[2] % 8 == 0) && s[2] >= kD; }
+bool strides_ok(const int64_t s[3]) {
+  return (s[0] % 8 == 0) && (s[1] % 8 == 0) && (s[2] % 8 == 0) && s[2] >= kD && s[2] < (1 << 20);
+}
 
 }  // namespace
 
@@ -315,7 +341,7 @@ extern "C" int stof_block_attn_fwd(
 
   AttnParams p;
   p.q = (const half_t*)q; p.k = (const half_t*)k; p.v = (const half_t*)v; p.out = (half_t*)out;
-  p.frp = full_row_ptr; p.fci = full_col_idx; p.prp = part_row_ptr; p.pci = part_col_idx;
+  p.prp = part_row_ptr; p.pci = part_col_idx;
   p.pbits = part_bitmask; p.lrp = load_row_ptr; p.lci = load_col_idx;
   for (int i = 0; i < 3; ++i) { p.qs[i] = q_strides[i]; p.ks[i] = k_strides[i]; p.vs[i] = v_strides[i]; p.os[i] = out_strides[i]; }
   p.lut_bs = lut_batch_stride;
@@ -323,7 +349,7 @@ extern "C" int stof_block_attn_fwd(
   p.total = (int)total64;
   p.chunk = (p.total + 7) / 8;
   p.c = softmax_scale * 1.4426950408889634f;
-  hipLaunchKernelGGL(block_attn_fwd_kernel, dim3(p.chunk * 8), dim3(64), 0, (hipStream_t)stream, p);
+  hipLaunchKernelGGL(block_attn_fwd_kernel, dim3(p.chunk * 8), dim3(128), 0, (hipStream_t)stream, p);
   return stof_check_launch();
 }
 

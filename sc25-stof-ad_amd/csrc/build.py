@@ -16,6 +16,8 @@ FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
     # packed-FP32 VALU forms are kept out of the generated code
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # MFMA accumulators live in VGPRs: no v_accvgpr copies around the softmax / epilogues
+    "-mllvm", "-amdgpu-mfma-vgpr-form",
     "-I" + os.path.join(ROOT, "include"), "-I" + HERE,
     "-Wno-unused-command-line-argument",
 ]
