@@ -35,6 +35,7 @@ constexpr int kBM = 64;       // query rows per block
 constexpr int kBN = 64;       // keys per block
 constexpr int kTile = kBN * kD * 2;   // bytes of one K or V tile in LDS (8 KB, unpadded)
 constexpr float kMasked = -INFINITY;  // score given to a masked element
+constexpr float kLazy = 8.0f;         // log2 slack before the running max is raised
 
 typedef __attribute__((address_space(3))) unsigned char lds_byte;
 typedef short short4_t __attribute__((ext_vector_type(4)));
@@ -75,9 +76,13 @@ __device__ __forceinline__ float pair_sum(float x) {
 __device__ __forceinline__ int swz(int row) { return (((row >> 1) & 1) << 2) | ((row >> 2) & 3); }
 
 __global__ __launch_bounds__(128) void block_attn_fwd_kernel(const AttnParams p) {
-  // [K buf 0][K buf 1][V buf 0][V buf 1]
-  __shared__ __attribute__((aligned(1024))) unsigned char smem[4 * kTile];
-  lds_byte* const lds = (lds_byte*)smem;
+  // Four distinct LDS objects (K and V, two buffers each): the compiler orders LDS reads
+  // after in-flight direct-to-LDS loads per object, so a read of the current buffer does
+  // not wait for the loads that fill the other one.
+  __shared__ __attribute__((aligned(1024))) unsigned char k_lds0[kTile];
+  __shared__ __attribute__((aligned(1024))) unsigned char k_lds1[kTile];
+  __shared__ __attribute__((aligned(1024))) unsigned char v_lds0[kTile];
+  __shared__ __attribute__((aligned(1024))) unsigned char v_lds1[kTile];
 
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int lane = threadIdx.x & 63;
@@ -155,11 +160,11 @@ __global__ __launch_bounds__(128) void block_attn_fwd_kernel(const AttnParams p)
   float m_run = -INFINITY;
   float l_run = 0.f;
 
-  auto issue_tile = [&](int col, int buf) {
+  auto issue_tile = [&](int col, lds_byte* kdst, lds_byte* vdst) {
     const half_t* kt = kb + (int64_t)col * kBN * p.ks[2];
     const half_t* vt = vb + (int64_t)col * kBN * p.vs[2];
-    lds_byte* kd = lds + buf * kTile + (4 * wave) * 1024;
-    lds_byte* vd = lds + (2 + buf) * kTile + (4 * wave) * 1024;
+    lds_byte* kd = kdst + (4 * wave) * 1024;
+    lds_byte* vd = vdst + (4 * wave) * 1024;
 #pragma unroll
     for (int i = 0; i < 4; ++i)
       __builtin_amdgcn_global_load_lds((gptr_t*)(kt + k_src[i]), (__attribute__((address_space(3))) void*)(kd + i * 1024), 16, 0, 0);
@@ -180,23 +185,19 @@ __global__ __launch_bounds__(128) void block_attn_fwd_kernel(const AttnParams p)
         if (ent_col == __builtin_amdgcn_readlane(pc, j)) ent_slot = p0 + pb + j;
     }
 
-    int buf = 0;
-    issue_tile(__builtin_amdgcn_readlane(ent_col, 0), 0);
-    for (int t = 0; t < n_here; ++t, buf ^= 1) {
+    // one key block: kt/vt hold tile t, the loads of tile t+1 go to kn/vn
+    auto step = [&](int t, const lds_byte* kt, const lds_byte* vt, lds_byte* kn, lds_byte* vn) {
       const int slot = __builtin_amdgcn_readlane(ent_slot, t);
-      // all DMA issued so far (tile t) has landed for this wave; the barrier makes both
-      // waves' halves visible and also orders last iteration's reads of the other buffer
-      // before the loads that overwrite it.
-      // (the row mask of a partial tile is fetched first so that its latency hides behind
-      // the same wait and no register-returning load is pending across the DMA issue)
+      // The row mask of a partial tile is fetched first so that its latency hides behind
+      // the wait below and no register-returning load is pending across the DMA issue.
       uint64_t bits = ~0ull;
       if (slot >= 0) bits = p.pbits[(int64_t)slot * kBM + 32 * wave + j32];
+      // All DMA issued so far (tile t) has landed for this wave; the barrier makes both
+      // waves' halves visible and also orders last step's reads of the other buffers
+      // before the loads that overwrite them.
       __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0)
       __syncthreads();
-      if (t + 1 < n_here) issue_tile(__builtin_amdgcn_readlane(ent_col, t + 1), buf ^ 1);
-
-      const lds_byte* kt = lds + buf * kTile;
-      const lds_byte* vt = lds + (2 + buf) * kTile;
+      if (t + 1 < n_here) issue_tile(__builtin_amdgcn_readlane(ent_col, t + 1), kn, vn);
 
       // ---- S^T = K . Q^T : sacc[mt][r] = S[query j32][key 32mt + 8(r/4) + 4g + r%4]
       floatx16 sacc[2];
@@ -223,28 +224,36 @@ __global__ __launch_bounds__(128) void block_attn_fwd_kernel(const AttnParams p)
         }
       }
 
-      // ---- online softmax; one query per lane (shared with the partner lane ^ 32)
+      // ---- online softmax; one query per lane (shared with the partner lane ^ 32).
+      // The running max is only raised when the tile's max exceeds it by more than kLazy
+      // (in log2 units): probabilities then stay below 2^kLazy, well inside fp16 range, the
+      // normalisation by the running sum stays exact, and the O rescale becomes rare.
       float mx = sacc[0][0];
 #pragma unroll
       for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
         for (int r = 0; r < 16; ++r) mx = fmaxf(mx, sacc[mt][r]);
       mx = pair_max(mx);
-      const float m_new = fmaxf(m_run, mx);
+      const float m_new = (mx * p.c > m_run * p.c + kLazy || m_run == -INFINITY) ? mx : m_run;
       // A row that has seen no allowed key yet has m_new == -inf: subtract 0 instead, so
       // that its probabilities are exp2(-inf) = 0 and no inf - inf appears.
       const float m_sub = (m_new == -INFINITY) ? 0.f : m_new;
       const float alpha = __builtin_amdgcn_exp2f((m_run - m_sub) * p.c);
       const float mc = m_sub * p.c;
-      float lsum = 0.f;
       half8_t pf[2][2];   // [key tile][half]: B operand of O^T = V^T . P^T
+      float lsum = 0.f;
+      const half2_t ones2 = {(half_t)1.0f, (half_t)1.0f};
 #pragma unroll
       for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const float e = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[mt][r], p.c, -mc));
-          lsum += e;
-          pf[mt][r >> 3][r & 7] = (half_t)e;
+        for (int r = 0; r < 16; r += 2) {
+          const float e0 = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[mt][r], p.c, -mc));
+          const float e1 = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[mt][r + 1], p.c, -mc));
+          const half2_t e2 = {(half_t)e0, (half_t)e1};
+          pf[mt][r >> 3][r & 7] = e2[0];
+          pf[mt][r >> 3][(r & 7) + 1] = e2[1];
+          // row sum of the ROUNDED probabilities (what P.V multiplies), two per instruction
+          lsum = __builtin_amdgcn_fdot2(e2, ones2, lsum, false);
         }
       l_run = l_run * alpha + lsum;   // per-lane partial sum; the two halves are added at the end
       m_run = m_new;
@@ -268,6 +277,13 @@ __global__ __launch_bounds__(128) void block_attn_fwd_kernel(const AttnParams p)
             const half8_t a = __builtin_bit_cast(half8_t, (short8_t)__builtin_shufflevector(a0, a1, 0, 1, 2, 3, 4, 5, 6, 7));
             oacc[dt] = mfma32(a, pf[mt][s2], oacc[dt]);
           }
+    };
+
+    issue_tile(__builtin_amdgcn_readlane(ent_col, 0), (lds_byte*)k_lds0, (lds_byte*)v_lds0);
+    for (int t = 0; t < n_here; t += 2) {
+      step(t, (const lds_byte*)k_lds0, (const lds_byte*)v_lds0, (lds_byte*)k_lds1, (lds_byte*)v_lds1);
+      if (t + 1 < n_here)
+        step(t + 1, (const lds_byte*)k_lds1, (const lds_byte*)v_lds1, (lds_byte*)k_lds0, (lds_byte*)v_lds0);
     }
     __syncthreads();   // the next chunk's first loads overwrite buffer 0
   }
