@@ -4,9 +4,12 @@
 // (src/ops/src/block_attn_mask_cuda.cu:269-6322) with one kernel designed around the
 // CDNA4 wavefront:
 //
-//  * a workgroup of two 64-lane wavefronts owns one 64-row query block; each wave keeps 32
-//    queries in registers and both walk the LUT's key blocks, sharing the K and V tiles
-//    in LDS.  S, P and O never touch LDS;
+//  * a workgroup of four 64-lane wavefronts owns TWO adjacent 64-row query blocks (two LUT
+//    rows); each wave keeps 32 queries in registers.  The two rows' key-block lists are
+//    merged on the fly: a key block wanted by both rows is brought into LDS once and used
+//    by all four waves, one wanted by a single row is skipped by the other row's waves.
+//    This halves the L2 -> LDS traffic per unit of MFMA work, which is what bounds the
+//    kernel at head size 64.  S, P and O never touch LDS;
 //  * K/V tiles travel HBM/L2 -> LDS with the asynchronous direct-to-LDS loads
 //    (global_load_lds_dwordx4), double buffered: the loads of block t+1 are issued before
 //    the math of block t, no VGPRs are used for staging and one barrier per block suffices;
@@ -49,7 +52,7 @@ struct AttnParams {
   const int32_t* lrp; const int32_t* lci;
   int64_t qs[3], ks[3], vs[3], os[3];
   int64_t lut_bs;
-  int B, S, H, nQ;
+  int B, S, H, nQ, nP;   // nP = query-block pairs per (batch, head)
   int total, chunk;
   float c;  // softmax_scale * log2(e)
 };
@@ -75,7 +78,29 @@ __device__ __forceinline__ float pair_sum(float x) {
 // c ^ swz(r).  swz is a bijection of row bits (1,2,3) onto chunk bits (2,0,1).
 __device__ __forceinline__ int swz(int row) { return (((row >> 1) & 1) << 2) | ((row >> 2) & 3); }
 
-__global__ __launch_bounds__(128) void block_attn_fwd_kernel(const AttnParams p) {
+// One LUT row (the key blocks of one 64-row query block) held in registers, 64 entries at
+// a time: lane i holds entry base+i.  `slot` is the bitmask slot of a partial entry, -1
+// for a full one.  LOAD is the union of FULL and PART (get_sparse_storage builds it so),
+// hence an entry is partial iff its key block is in the row's PART list.
+struct LutRow {
+  int t0, n, p0, np;      // first LOAD entry, entry count, first PART entry, PART count
+  int base;               // index of the entry held by lane 0
+  int col, slot;          // per lane
+  __device__ __forceinline__ void fill(const AttnParams& p, int lane, bool want_slots) {
+    col = 0x7fffffff; slot = -1;
+    if (base + lane < n) col = p.lci[t0 + base + lane];
+    if (!want_slots) return;
+    for (int pb = 0; pb < np; pb += 64) {
+      const int here = min(64, np - pb);
+      int pc = -1;
+      if (lane < here) pc = p.pci[p0 + pb + lane];
+      for (int j = 0; j < here; ++j)
+        if (col == __builtin_amdgcn_readlane(pc, j)) slot = p0 + pb + j;
+    }
+  }
+};
+
+__global__ __launch_bounds__(256) void block_attn_fwd_kernel(const AttnParams p) {
   // Four distinct LDS objects (K and V, two buffers each): the compiler orders LDS reads
   // after in-flight direct-to-LDS loads per object, so a read of the current buffer does
   // not wait for the loads that fill the other one.
@@ -88,48 +113,66 @@ __global__ __launch_bounds__(128) void block_attn_fwd_kernel(const AttnParams p)
   const int lane = threadIdx.x & 63;
   const int j32 = lane & 31;
   const int g = lane >> 5;
+  const int rsel = wave >> 1;    // which of the pair's two query blocks this wave serves
+  const int half = wave & 1;     // which 32 queries of that block
 
   // Workgroups are handed to the 8 XCDs round-robin; give each XCD a contiguous range
-  // of (batch, head, query block) so one head's K/V is read through a single L2.
+  // of (batch, head, query-block pair) so one head's K/V is read through a single L2.
   const int wg = blockIdx.x;
   const int vid = (wg & 7) * p.chunk + (wg >> 3);
   if (vid >= p.total) return;
-  const int bh = vid / p.nQ;
-  const int qi = p.nQ - 1 - (vid - bh * p.nQ);   // late (long, for causal-like masks) rows first
+  const int bh = vid / p.nP;
+  const int pair = p.nP - 1 - (vid - bh * p.nP);   // late (long, for causal-like masks) rows first
   const int b = bh / p.H;
   const int h = bh - b * p.H;
+  const int qi = 2 * pair + rsel;                  // this wave's query block
+  const bool q_valid = qi < p.nQ;                  // odd block count: the last pair has one row
 
-  const half_t* qb = p.q + b * p.qs[0] + h * p.qs[1] + ((int64_t)qi * kBM + 32 * wave) * p.qs[2];
+  const int64_t qrow0 = (int64_t)qi * kBM + 32 * half;
+  const half_t* qb = p.q + b * p.qs[0] + h * p.qs[1] + qrow0 * p.qs[2];
   const half_t* kb = p.k + b * p.ks[0] + h * p.ks[1];
   const half_t* vb = p.v + b * p.vs[0] + h * p.vs[1];
-  half_t* ob = p.out + b * p.os[0] + h * p.os[1] + ((int64_t)qi * kBM + 32 * wave) * p.os[2];
+  half_t* ob = p.out + b * p.os[0] + h * p.os[1] + qrow0 * p.os[2];
 
-  // ---- LUT row -> registers: lane i holds entry i (key block, bitmask slot or -1).
-  // LOAD is the sorted union of FULL and PART (get_sparse_storage builds it so), hence an
-  // entry is partial iff its key block is in this row's PART list, otherwise full.
+  // ---- both rows of the pair; every wave walks the same merged sequence of key blocks
   const int64_t lo = (int64_t)b * p.lut_bs;
-  const int t0 = __builtin_amdgcn_readfirstlane(p.lrp[lo + qi]);
-  const int n_ent = __builtin_amdgcn_readfirstlane(p.lrp[lo + qi + 1]) - t0;
-  const int p0 = __builtin_amdgcn_readfirstlane(p.prp[lo + qi]);
-  const int n_part = __builtin_amdgcn_readfirstlane(p.prp[lo + qi + 1]) - p0;
+  LutRow row[2];
+#pragma unroll
+  for (int r = 0; r < 2; ++r) {
+    const int qr = 2 * pair + r;
+    row[r].base = 0;
+    if (qr < p.nQ) {
+      row[r].t0 = __builtin_amdgcn_readfirstlane(p.lrp[lo + qr]);
+      row[r].n = __builtin_amdgcn_readfirstlane(p.lrp[lo + qr + 1]) - row[r].t0;
+      row[r].p0 = __builtin_amdgcn_readfirstlane(p.prp[lo + qr]);
+      row[r].np = __builtin_amdgcn_readfirstlane(p.prp[lo + qr + 1]) - row[r].p0;
+    } else {
+      row[r].t0 = row[r].n = row[r].p0 = row[r].np = 0;
+    }
+    row[r].fill(p, lane, true);
+  }
 
   // Q^T as the B operand: lane (n = query j32, k-group g) holds 8 consecutive d per k-step.
   half8_t qf[4];
 #pragma unroll
-  for (int ks = 0; ks < 4; ++ks)
-    qf[ks] = *reinterpret_cast<const half8_t*>(qb + (int64_t)j32 * p.qs[2] + 16 * ks + 8 * g);
+  for (int ks = 0; ks < 4; ++ks) {
+    if (q_valid) qf[ks] = *reinterpret_cast<const half8_t*>(qb + (int64_t)j32 * p.qs[2] + 16 * ks + 8 * g);
+    else
+#pragma unroll
+      for (int e = 0; e < 8; ++e) qf[ks][e] = (half_t)0.f;
+  }
 
   // ---- per-lane constants of the data movement
-  // DMA: instruction i of this wave fills tile rows 8*(4*wave+i) .. +7 (1 KB of LDS);
-  // lane l lands at (row 8*(4*wave+i) + l/8, chunk position l%8) and therefore fetches
-  // global chunk (l%8) ^ swz(row).
-  int k_src[4], v_src[4];
+  // DMA: a tile is 8 instructions of 1 KB (8 rows of 128 B); wave w issues instructions
+  // 2w and 2w+1 for K and for V.  Lane l lands at (row 8*ii + l/8, chunk position l%8) and
+  // therefore fetches global chunk (l%8) ^ swz(row).
+  int k_src[2], v_src[2];
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int row = 8 * (4 * wave + i) + (lane >> 3);
-    const int chunk = (lane & 7) ^ swz(row);
-    k_src[i] = row * (int)p.ks[2] + 8 * chunk;
-    v_src[i] = row * (int)p.vs[2] + 8 * chunk;
+  for (int i = 0; i < 2; ++i) {
+    const int trow = 8 * (2 * wave + i) + (lane >> 3);
+    const int chunk = (lane & 7) ^ swz(trow);
+    k_src[i] = trow * (int)p.ks[2] + 8 * chunk;
+    v_src[i] = trow * (int)p.vs[2] + 8 * chunk;
   }
   // K fragment (A operand of S^T): row = key 32*mt + j32, chunk 2*ks + g.
   int k_rd[4];
@@ -146,9 +189,9 @@ __global__ __launch_bounds__(128) void block_attn_fwd_kernel(const AttnParams p)
     for (int dt = 0; dt < 2; ++dt)
 #pragma unroll
       for (int hh = 0; hh < 2; ++hh) {
-        const int row = 8 * hh + 4 * g + (j >> 2);
+        const int vrow = 8 * hh + 4 * g + (j >> 2);
         const int chunk = 4 * dt + 2 * dh + ((j >> 1) & 1);
-        v_rd[dt][hh] = row * 128 + ((chunk ^ swz(row)) << 4) + 8 * (j & 1);
+        v_rd[dt][hh] = vrow * 128 + ((chunk ^ swz(vrow)) << 4) + 8 * (j & 1);
       }
   }
 
@@ -163,132 +206,150 @@ __global__ __launch_bounds__(128) void block_attn_fwd_kernel(const AttnParams p)
   auto issue_tile = [&](int col, lds_byte* kdst, lds_byte* vdst) {
     const half_t* kt = kb + (int64_t)col * kBN * p.ks[2];
     const half_t* vt = vb + (int64_t)col * kBN * p.vs[2];
-    lds_byte* kd = kdst + (4 * wave) * 1024;
-    lds_byte* vd = vdst + (4 * wave) * 1024;
+    lds_byte* kd = kdst + (2 * wave) * 1024;
+    lds_byte* vd = vdst + (2 * wave) * 1024;
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < 2; ++i)
       __builtin_amdgcn_global_load_lds((gptr_t*)(kt + k_src[i]), (__attribute__((address_space(3))) void*)(kd + i * 1024), 16, 0, 0);
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < 2; ++i)
       __builtin_amdgcn_global_load_lds((gptr_t*)(vt + v_src[i]), (__attribute__((address_space(3))) void*)(vd + i * 1024), 16, 0, 0);
   };
 
-  for (int base = 0; base < n_ent; base += 64) {
-    const int n_here = min(64, n_ent - base);
-    int ent_col = 0, ent_slot = -1;
-    if (lane < n_here) ent_col = p.lci[t0 + base + lane];
-    for (int pb = 0; pb < n_part; pb += 64) {
-      const int np_here = min(64, n_part - pb);
-      int pc = -1;
-      if (lane < np_here) pc = p.pci[p0 + pb + lane];
-      for (int j = 0; j < np_here; ++j)
-        if (ent_col == __builtin_amdgcn_readlane(pc, j)) ent_slot = p0 + pb + j;
-    }
+  // ---- merged walk over the two rows (wave-uniform and identical in all four waves):
+  // each step takes the smaller head of the two lists; a key block listed by both rows is
+  // loaded once and used by all four waves.
+  int it[2] = {0, 0};   // entries consumed per row
+  struct Step { int col; int mine; int slot; bool valid; };
+  auto next_step = [&]() -> Step {
+    Step s; s.col = 0; s.mine = 0; s.slot = -1; s.valid = false;
+#pragma unroll
+    for (int r = 0; r < 2; ++r)
+      if (it[r] < row[r].n && it[r] - row[r].base == 64) {   // refill the 64-entry window
+        row[r].base += 64;
+        row[r].fill(p, lane, true);
+      }
+    const int ca = it[0] < row[0].n ? __builtin_amdgcn_readlane(row[0].col, it[0] - row[0].base) : 0x7fffffff;
+    const int cb = it[1] < row[1].n ? __builtin_amdgcn_readlane(row[1].col, it[1] - row[1].base) : 0x7fffffff;
+    if (ca == 0x7fffffff && cb == 0x7fffffff) return s;
+    s.valid = true;
+    s.col = min(ca, cb);
+    const bool use_a = ca == s.col, use_b = cb == s.col;
+    const int slot_a = use_a ? __builtin_amdgcn_readlane(row[0].slot, it[0] - row[0].base) : -1;
+    const int slot_b = use_b ? __builtin_amdgcn_readlane(row[1].slot, it[1] - row[1].base) : -1;
+    s.mine = rsel ? use_b : use_a;
+    s.slot = rsel ? slot_b : slot_a;
+    if (use_a) ++it[0];
+    if (use_b) ++it[1];
+    return s;
+  };
 
-    // one key block: kt/vt hold tile t, the loads of tile t+1 go to kn/vn
-    auto step = [&](int t, const lds_byte* kt, const lds_byte* vt, lds_byte* kn, lds_byte* vn) {
-      const int slot = __builtin_amdgcn_readlane(ent_slot, t);
-      // The row mask of a partial tile is fetched first so that its latency hides behind
-      // the wait below and no register-returning load is pending across the DMA issue.
-      uint64_t bits = ~0ull;
-      if (slot >= 0) bits = p.pbits[(int64_t)slot * kBM + 32 * wave + j32];
-      // All DMA issued so far (tile t) has landed for this wave; the barrier makes both
-      // waves' halves visible and also orders last step's reads of the other buffers
-      // before the loads that overwrite them.
-      __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0)
-      __syncthreads();
-      if (t + 1 < n_here) issue_tile(__builtin_amdgcn_readlane(ent_col, t + 1), kn, vn);
+  // one key block: kt/vt hold the current tile, the next tile's loads go to kn/vn
+  auto step = [&](const Step cur, const Step nxt, const lds_byte* kt, const lds_byte* vt, lds_byte* kn, lds_byte* vn) {
+    // The row mask of a partial tile is fetched first so that its latency hides behind
+    // the wait below and no register-returning load is pending across the DMA issue.
+    uint64_t bits = ~0ull;
+    if (cur.slot >= 0) bits = p.pbits[(int64_t)cur.slot * kBM + 32 * half + j32];
+    // All DMA issued so far (the current tile) has landed for this wave; the barrier makes
+    // every wave's share visible and also orders last step's reads of the other buffers
+    // before the loads that overwrite them.
+    __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0)
+    __syncthreads();
+    if (nxt.valid) issue_tile(nxt.col, kn, vn);
+    if (!cur.mine) return;
 
-      // ---- S^T = K . Q^T : sacc[mt][r] = S[query j32][key 32mt + 8(r/4) + 4g + r%4]
-      floatx16 sacc[2];
+    // ---- S^T = K . Q^T : sacc[mt][r] = S[query j32][key 32mt + 8(r/4) + 4g + r%4]
+    floatx16 sacc[2];
 #pragma unroll
-      for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < 2; ++i)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) sacc[i][r] = 0.f;
+      for (int r = 0; r < 16; ++r) sacc[i][r] = 0.f;
 #pragma unroll
-      for (int ks = 0; ks < 4; ++ks)
+    for (int ks = 0; ks < 4; ++ks)
 #pragma unroll
-        for (int mt = 0; mt < 2; ++mt) {
-          const half8_t a = *reinterpret_cast<const __attribute__((address_space(3))) half8_t*>(kt + mt * 4096 + k_rd[ks]);
-          sacc[mt] = mfma32(a, qf[ks], sacc[mt]);
-        }
-
-      // ---- element mask of a partial tile
-      if (slot >= 0) {
-#pragma unroll
-        for (int mt = 0; mt < 2; ++mt) {
-          const uint32_t w = (uint32_t)(bits >> (32 * mt)) >> (4 * g);
-#pragma unroll
-          for (int r = 0; r < 16; ++r)
-            if (!((w >> (8 * (r >> 2) + (r & 3))) & 1u)) sacc[mt][r] = kMasked;
-        }
+      for (int mt = 0; mt < 2; ++mt) {
+        const half8_t a = *reinterpret_cast<const __attribute__((address_space(3))) half8_t*>(kt + mt * 4096 + k_rd[ks]);
+        sacc[mt] = mfma32(a, qf[ks], sacc[mt]);
       }
 
-      // ---- online softmax; one query per lane (shared with the partner lane ^ 32).
-      // The running max is only raised when the tile's max exceeds it by more than kLazy
-      // (in log2 units): probabilities then stay below 2^kLazy, well inside fp16 range, the
-      // normalisation by the running sum stays exact, and the O rescale becomes rare.
-      float mx = sacc[0][0];
+    // ---- element mask of a partial tile
+    if (cur.slot >= 0) {
 #pragma unroll
-      for (int mt = 0; mt < 2; ++mt)
+      for (int mt = 0; mt < 2; ++mt) {
+        const uint32_t w = (uint32_t)(bits >> (32 * mt)) >> (4 * g);
 #pragma unroll
-        for (int r = 0; r < 16; ++r) mx = fmaxf(mx, sacc[mt][r]);
-      mx = pair_max(mx);
-      const float m_new = (mx * p.c > m_run * p.c + kLazy || m_run == -INFINITY) ? mx : m_run;
-      // A row that has seen no allowed key yet has m_new == -inf: subtract 0 instead, so
-      // that its probabilities are exp2(-inf) = 0 and no inf - inf appears.
-      const float m_sub = (m_new == -INFINITY) ? 0.f : m_new;
-      const float alpha = __builtin_amdgcn_exp2f((m_run - m_sub) * p.c);
-      const float mc = m_sub * p.c;
-      half8_t pf[2][2];   // [key tile][half]: B operand of O^T = V^T . P^T
-      float lsum = 0.f;
-      const half2_t ones2 = {(half_t)1.0f, (half_t)1.0f};
-#pragma unroll
-      for (int mt = 0; mt < 2; ++mt)
-#pragma unroll
-        for (int r = 0; r < 16; r += 2) {
-          const float e0 = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[mt][r], p.c, -mc));
-          const float e1 = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[mt][r + 1], p.c, -mc));
-          const half2_t e2 = {(half_t)e0, (half_t)e1};
-          pf[mt][r >> 3][r & 7] = e2[0];
-          pf[mt][r >> 3][(r & 7) + 1] = e2[1];
-          // row sum of the ROUNDED probabilities (what P.V multiplies), two per instruction
-          lsum = __builtin_amdgcn_fdot2(e2, ones2, lsum, false);
-        }
-      l_run = l_run * alpha + lsum;   // per-lane partial sum; the two halves are added at the end
-      m_run = m_new;
-      if (__any(alpha != 1.0f)) {
-#pragma unroll
-        for (int dt = 0; dt < 2; ++dt)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) oacc[dt][r] *= alpha;
+        for (int r = 0; r < 16; ++r)
+          if (!((w >> (8 * (r >> 2) + (r & 3))) & 1u)) sacc[mt][r] = kMasked;
       }
-
-      // ---- O^T += V^T . P^T
-#pragma unroll
-      for (int mt = 0; mt < 2; ++mt)
-#pragma unroll
-        for (int s2 = 0; s2 < 2; ++s2)
-#pragma unroll
-          for (int dt = 0; dt < 2; ++dt) {
-            const lds_byte* vp = vt + (32 * mt + 16 * s2) * 128;
-            const short4_t a0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4*)(vp + v_rd[dt][0]));
-            const short4_t a1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4*)(vp + v_rd[dt][1]));
-            const half8_t a = __builtin_bit_cast(half8_t, (short8_t)__builtin_shufflevector(a0, a1, 0, 1, 2, 3, 4, 5, 6, 7));
-            oacc[dt] = mfma32(a, pf[mt][s2], oacc[dt]);
-          }
-    };
-
-    issue_tile(__builtin_amdgcn_readlane(ent_col, 0), (lds_byte*)k_lds0, (lds_byte*)v_lds0);
-    for (int t = 0; t < n_here; t += 2) {
-      step(t, (const lds_byte*)k_lds0, (const lds_byte*)v_lds0, (lds_byte*)k_lds1, (lds_byte*)v_lds1);
-      if (t + 1 < n_here)
-        step(t + 1, (const lds_byte*)k_lds1, (const lds_byte*)v_lds1, (lds_byte*)k_lds0, (lds_byte*)v_lds0);
     }
-    __syncthreads();   // the next chunk's first loads overwrite buffer 0
+
+    // ---- online softmax; one query per lane (shared with the partner lane ^ 32).
+    // The running max is only raised when the tile's max exceeds it by more than kLazy
+    // (in log2 units): probabilities then stay below 2^kLazy, well inside fp16 range, the
+    // normalisation by the running sum stays exact, and the O rescale becomes rare.
+    float mx = sacc[0][0];
+#pragma unroll
+    for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) mx = fmaxf(mx, sacc[mt][r]);
+    mx = pair_max(mx);
+    const float m_new = (mx * p.c > m_run * p.c + kLazy || m_run == -INFINITY) ? mx : m_run;
+    // A row that has seen no allowed key yet has m_new == -inf: subtract 0 instead, so
+    // that its probabilities are exp2(-inf) = 0 and no inf - inf appears.
+    const float m_sub = (m_new == -INFINITY) ? 0.f : m_new;
+    const float alpha = __builtin_amdgcn_exp2f((m_run - m_sub) * p.c);
+    const float mc = m_sub * p.c;
+    half8_t pf[2][2];   // [key tile][half]: B operand of O^T = V^T . P^T
+    float lsum = 0.f;
+    const half2_t ones2 = {(half_t)1.0f, (half_t)1.0f};
+#pragma unroll
+    for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+      for (int r = 0; r < 16; r += 2) {
+        const float e0 = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[mt][r], p.c, -mc));
+        const float e1 = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[mt][r + 1], p.c, -mc));
+        const half2_t e2 = {(half_t)e0, (half_t)e1};
+        pf[mt][r >> 3][r & 7] = e2[0];
+        pf[mt][r >> 3][(r & 7) + 1] = e2[1];
+        // row sum of the ROUNDED probabilities (what P.V multiplies), two per instruction
+        lsum = __builtin_amdgcn_fdot2(e2, ones2, lsum, false);
+      }
+    l_run = l_run * alpha + lsum;   // per-lane partial sum; the two halves are added at the end
+    m_run = m_new;
+    if (__any(alpha != 1.0f)) {
+#pragma unroll
+      for (int dt = 0; dt < 2; ++dt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) oacc[dt][r] *= alpha;
+    }
+
+    // ---- O^T += V^T . P^T
+#pragma unroll
+    for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+      for (int s2 = 0; s2 < 2; ++s2)
+#pragma unroll
+        for (int dt = 0; dt < 2; ++dt) {
+          const lds_byte* vp = vt + (32 * mt + 16 * s2) * 128;
+          const short4_t a0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4*)(vp + v_rd[dt][0]));
+          const short4_t a1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4*)(vp + v_rd[dt][1]));
+          const half8_t a = __builtin_bit_cast(half8_t, (short8_t)__builtin_shufflevector(a0, a1, 0, 1, 2, 3, 4, 5, 6, 7));
+          oacc[dt] = mfma32(a, pf[mt][s2], oacc[dt]);
+        }
+  };
+
+  Step cur = next_step();
+  if (cur.valid) issue_tile(cur.col, (lds_byte*)k_lds0, (lds_byte*)v_lds0);
+  while (cur.valid) {
+    Step nxt = next_step();
+    step(cur, nxt, (const lds_byte*)k_lds0, (const lds_byte*)v_lds0, (lds_byte*)k_lds1, (lds_byte*)v_lds1);
+    if (!nxt.valid) break;
+    cur = next_step();
+    step(nxt, cur, (const lds_byte*)k_lds1, (const lds_byte*)v_lds1, (lds_byte*)k_lds0, (lds_byte*)v_lds0);
   }
 
   // ---- normalise and store: oacc[dt][r] = O[query j32][d = 32dt + 8(r/4) + 4g + r%4]
+  if (!q_valid) return;
   const float l = pair_sum(l_run);
   const float inv = (l > 0.f) ? 1.0f / l : 0.f;   // no allowed key at all: zeros
   half_t* orow = ob + (int64_t)j32 * p.os[2];
@@ -352,7 +413,8 @@ extern "C" int stof_block_attn_fwd(
   if (!stof_aligned16(q) || !stof_aligned16(k) || !stof_aligned16(v) || !stof_aligned16(out)) return STOF_ERR_MISALIGNED;
   if (!strides_ok(q_strides) || !strides_ok(k_strides) || !strides_ok(v_strides) || !strides_ok(out_strides))
     return STOF_ERR_MISALIGNED;
-  const int64_t total64 = (int64_t)nQ * batch_size * head_num;
+  const int nP = (nQ + 1) / 2;
+  const int64_t total64 = (int64_t)nP * batch_size * head_num;
   if (total64 > (int64_t)1 << 30) return STOF_ERR_BAD_SHAPE;
 
   AttnParams p;
@@ -361,11 +423,11 @@ extern "C" int stof_block_attn_fwd(
   p.pbits = part_bitmask; p.lrp = load_row_ptr; p.lci = load_col_idx;
   for (int i = 0; i < 3; ++i) { p.qs[i] = q_strides[i]; p.ks[i] = k_strides[i]; p.vs[i] = v_strides[i]; p.os[i] = out_strides[i]; }
   p.lut_bs = lut_batch_stride;
-  p.B = batch_size; p.S = seq_len; p.H = head_num; p.nQ = nQ;
+  p.B = batch_size; p.S = seq_len; p.H = head_num; p.nQ = nQ; p.nP = nP;
   p.total = (int)total64;
   p.chunk = (p.total + 7) / 8;
   p.c = softmax_scale * 1.4426950408889634f;
-  hipLaunchKernelGGL(block_attn_fwd_kernel, dim3(p.chunk * 8), dim3(128), 0, (hipStream_t)stream, p);
+  hipLaunchKernelGGL(block_attn_fwd_kernel, dim3(p.chunk * 8), dim3(256), 0, (hipStream_t)stream, p);
   return stof_check_launch();
 }
 
