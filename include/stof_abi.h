@@ -64,11 +64,14 @@ const char* stof_status_string(int status);
 /*
  * Block-masked multi-head attention, forward.
  *   out[b,h,i,:] = sum_j softmax_j( scale * q[b,h,i,:].k[b,h,j,:]  over allowed j ) v[b,h,j,:]
- * where the allowed (i,j) are described by the block LUT: key blocks listed in LOAD for
- * query block i/block_m are visited in order; one that is next in the PART list uses the
- * 64-bit row masks part_bitmask[slot*block_m + (i % block_m)] (bit j%block_n set = allowed),
- * one that is next in the FULL list is unmasked, any other is skipped (the rule of
- * block_attn_mask_cuda.cu:3675-3700).  Query rows without any allowed key produce zeros.
+ * where the allowed (i,j) are described by the block LUT: the key blocks listed in LOAD for
+ * query block i/block_m are visited; one that also appears in that row's PART list (at
+ * position `slot` of the PART arrays) uses the 64-bit row masks
+ * part_bitmask[slot*block_m + (i % block_m)] (bit j%block_n set = allowed), any other is
+ * unmasked.  LOAD must be the union of FULL and PART, as get_sparse_storage builds it
+ * (src/util/masks.py:149-166), which makes this the three-way rule of
+ * block_attn_mask_cuda.cu:3675-3700; the FULL arrays are accepted for signature parity and
+ * not read.  Query rows without any allowed key produce zeros.
  *
  * Tensors are addressed as base + b*stride_b + h*stride_h + s*stride_s + d (strides in
  * ELEMENTS, d contiguous), separately for q, k, v and out, so [B,H,S,D], [B,S,H,D] and
@@ -132,7 +135,7 @@ int stof_bias_res_ln(const void* x, const void* bias, const void* residual,
 /*
  * C[M,N] = act( A[M,K] @ W^T + bias[N] ) with W given as Wt[N,K] (K contiguous, the
  * nn.Linear orientation).  A rows at pitch lda, C rows at pitch ldc (elements).
- * K % 32 == 0, N % 8 == 0; M arbitrary.  bias may be NULL.
+ * K % 64 == 0, N % 8 == 0, lda % 8 == 0, ldc % 4 == 0; M arbitrary.  bias may be NULL.
  */
 int stof_gemm_bias_act(const void* A, const void* Wt, const void* bias, void* C,
                        int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldc,

@@ -55,7 +55,11 @@ struct AttnParams {
   int B, S, H, nQ, nP;   // nP = query-block pairs per (batch, head)
   int total, chunk;
   float c;  // softmax_scale * log2(e)
+  // row-wise front-ends (KIND != 0): key blocks come from index arithmetic, not from a LUT
+  const uint64_t* row_bits; int words; int causal; int band;
 };
+
+enum { kKindLut = 0, kKindPred = 1, kKindBits = 2 };
 
 __device__ __forceinline__ floatx16 mfma32(half8_t a, half8_t b, floatx16 c) {
   return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
@@ -100,6 +104,7 @@ struct LutRow {
   }
 };
 
+template <int KIND>
 __global__ __launch_bounds__(256) void block_attn_fwd_kernel(const AttnParams p) {
   // Four distinct LDS objects (K and V, two buffers each): the compiler orders LDS reads
   // after in-flight direct-to-LDS loads per object, so a read of the current buffer does
@@ -137,19 +142,29 @@ __global__ __launch_bounds__(256) void block_attn_fwd_kernel(const AttnParams p)
   // ---- both rows of the pair; every wave walks the same merged sequence of key blocks
   const int64_t lo = (int64_t)b * p.lut_bs;
   LutRow row[2];
+  int row_lo[2] = {0, 0};   // KIND != 0: first key block of each row's contiguous range
 #pragma unroll
   for (int r = 0; r < 2; ++r) {
     const int qr = 2 * pair + r;
     row[r].base = 0;
+    row[r].t0 = row[r].n = row[r].p0 = row[r].np = 0;
+    row[r].col = 0; row[r].slot = -1;
     if (qr < p.nQ) {
-      row[r].t0 = __builtin_amdgcn_readfirstlane(p.lrp[lo + qr]);
-      row[r].n = __builtin_amdgcn_readfirstlane(p.lrp[lo + qr + 1]) - row[r].t0;
-      row[r].p0 = __builtin_amdgcn_readfirstlane(p.prp[lo + qr]);
-      row[r].np = __builtin_amdgcn_readfirstlane(p.prp[lo + qr + 1]) - row[r].p0;
-    } else {
-      row[r].t0 = row[r].n = row[r].p0 = row[r].np = 0;
+      if (KIND == kKindLut) {
+        row[r].t0 = __builtin_amdgcn_readfirstlane(p.lrp[lo + qr]);
+        row[r].n = __builtin_amdgcn_readfirstlane(p.lrp[lo + qr + 1]) - row[r].t0;
+        row[r].p0 = __builtin_amdgcn_readfirstlane(p.prp[lo + qr]);
+        row[r].np = __builtin_amdgcn_readfirstlane(p.prp[lo + qr + 1]) - row[r].p0;
+      } else {
+        // keys allowed for some query of block qr: (64qr - band, 64qr + 63] when sliding,
+        // up to the diagonal block when causal, else every block
+        const int hi = p.causal ? qr : p.nQ - 1;
+        const int first_key = (KIND == kKindPred && p.band > 0) ? 64 * qr - p.band + 1 : 0;
+        row_lo[r] = first_key > 0 ? first_key / 64 : 0;
+        row[r].n = hi - row_lo[r] + 1 > 0 ? hi - row_lo[r] + 1 : 0;
+      }
     }
-    row[r].fill(p, lane, true);
+    if (KIND == kKindLut) row[r].fill(p, lane, true);
   }
 
   // Q^T as the B operand: lane (n = query j32, k-group g) holds 8 consecutive d per k-step.
@@ -223,20 +238,29 @@ __global__ __launch_bounds__(256) void block_attn_fwd_kernel(const AttnParams p)
   struct Step { int col; int mine; int slot; bool valid; };
   auto next_step = [&]() -> Step {
     Step s; s.col = 0; s.mine = 0; s.slot = -1; s.valid = false;
+    int ca = 0x7fffffff, cb = 0x7fffffff;
+    if (KIND == kKindLut) {
 #pragma unroll
-    for (int r = 0; r < 2; ++r)
-      if (it[r] < row[r].n && it[r] - row[r].base == 64) {   // refill the 64-entry window
-        row[r].base += 64;
-        row[r].fill(p, lane, true);
-      }
-    const int ca = it[0] < row[0].n ? __builtin_amdgcn_readlane(row[0].col, it[0] - row[0].base) : 0x7fffffff;
-    const int cb = it[1] < row[1].n ? __builtin_amdgcn_readlane(row[1].col, it[1] - row[1].base) : 0x7fffffff;
+      for (int r = 0; r < 2; ++r)
+        if (it[r] < row[r].n && it[r] - row[r].base == 64) {   // refill the 64-entry window
+          row[r].base += 64;
+          row[r].fill(p, lane, true);
+        }
+      if (it[0] < row[0].n) ca = __builtin_amdgcn_readlane(row[0].col, it[0] - row[0].base);
+      if (it[1] < row[1].n) cb = __builtin_amdgcn_readlane(row[1].col, it[1] - row[1].base);
+    } else {
+      if (it[0] < row[0].n) ca = row_lo[0] + it[0];
+      if (it[1] < row[1].n) cb = row_lo[1] + it[1];
+    }
     if (ca == 0x7fffffff && cb == 0x7fffffff) return s;
     s.valid = true;
     s.col = min(ca, cb);
     const bool use_a = ca == s.col, use_b = cb == s.col;
-    const int slot_a = use_a ? __builtin_amdgcn_readlane(row[0].slot, it[0] - row[0].base) : -1;
-    const int slot_b = use_b ? __builtin_amdgcn_readlane(row[1].slot, it[1] - row[1].base) : -1;
+    int slot_a = -1, slot_b = -1;
+    if (KIND == kKindLut) {
+      if (use_a) slot_a = __builtin_amdgcn_readlane(row[0].slot, it[0] - row[0].base);
+      if (use_b) slot_b = __builtin_amdgcn_readlane(row[1].slot, it[1] - row[1].base);
+    }
     s.mine = rsel ? use_b : use_a;
     s.slot = rsel ? slot_b : slot_a;
     if (use_a) ++it[0];
@@ -249,7 +273,11 @@ __global__ __launch_bounds__(256) void block_attn_fwd_kernel(const AttnParams p)
     // The row mask of a partial tile is fetched first so that its latency hides behind
     // the wait below and no register-returning load is pending across the DMA issue.
     uint64_t bits = ~0ull;
-    if (cur.slot >= 0) bits = p.pbits[(int64_t)cur.slot * kBM + 32 * half + j32];
+    if (KIND == kKindLut) {
+      if (cur.slot >= 0) bits = p.pbits[(int64_t)cur.slot * kBM + 32 * half + j32];
+    } else if (KIND == kKindBits) {
+      if (cur.mine) bits = p.row_bits[(qrow0 + j32) * p.words + cur.col];
+    }
     // All DMA issued so far (the current tile) has landed for this wave; the barrier makes
     // every wave's share visible and also orders last step's reads of the other buffers
     // before the loads that overwrite them.
@@ -257,6 +285,27 @@ __global__ __launch_bounds__(256) void block_attn_fwd_kernel(const AttnParams p)
     __syncthreads();
     if (nxt.valid) issue_tile(nxt.col, kn, vn);
     if (!cur.mine) return;
+    // Row-wise front-ends: which elements of this tile may be used.  need_mask is wave-uniform.
+    bool need_mask = (KIND == kKindLut) ? (cur.slot >= 0) : false;
+    if (KIND != kKindLut) {
+      const int qmin = (int)qrow0, qmax = qmin + 31, kmin = cur.col * kBN, kmax = kmin + kBN - 1;
+      const bool range_full = (!p.causal || kmax <= qmin) && (!(KIND == kKindPred && p.band > 0) || kmin > qmax - p.band);
+      if (KIND == kKindBits) {
+        if (!__any(bits != 0ull)) return;            // nothing allowed for these 32 queries
+        need_mask = !range_full || __any(bits != ~0ull);
+      } else {
+        need_mask = !range_full;
+      }
+      if (need_mask) {
+        // fold the index predicates into the bit row: bit t = key kmin + t allowed
+        const int qg = qmin + j32;
+        if (p.causal) { const int nk = qg - kmin + 1; bits &= nk >= 64 ? ~0ull : (nk <= 0 ? 0ull : ((1ull << nk) - 1)); }
+        if (KIND == kKindPred && p.band > 0) {
+          const int first = qg - p.band + 1 - kmin;   // keys below this offset are outside the window
+          bits &= first <= 0 ? ~0ull : (first >= 64 ? 0ull : ~((1ull << first) - 1));
+        }
+      }
+    }
 
     // ---- S^T = K . Q^T : sacc[mt][r] = S[query j32][key 32mt + 8(r/4) + 4g + r%4]
     floatx16 sacc[2];
@@ -273,7 +322,7 @@ __global__ __launch_bounds__(256) void block_attn_fwd_kernel(const AttnParams p)
       }
 
     // ---- element mask of a partial tile
-    if (cur.slot >= 0) {
+    if (need_mask) {
 #pragma unroll
       for (int mt = 0; mt < 2; ++mt) {
         const uint32_t w = (uint32_t)(bits >> (32 * mt)) >> (4 * g);
@@ -427,7 +476,42 @@ extern "C" int stof_block_attn_fwd(
   p.total = (int)total64;
   p.chunk = (p.total + 7) / 8;
   p.c = softmax_scale * 1.4426950408889634f;
-  hipLaunchKernelGGL(block_attn_fwd_kernel, dim3(p.chunk * 8), dim3(256), 0, (hipStream_t)stream, p);
+  p.row_bits = nullptr; p.words = 0; p.causal = 0; p.band = 0;
+  hipLaunchKernelGGL(block_attn_fwd_kernel<kKindLut>, dim3(p.chunk * 8), dim3(256), 0, (hipStream_t)stream, p);
+  return stof_check_launch();
+}
+
+extern "C" int stof_rowwise_attn_fwd(
+    const void* q, const void* k, const void* v, void* out,
+    int kind, int is_causal, int bandwidth, const uint64_t* mask_bits,
+    int batch_size, int seq_len, int head_num, int head_size, void* stream) {
+  if (!q || !k || !v || !out) return STOF_ERR_NULL_POINTER;
+  if (kind != STOF_ROW_FULL && kind != STOF_ROW_SLIDING && kind != STOF_ROW_MASK) return STOF_ERR_UNSUPPORTED;
+  if (kind == STOF_ROW_MASK && !mask_bits) return STOF_ERR_NULL_POINTER;
+  if (batch_size <= 0 || seq_len <= 0 || head_num <= 0 || head_size <= 0) return STOF_ERR_BAD_SHAPE;
+  if (head_size != kD) return STOF_ERR_UNSUPPORTED;
+  if (seq_len % kBM != 0) return STOF_ERR_BAD_SHAPE;
+  if (kind == STOF_ROW_SLIDING && bandwidth <= 0) return STOF_ERR_BAD_SHAPE;
+  if (!stof_aligned16(q) || !stof_aligned16(k) || !stof_aligned16(v) || !stof_aligned16(out)) return STOF_ERR_MISALIGNED;
+  const int nQ = seq_len / kBM, nP = (nQ + 1) / 2;
+  const int64_t total64 = (int64_t)nP * batch_size * head_num;
+  if (total64 > (int64_t)1 << 30) return STOF_ERR_BAD_SHAPE;
+  AttnParams p;
+  p.q = (const half_t*)q; p.k = (const half_t*)k; p.v = (const half_t*)v; p.out = (half_t*)out;
+  p.prp = nullptr; p.pci = nullptr; p.pbits = nullptr; p.lrp = nullptr; p.lci = nullptr;
+  const int64_t in_s[3] = {(int64_t)head_num * seq_len * kD, (int64_t)seq_len * kD, kD};
+  const int64_t out_s[3] = {(int64_t)seq_len * head_num * kD, kD, (int64_t)head_num * kD};   // [B,S,H*D]
+  for (int i = 0; i < 3; ++i) { p.qs[i] = in_s[i]; p.ks[i] = in_s[i]; p.vs[i] = in_s[i]; p.os[i] = out_s[i]; }
+  p.lut_bs = 0;
+  p.B = batch_size; p.S = seq_len; p.H = head_num; p.nQ = nQ; p.nP = nP;
+  p.total = (int)total64; p.chunk = (p.total + 7) / 8;
+  p.c = (1.0f / sqrtf((float)head_size)) * 1.4426950408889634f;
+  p.row_bits = mask_bits; p.words = seq_len / 64; p.causal = is_causal ? 1 : 0;
+  p.band = kind == STOF_ROW_SLIDING ? bandwidth : 0;
+  if (kind == STOF_ROW_MASK)
+    hipLaunchKernelGGL(block_attn_fwd_kernel<kKindBits>, dim3(p.chunk * 8), dim3(256), 0, (hipStream_t)stream, p);
+  else
+    hipLaunchKernelGGL(block_attn_fwd_kernel<kKindPred>, dim3(p.chunk * 8), dim3(256), 0, (hipStream_t)stream, p);
   return stof_check_launch();
 }
 

@@ -1,0 +1,393 @@
+// Fused encoder GEMMs for gfx950 (MI355X):
+//   stof_gemm_bias_act     C = act(A @ W^T + bias)                       (bias / GELU / ReLU epilogue)
+//   stof_gemm_bias_res_ln  C = LN(A @ W^T + bias + residual) * g + b     (LayerNorm epilogue)
+//
+// They replace the reference's Triton templates (src/triton_template/gemm_gemm.py:99-150,
+// src/triton_template/gemm_add_layernorm.py:78-123).  Common design:
+//
+//  * both operands are K-contiguous (A [M,K], Wt [N,K]) and travel L2 -> LDS with
+//    direct-to-LDS loads, double buffered, one barrier per K tile; LDS tiles are unpadded
+//    rows of 128 B (64 halves) with a 16-byte-chunk XOR swizzle, so the 16-byte fragment
+//    reads of 16 consecutive rows hit distinct banks;
+//  * the product is formed TRANSPOSED, C^T = Wt . A^T, with v_mfma_f32_32x32x16_f16: the
+//    weights are the A operand, the activations the B operand.  In the accumulator layout
+//    a lane then owns ONE token row (lane & 31) and its registers run along the feature
+//    dimension in groups of four consecutive columns.  Bias, activation, residual and the
+//    LayerNorm statistics become per-lane register loops, and stores are 8-byte vectors;
+//  * the LayerNorm kernel gives one workgroup (8 waves) the full row of N features, each
+//    wave a slice of N/8 columns; mean and variance are reduced in registers, across the
+//    lane pair with v_permlane32_swap and across the 8 waves through 2 KB of LDS, so the
+//    pre-normalisation tensor never leaves the chip.
+#include "stof_common.h"
+
+namespace {
+
+typedef __attribute__((address_space(3))) unsigned char lds_byte;
+typedef __attribute__((address_space(1))) const void gptr_t;
+
+__device__ __forceinline__ floatx16 mfma32(half8_t a, half8_t b, floatx16 c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+}
+__device__ __forceinline__ float pair_sum(float x) {
+  const unsigned u = __builtin_bit_cast(unsigned, x);
+  const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  return __builtin_bit_cast(float, (unsigned)r[0]) + __builtin_bit_cast(float, (unsigned)r[1]);
+}
+// chunk c (16 B) of tile row r is stored at chunk position c ^ swz(r)
+__device__ __forceinline__ int swz(int row) { return (((row >> 1) & 1) << 2) | ((row >> 2) & 3); }
+
+__device__ __forceinline__ half8_t lds_frag(const lds_byte* tile, int byte_off) {
+  return *reinterpret_cast<const __attribute__((address_space(3))) half8_t*>(tile + byte_off);
+}
+__device__ __forceinline__ void dma16(const half_t* src, lds_byte* dst) {
+  __builtin_amdgcn_global_load_lds((gptr_t*)src, (__attribute__((address_space(3))) void*)dst, 16, 0, 0);
+}
+
+__device__ __forceinline__ float gelu_erf(float x) { return 0.5f * x * (1.0f + erff(x * 0.70710678118654752f)); }
+__device__ __forceinline__ float gelu_tanh(float x) {
+  // 0.5 x (1 + tanh(u)) = x * sigmoid(2u),  u = sqrt(2/pi) (x + 0.044715 x^3)
+  const float u = 0.7978845608028654f * (x + 0.044715f * x * x * x);
+  return x / (1.0f + __expf(-2.0f * u));
+}
+template <int ACT> __device__ __forceinline__ float activate(float x) {
+  if (ACT == STOF_ACT_GELU_ERF) return gelu_erf(x);
+  if (ACT == STOF_ACT_GELU_TANH) return gelu_tanh(x);
+  if (ACT == STOF_ACT_RELU) return fmaxf(x, 0.f);
+  return x;
+}
+
+// ------------------------------------------------------------------------------------------
+// C[M,N] = act(A[M,K] @ Wt[N,K]^T + bias[N]);  tile 128 (tokens) x 128 (features) x 64 (K),
+// 4 waves as 2 x 2, each 64 tokens x 64 features = 2 x 2 MFMA tiles.
+// ------------------------------------------------------------------------------------------
+struct GemmParams {
+  const half_t* A; const half_t* W; const half_t* bias; half_t* C;
+  int M, N, K; int lda, ldc;
+  int tiles_m, tiles_n;
+};
+
+constexpr int kGT = 128;            // tile edge (tokens and features)
+constexpr int kGK = 64;             // K per tile
+constexpr int kGTile = kGT * kGK * 2;   // bytes per operand tile (16 KB)
+
+template <int ACT>
+__global__ __launch_bounds__(256) void gemm_bias_act_kernel(const GemmParams p) {
+  __shared__ __attribute__((aligned(1024))) unsigned char a_lds0[kGTile];
+  __shared__ __attribute__((aligned(1024))) unsigned char a_lds1[kGTile];
+  __shared__ __attribute__((aligned(1024))) unsigned char w_lds0[kGTile];
+  __shared__ __attribute__((aligned(1024))) unsigned char w_lds1[kGTile];
+
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
+  const int j32 = lane & 31, g = lane >> 5;
+  const int wm = wave >> 1, wn = wave & 1;
+
+  // Consecutive workgroups share the weight tile (same tn) and walk the token tiles, so the
+  // weight tile stays hot in L2 while activations stream.
+  const int tm = blockIdx.x % p.tiles_m;
+  const int tn = blockIdx.x / p.tiles_m;
+  const int m0 = tm * kGT, n0 = tn * kGT;
+
+  // DMA: 16 instructions of 8 rows per operand tile; wave w issues 4w..4w+3.
+  const half_t* a_src[4]; const half_t* w_src[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int trow = 8 * (4 * wave + i) + (lane >> 3);
+    const int chunk = (lane & 7) ^ swz(trow);
+    const int am = min(m0 + trow, p.M - 1);       // rows past the edge re-read the last row
+    const int wnr = min(n0 + trow, p.N - 1);
+    a_src[i] = p.A + (int64_t)am * p.lda + 8 * chunk;
+    w_src[i] = p.W + (int64_t)wnr * p.K + 8 * chunk;
+  }
+  auto issue = [&](int kt, lds_byte* ad, lds_byte* wd) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) dma16(a_src[i] + kt * kGK, ad + (4 * wave + i) * 1024);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) dma16(w_src[i] + kt * kGK, wd + (4 * wave + i) * 1024);
+  };
+  // fragment read offsets: row (32*t + j32), chunk 2*ks + g
+  int rd[4];
+#pragma unroll
+  for (int ks = 0; ks < 4; ++ks) rd[ks] = j32 * 128 + (((2 * ks + g) ^ swz(j32)) << 4);
+
+  floatx16 acc[2][2];   // [feature tile ni][token tile mi]
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+  auto compute = [&](const lds_byte* at, const lds_byte* wt) {
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+      half8_t xa[2], wb[2];
+#pragma unroll
+      for (int mi = 0; mi < 2; ++mi) xa[mi] = lds_frag(at, (64 * wm + 32 * mi) * 128 + rd[ks]);
+#pragma unroll
+      for (int ni = 0; ni < 2; ++ni) wb[ni] = lds_frag(wt, (64 * wn + 32 * ni) * 128 + rd[ks]);
+#pragma unroll
+      for (int ni = 0; ni < 2; ++ni)
+#pragma unroll
+        for (int mi = 0; mi < 2; ++mi) acc[ni][mi] = mfma32(wb[ni], xa[mi], acc[ni][mi]);
+    }
+  };
+
+  const int nk = p.K / kGK;
+  issue(0, (lds_byte*)a_lds0, (lds_byte*)w_lds0);
+  for (int kt = 0; kt < nk; kt += 2) {
+    __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): this wave's share of tile kt landed
+    __syncthreads();
+    if (kt + 1 < nk) issue(kt + 1, (lds_byte*)a_lds1, (lds_byte*)w_lds1);
+    compute((const lds_byte*)a_lds0, (const lds_byte*)w_lds0);
+    if (kt + 1 >= nk) break;
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+    __syncthreads();
+    if (kt + 2 < nk) issue(kt + 2, (lds_byte*)a_lds0, (lds_byte*)w_lds0);
+    compute((const lds_byte*)a_lds1, (const lds_byte*)w_lds1);
+  }
+
+  // epilogue: acc[ni][mi][r] = C[m0 + 64wm + 32mi + j32][n0 + 64wn + 32ni + 8(r/4) + 4g + r%4]
+#pragma unroll
+  for (int mi = 0; mi < 2; ++mi) {
+    const int m = m0 + 64 * wm + 32 * mi + j32;
+    if (m >= p.M) continue;
+    half_t* crow = p.C + (int64_t)m * p.ldc;
+#pragma unroll
+    for (int ni = 0; ni < 2; ++ni)
+#pragma unroll
+      for (int q4 = 0; q4 < 4; ++q4) {
+        const int n = n0 + 64 * wn + 32 * ni + 8 * q4 + 4 * g;
+        if (n >= p.N) continue;          // N % 8 == 0: a group of 4 is inside or outside as a whole
+        half4_t bv = {(half_t)0.f, (half_t)0.f, (half_t)0.f, (half_t)0.f};
+        if (p.bias) bv = *reinterpret_cast<const half4_t*>(p.bias + n);
+        half4_t o;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) o[e] = (half_t)activate<ACT>(acc[ni][mi][4 * q4 + e] + (float)bv[e]);
+        *reinterpret_cast<half4_t*>(crow + n) = o;
+      }
+  }
+}
+
+// ------------------------------------------------------------------------------------------
+// C[M,N] = LN(A @ Wt^T + bias + residual) * gamma + beta, N = 256 * NC, one workgroup of 8
+// waves per 64 token rows; wave w owns features [32*NC*w, 32*NC*(w+1)).  K tile = 32.
+// ------------------------------------------------------------------------------------------
+struct LnGemmParams {
+  const half_t* A; const half_t* W; const half_t* bias; const half_t* res;
+  const half_t* gamma; const half_t* beta; half_t* C;
+  int M, N, K; float eps; float inv_n;
+};
+
+constexpr int kLM = 64;    // token rows per workgroup
+constexpr int kLK = 32;    // K per tile: rows of 64 B, 4 chunks of 16 B
+
+// 64-byte rows: chunk c of row r sits at position c ^ ((r >> 2) & 3); 16 rows fill 1 KB.
+__device__ __forceinline__ int swz4(int row) { return (row >> 2) & 3; }
+
+template <int NC>
+__global__ __launch_bounds__(512) void gemm_bias_res_ln_kernel(const LnGemmParams p) {
+  constexpr int N = 256 * NC;
+  constexpr int kWTile = N * kLK * 2;      // weight tile bytes: 16 KB * NC
+  constexpr int kATile = kLM * kLK * 2;    // 4 KB
+  __shared__ __attribute__((aligned(1024))) unsigned char w_lds0[kWTile];
+  __shared__ __attribute__((aligned(1024))) unsigned char w_lds1[kWTile];
+  __shared__ __attribute__((aligned(1024))) unsigned char a_lds0[kATile];
+  __shared__ __attribute__((aligned(1024))) unsigned char a_lds1[kATile];
+  __shared__ float red[2][8][kLM];         // per-wave partial sums for mean / variance
+
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
+  const int j32 = lane & 31, g = lane >> 5;
+  const int m0 = blockIdx.x * kLM;
+
+  // DMA: one instruction = 16 rows of 64 B.  Weight tile: 16*NC instructions, 2*NC per wave
+  // (its OWN feature rows: wave w reads back exactly what it loaded, plus the shared A tile);
+  // A tile: 4 instructions, issued by waves 0..3.
+  const int drow = lane >> 2;                    // row within the instruction's 16
+  const half_t* w_src[2 * NC];
+#pragma unroll
+  for (int i = 0; i < 2 * NC; ++i) {
+    const int trow = 16 * (2 * NC * wave + i) + drow;     // feature index (< N)
+    const int chunk = (lane & 3) ^ swz4(trow);
+    w_src[i] = p.W + (int64_t)trow * p.K + 8 * chunk;
+  }
+  const half_t* a_src;
+  {
+    const int trow = 16 * (wave & 3) + drow;
+    const int chunk = (lane & 3) ^ swz4(trow);
+    a_src = p.A + (int64_t)min(m0 + trow, p.M - 1) * p.K + 8 * chunk;
+  }
+  auto issue = [&](int kt, lds_byte* wd, lds_byte* ad) {
+#pragma unroll
+    for (int i = 0; i < 2 * NC; ++i) dma16(w_src[i] + kt * kLK, wd + (2 * NC * wave + i) * 1024);
+    if (wave < 4) dma16(a_src + kt * kLK, ad + wave * 1024);
+  };
+  // fragment read: row (32*t + j32), chunk 2*ks + g of 4, row pitch 64 B
+  int rd[2];
+#pragma unroll
+  for (int ks = 0; ks < 2; ++ks) rd[ks] = j32 * 64 + (((2 * ks + g) ^ swz4(j32)) << 4);
+
+  floatx16 acc[NC][2];   // [feature tile ni][token tile mi]
+#pragma unroll
+  for (int i = 0; i < NC; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+  auto compute = [&](const lds_byte* wt, const lds_byte* at) {
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) {
+      half8_t xa[2];
+#pragma unroll
+      for (int mi = 0; mi < 2; ++mi) xa[mi] = lds_frag(at, (32 * mi) * 64 + rd[ks]);
+#pragma unroll
+      for (int ni = 0; ni < NC; ++ni) {
+        const half8_t wb = lds_frag(wt, (32 * NC * wave + 32 * ni) * 64 + rd[ks]);
+#pragma unroll
+        for (int mi = 0; mi < 2; ++mi) acc[ni][mi] = mfma32(wb, xa[mi], acc[ni][mi]);
+      }
+    }
+  };
+
+  const int nk = p.K / kLK;
+  issue(0, (lds_byte*)w_lds0, (lds_byte*)a_lds0);
+  for (int kt = 0; kt < nk; kt += 2) {
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+    __syncthreads();
+    if (kt + 1 < nk) issue(kt + 1, (lds_byte*)w_lds1, (lds_byte*)a_lds1);
+    compute((const lds_byte*)w_lds0, (const lds_byte*)a_lds0);
+    if (kt + 1 >= nk) break;
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+    __syncthreads();
+    if (kt + 2 < nk) issue(kt + 2, (lds_byte*)w_lds0, (lds_byte*)a_lds0);
+    compute((const lds_byte*)w_lds1, (const lds_byte*)a_lds1);
+  }
+
+  // ---- epilogue.  acc[ni][mi][r] = X[m0 + 32mi + j32][nb + 32ni + 8(r/4) + 4g + r%4],
+  // nb = 32*NC*wave.  Add bias and residual, then LayerNorm over the full row.
+  const int nb = 32 * NC * wave;
+  float psum[2] = {0.f, 0.f};
+#pragma unroll
+  for (int mi = 0; mi < 2; ++mi) {
+    const int m = min(m0 + 32 * mi + j32, p.M - 1);
+#pragma unroll
+    for (int ni = 0; ni < NC; ++ni)
+#pragma unroll
+      for (int q4 = 0; q4 < 4; ++q4) {
+        const int n = nb + 32 * ni + 8 * q4 + 4 * g;
+        half4_t bv = {(half_t)0.f, (half_t)0.f, (half_t)0.f, (half_t)0.f};
+        half4_t rv = bv;
+        if (p.bias) bv = *reinterpret_cast<const half4_t*>(p.bias + n);
+        if (p.res) rv = *reinterpret_cast<const half4_t*>(p.res + (int64_t)m * N + n);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const float x = acc[ni][mi][4 * q4 + e] + (float)bv[e] + (float)rv[e];
+          acc[ni][mi][4 * q4 + e] = x;
+          psum[mi] += x;
+        }
+      }
+    psum[mi] = pair_sum(psum[mi]);
+  }
+  if (g == 0) { red[0][wave][j32] = psum[0]; red[0][wave][32 + j32] = psum[1]; }
+  __syncthreads();
+  float mean[2], rstd[2];
+#pragma unroll
+  for (int mi = 0; mi < 2; ++mi) {
+    float s = 0.f;
+#pragma unroll
+    for (int w = 0; w < 8; ++w) s += red[0][w][32 * mi + j32];
+    mean[mi] = s * p.inv_n;
+  }
+  float pvar[2] = {0.f, 0.f};
+#pragma unroll
+  for (int mi = 0; mi < 2; ++mi) {
+#pragma unroll
+    for (int ni = 0; ni < NC; ++ni)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) { const float d = acc[ni][mi][r] - mean[mi]; pvar[mi] += d * d; }
+    pvar[mi] = pair_sum(pvar[mi]);
+  }
+  if (g == 0) { red[1][wave][j32] = pvar[0]; red[1][wave][32 + j32] = pvar[1]; }
+  __syncthreads();
+#pragma unroll
+  for (int mi = 0; mi < 2; ++mi) {
+    float s = 0.f;
+#pragma unroll
+    for (int w = 0; w < 8; ++w) s += red[1][w][32 * mi + j32];
+    rstd[mi] = 1.0f / sqrtf(s * p.inv_n + p.eps);
+  }
+#pragma unroll
+  for (int mi = 0; mi < 2; ++mi) {
+    const int m = m0 + 32 * mi + j32;
+    if (m >= p.M) continue;
+    half_t* crow = p.C + (int64_t)m * N;
+#pragma unroll
+    for (int ni = 0; ni < NC; ++ni)
+#pragma unroll
+      for (int q4 = 0; q4 < 4; ++q4) {
+        const int n = nb + 32 * ni + 8 * q4 + 4 * g;
+        half4_t gv = {(half_t)1.f, (half_t)1.f, (half_t)1.f, (half_t)1.f};
+        half4_t tv = {(half_t)0.f, (half_t)0.f, (half_t)0.f, (half_t)0.f};
+        if (p.gamma) gv = *reinterpret_cast<const half4_t*>(p.gamma + n);
+        if (p.beta) tv = *reinterpret_cast<const half4_t*>(p.beta + n);
+        half4_t o;
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          o[e] = (half_t)((acc[ni][mi][4 * q4 + e] - mean[mi]) * rstd[mi] * (float)gv[e] + (float)tv[e]);
+        *reinterpret_cast<half4_t*>(crow + n) = o;
+      }
+  }
+}
+
+}  // namespace
+
+extern "C" int stof_gemm_bias_act(const void* A, const void* Wt, const void* bias, void* C,
+                                  int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldc,
+                                  int act, void* stream) {
+  if (!A || !Wt || !C) return STOF_ERR_NULL_POINTER;
+  if (M <= 0 || N <= 0 || K <= 0 || K % kGK != 0 || N % 8 != 0 || lda < K || ldc < N) return STOF_ERR_BAD_SHAPE;
+  if (M > (1 << 30) || N > (1 << 30) || K > (1 << 30)) return STOF_ERR_BAD_SHAPE;
+  if (!stof_aligned16(A) || !stof_aligned16(Wt) || !stof_aligned16(C) || (bias && ((uintptr_t)bias & 7)) ||
+      lda % 8 != 0 || ldc % 4 != 0 || ((uintptr_t)C & 7))
+    return STOF_ERR_MISALIGNED;
+  GemmParams p;
+  p.A = (const half_t*)A; p.W = (const half_t*)Wt; p.bias = (const half_t*)bias; p.C = (half_t*)C;
+  p.M = (int)M; p.N = (int)N; p.K = (int)K; p.lda = (int)lda; p.ldc = (int)ldc;
+  p.tiles_m = (int)((M + kGT - 1) / kGT); p.tiles_n = (int)((N + kGT - 1) / kGT);
+  const dim3 grid((unsigned)(p.tiles_m * p.tiles_n)), block(256);
+  hipStream_t st = (hipStream_t)stream;
+  switch (act) {
+    case STOF_ACT_NONE: hipLaunchKernelGGL(gemm_bias_act_kernel<STOF_ACT_NONE>, grid, block, 0, st, p); break;
+    case STOF_ACT_GELU_ERF: hipLaunchKernelGGL(gemm_bias_act_kernel<STOF_ACT_GELU_ERF>, grid, block, 0, st, p); break;
+    case STOF_ACT_GELU_TANH: hipLaunchKernelGGL(gemm_bias_act_kernel<STOF_ACT_GELU_TANH>, grid, block, 0, st, p); break;
+    case STOF_ACT_RELU: hipLaunchKernelGGL(gemm_bias_act_kernel<STOF_ACT_RELU>, grid, block, 0, st, p); break;
+    default: return STOF_ERR_UNSUPPORTED;
+  }
+  return stof_check_launch();
+}
+
+extern "C" int stof_gemm_bias_res_ln(const void* A, const void* Wt, const void* bias, const void* residual,
+                                     const void* gamma, const void* beta, void* C,
+                                     int64_t M, int64_t N, int64_t K, float eps, void* stream) {
+  if (!A || !Wt || !C) return STOF_ERR_NULL_POINTER;
+  if (M <= 0 || K <= 0 || K % kLK != 0 || M > (1 << 30) || K > (1 << 30)) return STOF_ERR_BAD_SHAPE;
+  if (N != 256 && N != 512 && N != 768 && N != 1024) return STOF_ERR_UNSUPPORTED;
+  if (!stof_aligned16(A) || !stof_aligned16(Wt) || ((uintptr_t)C & 7) || ((uintptr_t)bias & 7) ||
+      ((uintptr_t)residual & 7) || ((uintptr_t)gamma & 7) || ((uintptr_t)beta & 7) || K % 8 != 0)
+    return STOF_ERR_MISALIGNED;
+  LnGemmParams p;
+  p.A = (const half_t*)A; p.W = (const half_t*)Wt; p.bias = (const half_t*)bias; p.res = (const half_t*)residual;
+  p.gamma = (const half_t*)gamma; p.beta = (const half_t*)beta; p.C = (half_t*)C;
+  p.M = (int)M; p.N = (int)N; p.K = (int)K; p.eps = eps; p.inv_n = 1.0f / (float)N;
+  const dim3 grid((unsigned)((M + kLM - 1) / kLM)), block(512);
+  hipStream_t st = (hipStream_t)stream;
+  switch (N) {
+    case 256: hipLaunchKernelGGL(gemm_bias_res_ln_kernel<1>, grid, block, 0, st, p); break;
+    case 512: hipLaunchKernelGGL(gemm_bias_res_ln_kernel<2>, grid, block, 0, st, p); break;
+    case 768: hipLaunchKernelGGL(gemm_bias_res_ln_kernel<3>, grid, block, 0, st, p); break;
+    default: hipLaunchKernelGGL(gemm_bias_res_ln_kernel<4>, grid, block, 0, st, p); break;
+  }
+  return stof_check_launch();
+}

@@ -45,8 +45,6 @@ def lib():
                 "(hipcc, gfx950). There is no fallback path.")
         h = ctypes.CDLL(LIB_PATH)
         for name, (res, args) in _SIGNATURES.items():
-            if not hasattr(h, name):   # TEMP until every entry point is implemented
-                continue
             fn = getattr(h, name)
             fn.restype = res
             fn.argtypes = args

@@ -1,0 +1,106 @@
+"""Post-LayerNorm encoder layer and stack on the fused HIP operators.
+
+The layer is the reference's ``bert_fwd_std`` (src/benchmk_end2end.py:31-88) with the QKV
+projection of src/model-candidate/1-BERT-large.py:17-18 in front, so that a stack of layers
+runs end to end on its own hidden state:
+
+    qkv  = x @ W_qkv + b_qkv                      GEMM + bias              -> [B,S,3D]
+    attn = block-masked MHA(q, k, v; LUT)          q/k/v read in place from qkv, result [B,S,D]
+    h    = LN(attn @ W_o + b_o + x; g1, be1)       GEMM + bias + residual + LayerNorm
+    f    = GELU(h @ W_1 + b_1)                     GEMM + bias + GELU
+    y    = LN(f @ W_2 + b_2 + h; g2, be2)          GEMM + bias + residual + LayerNorm
+
+Five launches per layer, no permute / contiguous copies, no standalone elementwise kernels.
+``ln_fusion`` selects how the two LayerNorm GEMMs run: "fused" = LayerNorm in the GEMM
+epilogue (one workgroup owns the full row), "split" = tiled GEMM followed by the
+bias+residual+LayerNorm kernel.  "auto" is a fixed rule on the shape (the reference likewise
+switches its fused GEMM+LN per shape, data/triton_perf.csv), not a run-time tuner.
+"""
+import torch
+
+from . import fused
+from .ops import block_attn
+
+
+class EncoderLayer:
+    def __init__(self, weights, n_heads, eps=1e-12, gelu="erf", ln_fusion="auto"):
+        """``weights``: dict with W_qkv [D,3D], b_qkv, W_o [D,D], b_o, g1, be1, W_1 [D,F], b_1,
+        W_2 [F,D], b_2, g2, be2 in the reference's [in, out] orientation, fp16 on the GPU."""
+        self.n_heads = n_heads
+        self.eps = eps
+        self.act = "gelu" if gelu == "erf" else "gelu_tanh"
+        self.ln_fusion = ln_fusion
+        w = weights
+        self.Wqkv = w["W_qkv"].t().contiguous(); self.bqkv = w["b_qkv"].contiguous()
+        self.Wo = w["W_o"].t().contiguous(); self.bo = w["b_o"].contiguous()
+        self.W1 = w["W_1"].t().contiguous(); self.b1 = w["b_1"].contiguous()
+        self.W2 = w["W_2"].t().contiguous(); self.b2 = w["b_2"].contiguous()
+        self.g1, self.be1 = w["g1"].contiguous(), w["be1"].contiguous()
+        self.g2, self.be2 = w["g2"].contiguous(), w["be2"].contiguous()
+        self.hidden = self.Wo.shape[0]
+
+    def _fuse(self, M):
+        if self.ln_fusion in ("fused", "split"):
+            return self.ln_fusion == "fused"
+        # One workgroup per 64 rows: below ~2 workgroups per CU the fused kernel cannot fill
+        # the 256 CUs, and at hidden 1024 its register budget is exhausted.
+        return self.hidden <= 768 and M >= 64 * 256
+
+    def _gemm_ln(self, x, Wt, bias, residual, gamma, beta):
+        M = x.numel() // x.shape[-1]
+        if self._fuse(M):
+            return fused.gemm_bias_residual_layernorm(x, Wt, bias, residual, gamma, beta, self.eps)
+        y = fused.gemm_bias_act(x, Wt, None, "none")
+        return fused.bias_residual_layernorm(y, bias, residual, gamma, beta, self.eps)
+
+    def forward(self, x, lut, block=64):
+        B, S, D = x.shape
+        H = self.n_heads
+        hd = D // H
+        qkv = fused.gemm_bias_act(x, self.Wqkv, self.bqkv, "none")           # [B,S,3D]
+        q, k, v = (qkv[..., t * D:(t + 1) * D].view(B, S, H, hd).permute(0, 2, 1, 3) for t in range(3))
+        attn = block_attn(q, k, v, lut, block, block, out_layout="bshd")      # [B,S,D]
+        h = self._gemm_ln(attn, self.Wo, self.bo, x, self.g1, self.be1)
+        f = fused.gemm_bias_act(h, self.W1, self.b1, self.act)
+        return self._gemm_ln(f, self.W2, self.b2, h, self.g2, self.be2)
+
+    __call__ = forward
+
+
+class EncoderStack:
+    """``layers`` independent EncoderLayers applied in sequence (24 for the BERT-large /
+    GPT-2-medium style stack)."""
+
+    def __init__(self, layer_weights, n_heads, eps=1e-12, gelu="erf", ln_fusion="auto"):
+        self.layers = [EncoderLayer(w, n_heads, eps, gelu, ln_fusion) for w in layer_weights]
+
+    def forward(self, x, lut, block=64):
+        for layer in self.layers:
+            x = layer(x, lut, block)
+        return x
+
+    __call__ = forward
+
+
+def eager_layer(x, w, mask, n_heads, eps=1e-12):
+    """The same layer in plain PyTorch ops on x's device (matmul, add, softmax, F.gelu,
+    F.layer_norm, permute + contiguous exactly as src/benchmk_end2end.py:31-88): the unfused
+    comparator the fused layer is timed against.  ``mask`` [B,S,S] or [1,S,S] of 0/1."""
+    import torch.nn.functional as F
+    B, S, D = x.shape
+    hd = D // n_heads
+    qkv = torch.matmul(x, w["W_qkv"]) + w["b_qkv"]
+    q, k, v = qkv.chunk(3, dim=-1)
+    tr = lambda t: t.view(B, S, n_heads, hd).permute(0, 2, 1, 3)
+    q, k, v = tr(q), tr(k), tr(v)
+    scores = torch.matmul(q, k.transpose(-2, -1)) / (hd ** .5)
+    scores -= 10000.0 * (1.0 - mask.unsqueeze(1))
+    probs = F.softmax(scores, dim=-1)
+    h = torch.matmul(probs, v)
+    h = h.permute(0, 2, 1, 3).contiguous().view(B, S, D)
+    h = torch.matmul(h, w["W_o"]) + w["b_o"]
+    h = F.layer_norm(h + x, (D,), weight=w["g1"], bias=w["be1"], eps=eps)
+    r = h
+    h = F.gelu(torch.matmul(h, w["W_1"]) + w["b_1"])
+    h = torch.matmul(h, w["W_2"]) + w["b_2"]
+    return F.layer_norm(h + r, (D,), weight=w["g2"], bias=w["be2"], eps=eps)

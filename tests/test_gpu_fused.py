@@ -1,0 +1,143 @@
+"""GPU parity of the fused encoder operators, the row-wise attention front-ends and the
+encoder layer against the CPU oracle.  Tolerance: |got - want| <= 2e-3 + 1e-2 * |want|
+(fp16 kernels, fp32 accumulation, vs the fp32 oracle on the same fp16-rounded inputs)."""
+import pytest
+import torch
+
+from oracle import attention as oa
+from oracle import encoder as oe
+from stof import configs, fused, masks as pm
+from stof.layer import EncoderLayer, EncoderStack
+from stof.ops import (rowwise_attn_full_op, rowwise_attn_sliding_op, rowwise_attn_mask_op, StofError)
+
+pytestmark = pytest.mark.gpu
+
+
+def _close(got, want, what="", atol=2e-3, rtol=1e-2):
+    got = got.float().cpu(); want = want.float().cpu()
+    assert got.shape == want.shape, f"{what}: shape {tuple(got.shape)} vs {tuple(want.shape)}"
+    err = (got - want).abs()
+    bad = err > atol + rtol * want.abs()
+    assert not bool(bad.any()), f"{what}: {int(bad.sum())} out of tolerance, max abs err {float(err.max()):.3e}"
+
+
+def _rand(*shape, seed=0, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(*shape, generator=g) * scale).half()
+
+
+# ---- GEMM + bias + activation -----------------------------------------------------------------
+
+@pytest.mark.parametrize("M,N,K", [(8192, 3072, 768), (300, 768, 3072), (64, 2304, 768), (1, 8, 64), (129, 136, 128)])
+@pytest.mark.parametrize("act", ["none", "gelu", "gelu_tanh", "relu"])
+def test_gemm_bias_act(M, N, K, act):
+    print(f"gemm M{M} N{N} K{K} {act}", flush=True)
+    x = _rand(M, K, seed=1); W = _rand(K, N, seed=2, scale=0.05); b = _rand(N, seed=3, scale=0.5)
+    got = fused.gemm_bias_act(x.cuda(), fused.pack_weight(W.cuda()), b.cuda(), act)
+    _close(got, oe.gemm_bias_act(x, W, b, act), f"gemm {act}")
+
+
+def test_gemm_strided_rows_and_no_bias():
+    x = _rand(100, 256, seed=4)
+    xs = x.cuda()[:, :128]                       # row pitch 256, K = 128
+    W = _rand(128, 72, seed=5, scale=0.1)
+    got = fused.gemm_bias_act(xs, fused.pack_weight(W.cuda()), None, "none")
+    _close(got, x[:, :128].float() @ W.float(), "strided")
+    ident = torch.eye(64).half()                  # closed form: W = I returns the input
+    _close(fused.gemm_bias_act(x.cuda()[:, :64].contiguous(), ident.cuda(), None, "none"), x[:, :64], "identity")
+
+
+# ---- GEMM + bias + residual + LayerNorm -------------------------------------------------------
+
+@pytest.mark.parametrize("M,N,K", [(8192, 768, 768), (2048, 768, 3072), (1000, 1024, 1024), (64, 512, 128), (7, 256, 32)])
+@pytest.mark.parametrize("eps", [1e-5, 1e-12])
+def test_gemm_bias_residual_layernorm(M, N, K, eps):
+    print(f"gemm_ln M{M} N{N} K{K}", flush=True)
+    x = _rand(M, K, seed=6); W = _rand(K, N, seed=7, scale=0.05); b = _rand(N, seed=8, scale=0.5)
+    r = _rand(M, N, seed=9); gm = (1 + 0.1 * _rand(N, seed=10).float()).half(); bt = _rand(N, seed=11, scale=0.1)
+    got = fused.gemm_bias_residual_layernorm(x.cuda(), fused.pack_weight(W.cuda()), b.cuda(), r.cuda(),
+                                             gm.cuda(), bt.cuda(), eps)
+    _close(got, oe.gemm_bias_residual_layernorm(x, W, b, r, gm, bt, eps), "gemm_ln")
+
+
+def test_reference_named_fused_ops():
+    Bn, M, K, N = 4, 192, 768, 768
+    A = _rand(Bn, M, K, seed=12); W = _rand(K, N, seed=13, scale=0.05); bias = _rand(N, seed=14, scale=0.5)
+    Wexp = W.cuda().unsqueeze(0).expand(Bn, -1, -1)
+    got = fused.triton_matmul_bias_layernorm(A.cuda(), Wexp, bias.cuda())
+    _close(got, oe.matmul_bias_layernorm(A, W.unsqueeze(0).expand(Bn, -1, -1), bias), "matmul_bias_ln [N] bias")
+    mean = got.float().mean(-1); var = got.float().var(-1, unbiased=False)
+    assert float(mean.abs().max()) < 2e-3 and float((var - 1).abs().max()) < 1e-2     # no affine: mean 0, var 1
+    res = _rand(Bn, M, N, seed=15)
+    got = fused.triton_matmul_bias_layernorm(A.cuda(), Wexp, (bias + res).cuda())     # the call-site form
+    _close(got, oe.matmul_bias_layernorm(A, W.unsqueeze(0).expand(Bn, -1, -1), bias + res), "matmul_bias_ln bias+residual")
+    a = _rand(2, 128, 256, seed=16); b = _rand(256, 1024, seed=17, scale=0.05); d = _rand(1024, 256, seed=18, scale=0.05)
+    bb = _rand(1024, seed=19, scale=0.5)
+    got = fused.triton_matmul_batch(a.cuda(), b.cuda(), d.cuda(), bb.cuda())
+    _close(got, oe.matmul_gelu_matmul(a, b, d, bb), "matmul_batch", atol=4e-3)
+
+
+def test_fused_op_errors():
+    x = _rand(64, 96, seed=20).cuda(); W = _rand(72, 96, seed=21).cuda()
+    with pytest.raises(StofError):
+        fused.gemm_bias_act(x, W, None, "none")                                    # K % 64 != 0
+    with pytest.raises(StofError):
+        fused.gemm_bias_residual_layernorm(_rand(64, 128).cuda(), _rand(384, 128).cuda(), None, None, None, None)  # N = 384
+    with pytest.raises(StofError):
+        fused.gemm_bias_act(x.float(), W, None, "none")
+
+
+# ---- row-wise attention front-ends ---------------------------------------------------------------
+
+@pytest.mark.parametrize("B,H,S", [(2, 12, 256), (1, 3, 128), (1, 12, 576)])
+def test_rowwise_ops(B, H, S):
+    cfg = configs.AttnConfig("t", B, H, S)
+    q, k, v = configs.qkv(cfg, seed=22, device="cuda")
+    qc, kc, vc = q.cpu().float(), k.cpu().float(), v.cpu().float()
+    for causal in (False, True):
+        got = rowwise_attn_full_op(q, k, v, causal)
+        assert got.shape == (B, S, H * 64)
+        _close(got, oa.rowwise_attn_full(qc, kc, vc, causal), f"full causal={causal}")
+    for causal, band in ((True, 32), (True, 100), (False, 7), (True, 1)):
+        _close(rowwise_attn_sliding_op(q, k, v, causal, band), oa.rowwise_attn_sliding(qc, kc, vc, causal, band),
+               f"sliding causal={causal} band={band}")
+    g = torch.Generator().manual_seed(23)
+    rm = (torch.rand(S, S, generator=g) < 0.3).half()
+    rm[:, :64] = 0; rm[5, :] = 0; rm[:, 70] = 1; rm[5, 70] = 0      # an empty tile column, a dead row
+    for causal in (False, True):
+        _close(rowwise_attn_mask_op(q, k, v, causal, rm.cuda()), oa.rowwise_attn_mask(qc, kc, vc, causal, rm),
+               f"mask causal={causal}")
+    long = configs.mask_c1(S).half()
+    _close(rowwise_attn_mask_op(q, k, v, False, long.cuda()), oa.rowwise_attn_mask(qc, kc, vc, False, long), "mask C1")
+
+
+# ---- encoder layer -----------------------------------------------------------------------------
+
+@pytest.mark.parametrize("fusion", ["fused", "split"])
+def test_encoder_layer_c3_reduced_batch(fusion):
+    """BERT-base layer (hidden 768, 12 heads, FFN 3072, eps 1e-12) at batch 4, per-sample
+    padding x sliding-window mask, against the fp32 oracle of the same layer."""
+    B, S, D, H, F = 4, 512, 768, 12, 3072
+    w = configs.layer_weights(D, F, seed=0)
+    x = configs.layer_input(configs.LayerConfig("t", B, S, D, H, F, 1), seed=1)
+    mask, L = configs.mask_c3(batch=B, s=S, window=256, seed=0)
+    lut = pm.get_sparse_storage_batched(mask.float().cuda(), 64, 64)[1:]
+    layer = EncoderLayer({k: v.cuda() for k, v in w.items()}, H, eps=1e-12, ln_fusion=fusion)
+    got = layer(x.cuda(), lut)
+    want = oe.bert_layer(x, w, mask.float(), H, eps=1e-12)
+    valid = torch.arange(S)[None, :] < L[:, None]          # rows past the sample length are don't-care
+    _close(got.cpu()[valid], want[valid], f"layer {fusion}", atol=4e-3)
+
+
+def test_encoder_stack_two_layers_c5_shape_reduced():
+    B, S, D, H, F = 1, 512, 1024, 16, 4096
+    ws = [configs.layer_weights(D, F, seed=s) for s in (0, 1)]
+    x = configs.layer_input(configs.LayerConfig("t", B, S, D, H, F, 2), seed=2)
+    mask = configs.mask_c5(S)[None]
+    lut = pm.get_sparse_storage(mask.float().cuda(), 64, 64)[1:]
+    stack = EncoderStack([{k: v.cuda() for k, v in w.items()} for w in ws], H, eps=1e-12)
+    got = stack(x.cuda(), lut)
+    want = x
+    for w in ws:
+        want = oe.bert_layer(want, w, mask.float(), H, eps=1e-12)
+    _close(got, want, "stack", atol=6e-3)
