@@ -1,0 +1,196 @@
+#!/usr/bin/env python3
+"""Benchmark of the STOF hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-extras] [--no-cpu]
+
+One "step" is one launch of block-masked multi-head attention on workload C2 (fp16,
+B8 H12 S1024 D64, banded + global + random key blocks, 129 active 64x64 blocks), inputs
+resident in HBM.  The timed region is K steps between device synchronisations; the same
+region is bracketed by HIP events on the launch stream for the per-launch kernel time that
+the roofline figure uses.  One JSON line is printed:
+
+  value        TFLOP/s counted on ACTIVE blocks only (4*64*64*64 FLOP per block, per batch
+               and head: QK^T and PV), whole job, wall clock
+  roofline     the attention kernel against the MI355X dense fp16 MFMA peak (2.5 PFLOP/s)
+  cpu_baseline the reference's PyTorch-native dense attention (restated in oracle/) timed on
+               this machine's host cores on the same workload, in the same unit
+  also         the other single-GPU workloads: C4 (S4096 long-sequence MHA), the C3 BERT-base
+               encoder layer (fused vs PyTorch-ROCm eager, ms) and the HBM-bound kernels
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "sc25-stof-ad_amd"))
+
+import torch  # noqa: E402
+
+PEAK_FP16_TFLOPS = 2500.0     # MI355X dense fp16 matrix peak (published)
+PEAK_HBM_GBS = 8000.0         # MI355X HBM3E peak (published)
+FLOP_PER_BLOCK = 4 * 64 * 64 * 64
+
+# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (two runs),
+# scaled by the same counters on a torch copy kernel of known size; see profiles/.
+MEASURED_TRAFFIC_BYTES = {"C2": None}
+
+
+def attn_setup(cfg, mask_fn, device):
+    from stof import configs, masks as pm
+    mask = mask_fn(cfg.seq)
+    q, k, v = configs.qkv(cfg, seed=0, device=device)
+    lut = pm.get_sparse_storage(mask.float()[None].to(device), 64, 64)[1:]
+    n_active = int(lut[5][-1])
+    return q, k, v, lut, n_active, mask
+
+
+def time_region(fn, steps, warmup):
+    """(wall ms per step, event ms per step) for `steps` calls after `warmup` untimed ones."""
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    e0 = torch.cuda.Event(enable_timing=True)
+    e1 = torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(steps):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    return (t1 - t0) * 1e3 / steps, e0.elapsed_time(e1) / steps
+
+
+def bench_attn(cfg, mask_fn, steps, warmup):
+    from stof.ops import block_attn
+    q, k, v, lut, n_active, _ = attn_setup(cfg, mask_fn, "cuda")
+    out = torch.empty_like(q)
+    block_attn(q, k, v, lut, out=out)          # packs the partial-block bit masks once
+    wall_ms, ev_ms = time_region(lambda: block_attn(q, k, v, lut, out=out), steps, warmup)
+    flop = FLOP_PER_BLOCK * cfg.batch * cfg.heads * n_active
+    return {"wall_ms": wall_ms, "kernel_ms": ev_ms, "flop": flop, "active_blocks": n_active,
+            "tflops_wall": flop / wall_ms / 1e9, "tflops_kernel": flop / ev_ms / 1e9}
+
+
+def cpu_baseline_attn(cfg, mask_fn, n_active, budget_s=12.0, max_iters=20):
+    """The reference's dense PyTorch attention (oracle.attention.torch_attn_std) in fp32 on the
+    host cores; bounded sample of whole-workload iterations."""
+    from oracle import attention as oa
+    from stof import configs
+    cores = os.cpu_count() or 1
+    if os.environ.get("OMP_NUM_THREADS"):
+        cores = min(cores, int(os.environ["OMP_NUM_THREADS"]))
+    torch.set_num_threads(cores)
+    q, k, v = configs.qkv(cfg, seed=0, dtype=torch.float32, device="cpu")
+    mask = mask_fn(cfg.seq).float()[None]
+    oa.torch_attn_std(q, k, v, mask)           # warm-up
+    iters, t0 = 0, time.perf_counter()
+    while iters < max_iters and (time.perf_counter() - t0) < budget_s:
+        oa.torch_attn_std(q, k, v, mask)
+        iters += 1
+    dt = (time.perf_counter() - t0) / iters
+    flop = FLOP_PER_BLOCK * cfg.batch * cfg.heads * n_active
+    return {"value": flop / dt / 1e12, "unit": "TFLOP/s", "cores": cores, "kind": "port",
+            "ms_per_step": dt * 1e3,
+            "sample": f"{iters} full passes of the {cfg.name} workload (dense fp32 softmax(QK^T/8 - 10000(1-M))V, "
+                      f"B{cfg.batch} H{cfg.heads} S{cfg.seq} D64), active-block FLOPs / time"}
+
+
+def bench_layer_c3(steps, warmup):
+    """BERT-base encoder layer, B16 S512: fused HIP layer vs PyTorch-ROCm eager."""
+    from stof import configs, masks as pm
+    from stof.layer import EncoderLayer, eager_layer
+    cfg = configs.C3
+    w = {k: v.cuda() for k, v in configs.layer_weights(cfg.hidden, cfg.ffn, seed=0).items()}
+    x = configs.layer_input(cfg, seed=1, device="cuda")
+    mask, _ = configs.mask_c3(cfg.batch, cfg.seq, 256, seed=0)
+    maskg = mask.cuda().half()
+    lut = pm.get_sparse_storage_batched(mask.float().cuda(), 64, 64)[1:]
+    out = {}
+    for fusion in ("fused", "split"):
+        layer = EncoderLayer(w, cfg.heads, eps=cfg.eps, ln_fusion=fusion)
+        layer(x, lut)
+        out[fusion + "_ms"], _ = time_region(lambda: layer(x, lut), steps, warmup)
+    with torch.no_grad():
+        out["eager_ms"], _ = time_region(lambda: eager_layer(x, w, maskg, cfg.heads, cfg.eps), max(steps // 4, 5), 5)
+    best = min(out["fused_ms"], out["split_ms"])
+    out["layer_ms"] = best
+    out["speedup_vs_eager"] = out["eager_ms"] / best
+    flop = 2 * cfg.batch * cfg.seq * cfg.hidden * (3 * cfg.hidden + cfg.hidden + 2 * cfg.ffn)
+    out["gemm_tflops_at_layer_ms"] = flop / best / 1e9
+    return out
+
+
+def bench_hbm_kernels(steps, warmup):
+    from stof import fused
+    from stof.ops import pack_mask_bits
+    M, N = 8192, 768
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(M, N, generator=g).half().cuda(); r = torch.randn(M, N, generator=g).half().cuda()
+    b = torch.randn(N, generator=g).half().cuda()
+    _, ev = time_region(lambda: fused.bias_residual_layernorm(x, b, r, b, b, 1e-12), steps, warmup)
+    ln_bytes = 3 * M * N * 2
+    S = 4096
+    m = (torch.rand(S, S, generator=g) < 0.5).half().cuda()
+    _, ev2 = time_region(lambda: pack_mask_bits(m, additive=False), steps, warmup)
+    pk_bytes = S * S * 2 + S * S // 8
+    return {"bias_res_ln": {"ms": ev, "GBs": ln_bytes / ev / 1e6, "frac_hbm": ln_bytes / ev / 1e6 / PEAK_HBM_GBS,
+                            "shape": [M, N]},
+            "pack_mask_bits": {"ms": ev2, "GBs": pk_bytes / ev2 / 1e6, "frac_hbm": pk_bytes / ev2 / 1e6 / PEAK_HBM_GBS,
+                               "shape": [S, S]}}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--no-extras", action="store_true", help="skip C4 / C3 layer / HBM-bound kernels")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU only (the hot path shards by batch x head with no "
+              "exchange step; nothing here uses a second device). Run with --gpus 1.", file=sys.stderr)
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible; the HIP path has no CPU fallback.", file=sys.stderr)
+        sys.exit(2)
+
+    from stof import configs
+    torch.cuda.set_device(0)
+    c2 = bench_attn(configs.C2, configs.mask_c2, args.steps, args.warmup)
+    line = {
+        "metric": "masked-MHA TFLOP/s (active blocks) + encoder-layer ms, fp16, 1xMI355X",
+        "value": c2["tflops_wall"], "unit": "TFLOP/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": c2["wall_ms"],
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f16", "data": "synthetic",
+        "config": {"workload": "C2: block-masked MHA, B8 H12 S1024 D64, band 3 + 2 global + 3 random key blocks "
+                               "per 64-row query block", "active_blocks": c2["active_blocks"], "block": 64,
+                   "flop_per_step": c2["flop"]},
+        "roofline": {"bound": "mfma", "achieved": c2["tflops_kernel"], "peak": PEAK_FP16_TFLOPS, "unit": "TFLOP/s",
+                     "frac": c2["tflops_kernel"] / PEAK_FP16_TFLOPS, "traffic": MEASURED_TRAFFIC_BYTES["C2"],
+                     "kernel": "block_attn_fwd_kernel", "kernel_ms": c2["kernel_ms"]},
+    }
+    if not args.no_cpu:
+        line["cpu_baseline"] = cpu_baseline_attn(configs.C2, configs.mask_c2, c2["active_blocks"])
+    if not args.no_extras:
+        also = {}
+        c4 = bench_attn(configs.C4, configs.mask_c4, args.steps, args.warmup)
+        also["C4_mha_S4096"] = {"tflops": c4["tflops_kernel"], "frac_mfma_peak": c4["tflops_kernel"] / PEAK_FP16_TFLOPS,
+                                "kernel_ms": c4["kernel_ms"], "active_blocks": c4["active_blocks"]}
+        big = configs.AttnConfig("C4x8", 16, 16, 4096)
+        c4b = bench_attn(big, configs.mask_c4, max(args.steps // 4, 10), 5)
+        also["C4_mask_B16_H16"] = {"tflops": c4b["tflops_kernel"], "frac_mfma_peak": c4b["tflops_kernel"] / PEAK_FP16_TFLOPS,
+                                   "kernel_ms": c4b["kernel_ms"]}
+        also["C3_bert_base_layer"] = bench_layer_c3(max(args.steps // 4, 20), 10)
+        also["hbm_bound"] = bench_hbm_kernels(args.steps, args.warmup)
+        line["also"] = also
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

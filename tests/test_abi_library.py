@@ -1,0 +1,87 @@
+"""The C-ABI shared library loads and exports every symbol include/stof_abi.h declares, and
+its host-side argument checks reject bad calls before any launch (no GPU needed: every call
+here fails validation and returns a negative status)."""
+import ctypes
+import os
+import re
+
+import pytest
+
+from stof import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "stof_abi.h")
+
+
+def _declared_symbols():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(stof_[a-z0-9_]+)\s*\(", text)))
+
+
+@pytest.fixture(scope="module")
+def lib():
+    if not os.path.exists(_lib.LIB_PATH):
+        pytest.skip("libstof_hip.so not built (python sc25-stof-ad_amd/csrc/build.py)")
+    return _lib.lib()
+
+
+def test_every_declared_symbol_is_exported_and_bound(lib):
+    syms = _declared_symbols()
+    assert len(syms) >= 8
+    raw = ctypes.CDLL(_lib.LIB_PATH)
+    for s in syms:
+        assert hasattr(raw, s), f"{s} declared in stof_abi.h but not exported"
+        assert s in _lib._SIGNATURES, f"{s} has no ctypes signature"
+    assert sorted(_lib._SIGNATURES) == syms
+
+
+def test_version_and_status_strings(lib):
+    assert lib.stof_abi_version() == 1
+    for code in (0, -1, -2, -3, -4, -5, -6, -99):
+        assert len(lib.stof_status_string(code)) > 0
+
+
+def _s3(a, b, c):
+    return (ctypes.c_int64 * 3)(a, b, c)
+
+
+def test_block_attn_argument_checks(lib):
+    st = _s3(12 * 128 * 64, 128 * 64, 64)
+    P = 4096   # fake, 16-byte aligned, never dereferenced: validation fails first
+    call = lambda **kw: lib.stof_block_attn_fwd(
+        kw.get("q", P), P, P, P, P, P, P, P, P, P, P, kw.get("bm", 64), kw.get("bn", 64), 0.125,
+        kw.get("qs", st), st, st, st, 1, kw.get("S", 128), 12, kw.get("D", 64), kw.get("lbs", 0), None)
+    assert call(q=None) == -1            # NULL pointer
+    assert call(S=100) == -2             # seq_len not a multiple of 64
+    assert call(S=0) == -2
+    assert call(D=128) == -3             # head size
+    assert call(bm=32, bn=32) == -3      # block size
+    assert call(q=P + 2) == -4           # misaligned pointer
+    assert call(qs=_s3(12 * 128 * 64, 128 * 64, 65)) == -4   # stride not a multiple of 8
+    assert call(lbs=2) == -6             # per-sample LUT stride too small
+
+
+def test_other_entry_points_argument_checks(lib):
+    P = 4096
+    assert lib.stof_pack_mask_bits(None, P, 64, 64, 64, 1, None) == -1
+    assert lib.stof_pack_mask_bits(P, P, 64, 100, 100, 1, None) == -2
+    assert lib.stof_bias_res_ln(P, None, None, None, None, P, None, None, 10, 12, 1e-5, None) == -2   # N % 8
+    assert lib.stof_bias_res_ln(P, None, None, None, None, P, None, None, 10, 16384, 1e-5, None) == -2
+    assert lib.stof_bias_res_ln(None, None, None, None, None, P, None, None, 10, 64, 1e-5, None) == -1
+    assert lib.stof_gemm_bias_act(P, P, None, P, 64, 64, 96, 96, 64, 0, None) == -2      # K % 64
+    assert lib.stof_gemm_bias_act(P, P, None, P, 64, 64, 64, 64, 64, 9, None) == -3      # activation
+    assert lib.stof_gemm_bias_act(P, P + 8, None, P, 64, 64, 64, 64, 64, 0, None) == -4
+    assert lib.stof_gemm_bias_res_ln(P, P, None, None, None, None, P, 64, 384, 64, 1e-5, None) == -3   # N
+    assert lib.stof_gemm_bias_res_ln(P, P, None, None, None, None, P, 64, 768, 48, 1e-5, None) == -2   # K % 32
+    assert lib.stof_rowwise_attn_fwd(P, P, P, P, 7, 0, 0, None, 1, 128, 12, 64, None) == -3
+    assert lib.stof_rowwise_attn_fwd(P, P, P, P, 2, 0, 0, None, 1, 128, 12, 64, None) == -1            # mask kind, no bits
+    assert lib.stof_rowwise_attn_fwd(P, P, P, P, 1, 1, 0, None, 1, 128, 12, 64, None) == -2            # band <= 0
+    assert lib.stof_rowwise_attn_fwd(P, P, P, P, 0, 0, 0, None, 1, 130, 12, 64, None) == -2
+
+
+def test_missing_library_fails_loudly(monkeypatch, tmp_path):
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "nope.so"))
+    with pytest.raises(_lib.StofError):
+        _lib.lib()
