@@ -150,6 +150,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-extras", action="store_true", help="skip C4 / C3 layer / HBM-bound kernels")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="also run one plain device copy of 256 MiB, so that a counter run of this "
+                         "command holds a kernel of known traffic to scale FETCH_SIZE / WRITE_SIZE by")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (the hot path shards by batch x head with no "
@@ -161,6 +164,11 @@ def main():
 
     from stof import configs
     torch.cuda.set_device(0)
+    if args.copy_probe:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device="cuda").fill_(1)
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
     c2 = bench_attn(configs.C2, configs.mask_c2, args.steps, args.warmup)
     line = {
         "metric": "masked-MHA TFLOP/s (active blocks) + encoder-layer ms, fp16, 1xMI355X",
