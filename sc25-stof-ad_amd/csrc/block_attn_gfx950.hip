@@ -127,7 +127,12 @@ __global__ __launch_bounds__(256) void block_attn_fwd_kernel(const AttnParams p)
   const int vid = (wg & 7) * p.chunk + (wg >> 3);
   if (vid >= p.total) return;
   const int bh = vid / p.nP;
-  const int pair = p.nP - 1 - (vid - bh * p.nP);   // late (long, for causal-like masks) rows first
+  // Row length usually grows (causal) or is flat along the sequence.  Workgroups are placed
+  // on CUs round-robin, so consecutive heads walk the sequence in opposite directions: a CU
+  // that receives the longest rows of one head receives the shortest rows of the next.
+  const int pidx = vid - bh * p.nP;
+  const int zig = ((pidx + bh) & 1) ? (pidx >> 1) : p.nP - 1 - (pidx >> 1);   // long, short, long, ...
+  const int pair = zig;
   const int b = bh / p.H;
   const int h = bh - b * p.H;
   const int qi = 2 * pair + rsel;                  // this wave's query block
