@@ -82,30 +82,19 @@ __device__ __forceinline__ float pair_sum(float x) {
 // c ^ swz(r).  swz is a bijection of row bits (1,2,3) onto chunk bits (2,0,1).
 __device__ __forceinline__ int swz(int row) { return (((row >> 1) & 1) << 2) | ((row >> 2) & 3); }
 
-// One LUT row (the key blocks of one 64-row query block) held in registers, 64 entries at
-// a time: lane i holds entry base+i.  `slot` is the bitmask slot of a partial entry, -1
-// for a full one.  LOAD is the union of FULL and PART (get_sparse_storage builds it so),
-// hence an entry is partial iff its key block is in the row's PART list.
-struct LutRow {
-  int t0, n, p0, np;      // first LOAD entry, entry count, first PART entry, PART count
-  int base;               // index of the entry held by lane 0
-  int col, slot;          // per lane
-  __device__ __forceinline__ void fill(const AttnParams& p, int lane, bool want_slots) {
-    col = 0x7fffffff; slot = -1;
-    if (base + lane < n) col = p.lci[t0 + base + lane];
-    if (!want_slots) return;
-    for (int pb = 0; pb < np; pb += 64) {
-      const int here = min(64, np - pb);
-      int pc = -1;
-      if (lane < here) pc = p.pci[p0 + pb + lane];
-      for (int j = 0; j < here; ++j)
-        if (col == __builtin_amdgcn_readlane(pc, j)) slot = p0 + pb + j;
-    }
-  }
+// Extents of one LUT row (the key blocks of one 64-row query block).  LOAD is the union of
+// FULL and PART with ascending key-block indices (get_sparse_storage builds it so), hence an
+// entry is partial iff its key block is in the row's PART list, and the PART slot of a block
+// is its rank in that list.
+struct RowList {
+  int t0, n, p0, np;   // KIND LUT: first LOAD entry, LOAD count, first PART entry, PART count
+  int ptr, pptr;       // LOAD / PART entries already handed out to earlier 64-column windows
+  int lo, hi;          // KIND != LUT: the contiguous key-block range [lo, hi]
 };
 
-template <int KIND>
-__global__ __launch_bounds__(256) void block_attn_fwd_kernel(const AttnParams p) {
+template <int KIND, int ROWS>
+__global__ __launch_bounds__(128 * ROWS) void block_attn_fwd_kernel(const AttnParams p) {
+  constexpr int kDma = 4 / ROWS;   // direct-to-LDS instructions per wave and operand tile (8 over 2*ROWS waves)
   // Four distinct LDS objects (K and V, two buffers each): the compiler orders LDS reads
   // after in-flight direct-to-LDS loads per object, so a read of the current buffer does
   // not wait for the loads that fill the other one.
@@ -135,8 +124,8 @@ __global__ __launch_bounds__(256) void block_attn_fwd_kernel(const AttnParams p)
   const int pair = zig;
   const int b = bh / p.H;
   const int h = bh - b * p.H;
-  const int qi = 2 * pair + rsel;                  // this wave's query block
-  const bool q_valid = qi < p.nQ;                  // odd block count: the last pair has one row
+  const int qi = ROWS * pair + rsel;               // this wave's query block
+  const bool q_valid = qi < p.nQ;                  // block count not a multiple of ROWS: the last group is short
 
   const int64_t qrow0 = (int64_t)qi * kBM + 32 * half;
   const half_t* qb = p.q + b * p.qs[0] + h * p.qs[1] + qrow0 * p.qs[2];
@@ -144,16 +133,14 @@ __global__ __launch_bounds__(256) void block_attn_fwd_kernel(const AttnParams p)
   const half_t* vb = p.v + b * p.vs[0] + h * p.vs[1];
   half_t* ob = p.out + b * p.os[0] + h * p.os[1] + qrow0 * p.os[2];
 
-  // ---- both rows of the pair; every wave walks the same merged sequence of key blocks
+  // ---- the ROWS rows of the group; every wave walks the same merged sequence of key blocks
   const int64_t lo = (int64_t)b * p.lut_bs;
-  LutRow row[2];
-  int row_lo[2] = {0, 0};   // KIND != 0: first key block of each row's contiguous range
+  RowList row[ROWS];
 #pragma unroll
-  for (int r = 0; r < 2; ++r) {
-    const int qr = 2 * pair + r;
-    row[r].base = 0;
-    row[r].t0 = row[r].n = row[r].p0 = row[r].np = 0;
-    row[r].col = 0; row[r].slot = -1;
+  for (int r = 0; r < ROWS; ++r) {
+    const int qr = ROWS * pair + r;
+    row[r].t0 = row[r].n = row[r].p0 = row[r].np = row[r].ptr = row[r].pptr = 0;
+    row[r].lo = 0; row[r].hi = -1;
     if (qr < p.nQ) {
       if (KIND == kKindLut) {
         row[r].t0 = __builtin_amdgcn_readfirstlane(p.lrp[lo + qr]);
@@ -163,13 +150,11 @@ __global__ __launch_bounds__(256) void block_attn_fwd_kernel(const AttnParams p)
       } else {
         // keys allowed for some query of block qr: (64qr - band, 64qr + 63] when sliding,
         // up to the diagonal block when causal, else every block
-        const int hi = p.causal ? qr : p.nQ - 1;
+        row[r].hi = p.causal ? qr : p.nQ - 1;
         const int first_key = (KIND == kKindPred && p.band > 0) ? 64 * qr - p.band + 1 : 0;
-        row_lo[r] = first_key > 0 ? first_key / 64 : 0;
-        row[r].n = hi - row_lo[r] + 1 > 0 ? hi - row_lo[r] + 1 : 0;
+        row[r].lo = first_key > 0 ? first_key / 64 : 0;
       }
     }
-    if (KIND == kKindLut) row[r].fill(p, lane, true);
   }
 
   // Q^T as the B operand: lane (n = query j32, k-group g) holds 8 consecutive d per k-step.
@@ -184,12 +169,12 @@ __global__ __launch_bounds__(256) void block_attn_fwd_kernel(const AttnParams p)
 
   // ---- per-lane constants of the data movement
   // DMA: a tile is 8 instructions of 1 KB (8 rows of 128 B); wave w issues instructions
-  // 2w and 2w+1 for K and for V.  Lane l lands at (row 8*ii + l/8, chunk position l%8) and
-  // therefore fetches global chunk (l%8) ^ swz(row).
-  int k_src[2], v_src[2];
+  // kDma*w .. kDma*w + kDma - 1 for K and for V.  Lane l lands at (row 8*ii + l/8, chunk
+  // position l%8) and therefore fetches global chunk (l%8) ^ swz(row).
+  int k_src[kDma], v_src[kDma];
 #pragma unroll
-  for (int i = 0; i < 2; ++i) {
-    const int trow = 8 * (2 * wave + i) + (lane >> 3);
+  for (int i = 0; i < kDma; ++i) {
+    const int trow = 8 * (kDma * wave + i) + (lane >> 3);
     const int chunk = (lane & 7) ^ swz(trow);
     k_src[i] = trow * (int)p.ks[2] + 8 * chunk;
     v_src[i] = trow * (int)p.vs[2] + 8 * chunk;
@@ -226,50 +211,66 @@ __global__ __launch_bounds__(256) void block_attn_fwd_kernel(const AttnParams p)
   auto issue_tile = [&](int col, lds_byte* kdst, lds_byte* vdst) {
     const half_t* kt = kb + (int64_t)col * kBN * p.ks[2];
     const half_t* vt = vb + (int64_t)col * kBN * p.vs[2];
-    lds_byte* kd = kdst + (2 * wave) * 1024;
-    lds_byte* vd = vdst + (2 * wave) * 1024;
+    lds_byte* kd = kdst + (kDma * wave) * 1024;
+    lds_byte* vd = vdst + (kDma * wave) * 1024;
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < kDma; ++i)
       __builtin_amdgcn_global_load_lds((gptr_t*)(kt + k_src[i]), (__attribute__((address_space(3))) void*)(kd + i * 1024), 16, 0, 0);
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < kDma; ++i)
       __builtin_amdgcn_global_load_lds((gptr_t*)(vt + v_src[i]), (__attribute__((address_space(3))) void*)(vd + i * 1024), 16, 0, 0);
   };
 
-  // ---- merged walk over the two rows (wave-uniform and identical in all four waves):
-  // each step takes the smaller head of the two lists; a key block listed by both rows is
-  // loaded once and used by all four waves.
-  int it[2] = {0, 0};   // entries consumed per row
+  // ---- merged walk over the group's rows, wave-uniform and identical in every wave.
+  // Key blocks are handled in windows of 64: per window each row's active blocks form a
+  // 64-bit set, the union of the sets is walked with find-first-set, a block listed by
+  // several rows is loaded once, and the bitmask slot of a partial block is the PART list
+  // offset of the window plus the population count of the PART set below the block.
   struct Step { int col; int mine; int slot; bool valid; };
+  const int n_win = (p.nQ + 63) >> 6;
+  int win = -1;
+  uint64_t set_union = 0, set_mine = 0, set_part = 0;
+  int part_base = 0;
+  auto load_window = [&](int w) {
+    set_union = 0; set_mine = 0; set_part = 0;
+#pragma unroll
+    for (int r = 0; r < ROWS; ++r) {
+      uint64_t m = 0;
+      if (KIND == kKindLut) {
+        int e = 0x7fffffff;
+        if (row[r].ptr + lane < row[r].n) e = p.lci[row[r].t0 + row[r].ptr + lane];
+        const int cnt = __builtin_popcountll(__ballot(e < 64 * (w + 1)));
+        for (int j = 0; j < cnt; ++j) m |= 1ull << (__builtin_amdgcn_readlane(e, j) - 64 * w);
+        row[r].ptr += cnt;
+        if (r == rsel) {
+          int pe = 0x7fffffff;
+          if (row[r].pptr + lane < row[r].np) pe = p.pci[row[r].p0 + row[r].pptr + lane];
+          const int pcnt = __builtin_popcountll(__ballot(pe < 64 * (w + 1)));
+          for (int j = 0; j < pcnt; ++j) set_part |= 1ull << (__builtin_amdgcn_readlane(pe, j) - 64 * w);
+          part_base = row[r].p0 + row[r].pptr;
+          row[r].pptr += pcnt;
+        }
+      } else {
+        const int a = max(row[r].lo, 64 * w), z = min(row[r].hi, 64 * w + 63);
+        if (a <= z) m = ((z - a == 63) ? ~0ull : ((1ull << (z - a + 1)) - 1)) << (a - 64 * w);
+      }
+      set_union |= m;
+      if (r == rsel) set_mine = m;
+    }
+  };
   auto next_step = [&]() -> Step {
     Step s; s.col = 0; s.mine = 0; s.slot = -1; s.valid = false;
-    int ca = 0x7fffffff, cb = 0x7fffffff;
-    if (KIND == kKindLut) {
-#pragma unroll
-      for (int r = 0; r < 2; ++r)
-        if (it[r] < row[r].n && it[r] - row[r].base == 64) {   // refill the 64-entry window
-          row[r].base += 64;
-          row[r].fill(p, lane, true);
-        }
-      if (it[0] < row[0].n) ca = __builtin_amdgcn_readlane(row[0].col, it[0] - row[0].base);
-      if (it[1] < row[1].n) cb = __builtin_amdgcn_readlane(row[1].col, it[1] - row[1].base);
-    } else {
-      if (it[0] < row[0].n) ca = row_lo[0] + it[0];
-      if (it[1] < row[1].n) cb = row_lo[1] + it[1];
+    while (set_union == 0) {
+      if (++win >= n_win) return s;
+      load_window(win);
     }
-    if (ca == 0x7fffffff && cb == 0x7fffffff) return s;
+    const int bit = __builtin_ctzll(set_union);
+    set_union &= set_union - 1;
     s.valid = true;
-    s.col = min(ca, cb);
-    const bool use_a = ca == s.col, use_b = cb == s.col;
-    int slot_a = -1, slot_b = -1;
-    if (KIND == kKindLut) {
-      if (use_a) slot_a = __builtin_amdgcn_readlane(row[0].slot, it[0] - row[0].base);
-      if (use_b) slot_b = __builtin_amdgcn_readlane(row[1].slot, it[1] - row[1].base);
-    }
-    s.mine = rsel ? use_b : use_a;
-    s.slot = rsel ? slot_b : slot_a;
-    if (use_a) ++it[0];
-    if (use_b) ++it[1];
+    s.col = 64 * win + bit;
+    s.mine = (int)((set_mine >> bit) & 1);
+    if (KIND == kKindLut && s.mine && ((set_part >> bit) & 1))
+      s.slot = part_base + __builtin_popcountll(set_part & ((1ull << bit) - 1));
     return s;
   };
 
@@ -437,6 +438,11 @@ __global__ __launch_bounds__(256) void pack_mask_bits_kernel(const half_t* __res
   }
 }
 
+// Query blocks per workgroup.  Four rows share each K/V tile among eight waves and halve the
+// L2 -> LDS traffic again, but lengthen every workgroup's chain of key blocks; that pays only
+// when the grid still fills the 256 CUs several times over.
+int rows_per_group(int64_t query_blocks) { return query_blocks >= 4 * 2048 ? 4 : 2; }
+
 bool strides_ok(const int64_t s[3]) {
   return (s[0] % 8 == 0) && (s[1] % 8 == 0) && (s[2] % 8 == 0) && s[2] >= kD && s[2] < (1 << 20);
 }
@@ -467,7 +473,8 @@ extern "C" int stof_block_attn_fwd(
   if (!stof_aligned16(q) || !stof_aligned16(k) || !stof_aligned16(v) || !stof_aligned16(out)) return STOF_ERR_MISALIGNED;
   if (!strides_ok(q_strides) || !strides_ok(k_strides) || !strides_ok(v_strides) || !strides_ok(out_strides))
     return STOF_ERR_MISALIGNED;
-  const int nP = (nQ + 1) / 2;
+  const int rows = rows_per_group((int64_t)nQ * batch_size * head_num);
+  const int nP = (nQ + rows - 1) / rows;
   const int64_t total64 = (int64_t)nP * batch_size * head_num;
   if (total64 > (int64_t)1 << 30) return STOF_ERR_BAD_SHAPE;
 
@@ -482,7 +489,10 @@ extern "C" int stof_block_attn_fwd(
   p.chunk = (p.total + 7) / 8;
   p.c = softmax_scale * 1.4426950408889634f;
   p.row_bits = nullptr; p.words = 0; p.causal = 0; p.band = 0;
-  hipLaunchKernelGGL(block_attn_fwd_kernel<kKindLut>, dim3(p.chunk * 8), dim3(256), 0, (hipStream_t)stream, p);
+  if (rows == 4)
+    hipLaunchKernelGGL((block_attn_fwd_kernel<kKindLut, 4>), dim3(p.chunk * 8), dim3(512), 0, (hipStream_t)stream, p);
+  else
+    hipLaunchKernelGGL((block_attn_fwd_kernel<kKindLut, 2>), dim3(p.chunk * 8), dim3(256), 0, (hipStream_t)stream, p);
   return stof_check_launch();
 }
 
@@ -498,7 +508,7 @@ extern "C" int stof_rowwise_attn_fwd(
   if (seq_len % kBM != 0) return STOF_ERR_BAD_SHAPE;
   if (kind == STOF_ROW_SLIDING && bandwidth <= 0) return STOF_ERR_BAD_SHAPE;
   if (!stof_aligned16(q) || !stof_aligned16(k) || !stof_aligned16(v) || !stof_aligned16(out)) return STOF_ERR_MISALIGNED;
-  const int nQ = seq_len / kBM, nP = (nQ + 1) / 2;
+  const int nQ = seq_len / kBM, nP = (nQ + 1) / 2;   // row-wise front-ends: pairs of query blocks
   const int64_t total64 = (int64_t)nP * batch_size * head_num;
   if (total64 > (int64_t)1 << 30) return STOF_ERR_BAD_SHAPE;
   AttnParams p;
@@ -514,9 +524,9 @@ extern "C" int stof_rowwise_attn_fwd(
   p.row_bits = mask_bits; p.words = seq_len / 64; p.causal = is_causal ? 1 : 0;
   p.band = kind == STOF_ROW_SLIDING ? bandwidth : 0;
   if (kind == STOF_ROW_MASK)
-    hipLaunchKernelGGL(block_attn_fwd_kernel<kKindBits>, dim3(p.chunk * 8), dim3(256), 0, (hipStream_t)stream, p);
+    hipLaunchKernelGGL((block_attn_fwd_kernel<kKindBits, 2>), dim3(p.chunk * 8), dim3(256), 0, (hipStream_t)stream, p);
   else
-    hipLaunchKernelGGL(block_attn_fwd_kernel<kKindPred>, dim3(p.chunk * 8), dim3(256), 0, (hipStream_t)stream, p);
+    hipLaunchKernelGGL((block_attn_fwd_kernel<kKindPred, 2>), dim3(p.chunk * 8), dim3(256), 0, (hipStream_t)stream, p);
   return stof_check_launch();
 }
 
