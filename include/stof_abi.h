@@ -68,7 +68,8 @@ const char* stof_status_string(int status);
  * query block i/block_m are visited; one that also appears in that row's PART list (at
  * position `slot` of the PART arrays) uses the 64-bit row masks
  * part_bitmask[slot*block_m + (i % block_m)] (bit j%block_n set = allowed), any other is
- * unmasked.  LOAD must be the union of FULL and PART, as get_sparse_storage builds it
+ * unmasked.  LOAD must be the union of FULL and PART and every row's LOAD and PART lists
+ * must hold strictly ascending key-block indices, as get_sparse_storage builds them
  * (src/util/masks.py:149-166), which makes this the three-way rule of
  * block_attn_mask_cuda.cu:3675-3700; the FULL arrays are accepted for signature parity and
  * not read.  Query rows without any allowed key produce zeros.
@@ -84,7 +85,7 @@ const char* stof_status_string(int status);
  * offsets into the (concatenated) column lists and bitmask slots.
  *
  * Supported: D == 64, block_m == block_n == 64, S % 64 == 0.  num_warps of the
- * reference launcher has no counterpart: one wavefront owns one query block.
+ * reference launcher has no counterpart: a workgroup of four wavefronts owns two query blocks.
  */
 int stof_block_attn_fwd(
     const void* q, const void* k, const void* v, void* out,

@@ -438,10 +438,11 @@ __global__ __launch_bounds__(256) void pack_mask_bits_kernel(const half_t* __res
   }
 }
 
-// Query blocks per workgroup.  Four rows share each K/V tile among eight waves and halve the
-// L2 -> LDS traffic again, but lengthen every workgroup's chain of key blocks; that pays only
-// when the grid still fills the 256 CUs several times over.
-int rows_per_group(int64_t query_blocks) { return query_blocks >= 4 * 2048 ? 4 : 2; }
+// Query blocks per workgroup.  Two rows (four waves) is what is launched: four rows (eight
+// waves) halve the L2 -> LDS traffic once more but measured no faster on MI355X (the kernel
+// is bound by VALU/MFMA issue, not by that traffic) while lengthening every workgroup's chain
+// of key blocks.
+constexpr int kRowsPerGroup = 2;
 
 bool strides_ok(const int64_t s[3]) {
   return (s[0] % 8 == 0) && (s[1] % 8 == 0) && (s[2] % 8 == 0) && s[2] >= kD && s[2] < (1 << 20);
@@ -473,8 +474,7 @@ extern "C" int stof_block_attn_fwd(
   if (!stof_aligned16(q) || !stof_aligned16(k) || !stof_aligned16(v) || !stof_aligned16(out)) return STOF_ERR_MISALIGNED;
   if (!strides_ok(q_strides) || !strides_ok(k_strides) || !strides_ok(v_strides) || !strides_ok(out_strides))
     return STOF_ERR_MISALIGNED;
-  const int rows = rows_per_group((int64_t)nQ * batch_size * head_num);
-  const int nP = (nQ + rows - 1) / rows;
+  const int nP = (nQ + kRowsPerGroup - 1) / kRowsPerGroup;
   const int64_t total64 = (int64_t)nP * batch_size * head_num;
   if (total64 > (int64_t)1 << 30) return STOF_ERR_BAD_SHAPE;
 
@@ -489,10 +489,8 @@ extern "C" int stof_block_attn_fwd(
   p.chunk = (p.total + 7) / 8;
   p.c = softmax_scale * 1.4426950408889634f;
   p.row_bits = nullptr; p.words = 0; p.causal = 0; p.band = 0;
-  if (rows == 4)
-    hipLaunchKernelGGL((block_attn_fwd_kernel<kKindLut, 4>), dim3(p.chunk * 8), dim3(512), 0, (hipStream_t)stream, p);
-  else
-    hipLaunchKernelGGL((block_attn_fwd_kernel<kKindLut, 2>), dim3(p.chunk * 8), dim3(256), 0, (hipStream_t)stream, p);
+  hipLaunchKernelGGL((block_attn_fwd_kernel<kKindLut, kRowsPerGroup>), dim3(p.chunk * 8), dim3(128 * kRowsPerGroup), 0,
+                     (hipStream_t)stream, p);
   return stof_check_launch();
 }
 
@@ -508,7 +506,7 @@ extern "C" int stof_rowwise_attn_fwd(
   if (seq_len % kBM != 0) return STOF_ERR_BAD_SHAPE;
   if (kind == STOF_ROW_SLIDING && bandwidth <= 0) return STOF_ERR_BAD_SHAPE;
   if (!stof_aligned16(q) || !stof_aligned16(k) || !stof_aligned16(v) || !stof_aligned16(out)) return STOF_ERR_MISALIGNED;
-  const int nQ = seq_len / kBM, nP = (nQ + 1) / 2;   // row-wise front-ends: pairs of query blocks
+  const int nQ = seq_len / kBM, nP = (nQ + kRowsPerGroup - 1) / kRowsPerGroup;
   const int64_t total64 = (int64_t)nP * batch_size * head_num;
   if (total64 > (int64_t)1 << 30) return STOF_ERR_BAD_SHAPE;
   AttnParams p;
@@ -524,9 +522,9 @@ extern "C" int stof_rowwise_attn_fwd(
   p.row_bits = mask_bits; p.words = seq_len / 64; p.causal = is_causal ? 1 : 0;
   p.band = kind == STOF_ROW_SLIDING ? bandwidth : 0;
   if (kind == STOF_ROW_MASK)
-    hipLaunchKernelGGL((block_attn_fwd_kernel<kKindBits, 2>), dim3(p.chunk * 8), dim3(256), 0, (hipStream_t)stream, p);
+    hipLaunchKernelGGL((block_attn_fwd_kernel<kKindBits, kRowsPerGroup>), dim3(p.chunk * 8), dim3(128 * kRowsPerGroup), 0, (hipStream_t)stream, p);
   else
-    hipLaunchKernelGGL((block_attn_fwd_kernel<kKindPred, 2>), dim3(p.chunk * 8), dim3(256), 0, (hipStream_t)stream, p);
+    hipLaunchKernelGGL((block_attn_fwd_kernel<kKindPred, kRowsPerGroup>), dim3(p.chunk * 8), dim3(128 * kRowsPerGroup), 0, (hipStream_t)stream, p);
   return stof_check_launch();
 }
 

@@ -73,6 +73,37 @@ def _packed_partial_bits(part_block_mask):
     return bits
 
 
+_LUT_OK_ATTR = "_stof_lut_checked"
+
+
+def _check_lut_order(lrp, lci, prp, pci, n_cols):
+    """The kernel walks each row's LOAD and PART lists as ascending sets (that is how
+    get_sparse_storage emits them); verify once per column-list tensor and content version."""
+    cached = getattr(lci, _LUT_OK_ATTR, None)
+    key = (lci._version, pci._version, lrp._version, prp._version)
+    if cached == key:
+        return
+    for name, rp, ci in (("load", lrp, lci), ("part", prp, pci)):
+        if ci.numel() == 0:
+            continue
+        flat = rp.reshape(-1, rp.shape[-1]).long()
+        ok = bool((ci >= 0).all()) and bool((ci < n_cols).all())
+        if ci.numel() > 1:
+            inc = ci[1:] > ci[:-1]
+            starts = torch.zeros(ci.numel(), dtype=torch.bool, device=ci.device)
+            idx = flat[:, :-1].reshape(-1)
+            idx = idx[idx < ci.numel()]
+            starts[idx] = True               # a row boundary may go down
+            ok = ok and bool((inc | starts[1:]).all())
+        ok = ok and bool((flat[:, 1:] >= flat[:, :-1]).all()) and int(flat.max()) <= ci.numel()
+        _require(ok, f"{name}_row_ptr / {name}_col_idx must describe rows of strictly ascending key-block "
+                     f"indices in [0, {n_cols}) (get_sparse_storage's layout)")
+    try:
+        setattr(lci, _LUT_OK_ATTR, key)
+    except AttributeError:
+        pass
+
+
 def _check_i32(name, t, device):
     _require(t.dtype == torch.int32, f"{name} must be int32, got {t.dtype}")
     _require(t.device == device, f"{name} is on {t.device}, expected {device}")
@@ -110,6 +141,7 @@ def block_attn(q, k, v, lut, block_m=64, block_n=64, out=None, out_layout="bhsd"
         _require(lrp.numel() == nq + 1 and frp.numel() == nq + 1 and prp.numel() == nq + 1,
                  f"row pointers must have {nq + 1} entries for seq_len {S}, block_m {block_m}")
         lut_bs = 0
+    _check_lut_order(lrp, lci, prp, pci, S // block_n)
     bits = _packed_partial_bits(pbm)
     if out is None:
         if out_layout == "bhsd":

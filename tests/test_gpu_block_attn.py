@@ -179,6 +179,12 @@ def test_error_paths_raise():
     bad = list(lut); bad[5] = lut[5].long()
     with pytest.raises(StofError):
         block_attn(q, k, v, tuple(bad))                        # int64 row pointers
+    bad = list(lut); bad[6] = torch.flip(lut[6], dims=[0])
+    with pytest.raises(StofError):
+        block_attn(q, k, v, tuple(bad))                        # column indices not ascending within rows
+    bad = list(lut); bad[6] = lut[6] + 5
+    with pytest.raises(StofError):
+        block_attn(q, k, v, tuple(bad))                        # column index out of range
     q96 = torch.randn(1, 2, 128, 96, device="cuda").half()
     with pytest.raises(StofError):
         block_attn(q96, q96, q96, lut)                         # head size 96
