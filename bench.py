@@ -34,8 +34,8 @@ PEAK_HBM_GBS = 8000.0         # MI355X HBM3E peak (published)
 FLOP_PER_BLOCK = 4 * 64 * 64 * 64
 
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (two runs),
-# scaled by the same counters on a torch copy kernel of known size; see profiles/.
-MEASURED_TRAFFIC_BYTES = {"C2": None}
+# scaled by the same counters on a 256 MiB fill + copy in the same run (profiles/block_attn_C2_hbm_traffic.txt).
+MEASURED_TRAFFIC_BYTES = {"C2": 50.5e6}   # fetch 37.9 MB + write 12.6 MB; algorithmic minimum 50.3 MB
 
 
 def attn_setup(cfg, mask_fn, device):
