@@ -356,7 +356,6 @@ __global__ __launch_bounds__(128 * ROWS) void block_attn_fwd_kernel(const AttnPa
     const float mc = m_sub * p.c;
     half8_t pf[2][2];   // [key tile][half]: B operand of O^T = V^T . P^T
     float lsum = 0.f;
-    const half2_t ones2 = {(half_t)1.0f, (half_t)1.0f};
 #pragma unroll
     for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
@@ -366,8 +365,9 @@ __global__ __launch_bounds__(128 * ROWS) void block_attn_fwd_kernel(const AttnPa
         const half2_t e2 = {(half_t)e0, (half_t)e1};
         pf[mt][r >> 3][r & 7] = e2[0];
         pf[mt][r >> 3][(r & 7) + 1] = e2[1];
-        // row sum of the ROUNDED probabilities (what P.V multiplies), two per instruction
-        lsum = __builtin_amdgcn_fdot2(e2, ones2, lsum, false);
+        // Row sum with plain adds: v_dot2c_f32_f16 would halve the instruction count but runs
+        // on the matrix pipeline and stalls behind every MFMA in flight on the SIMD.
+        lsum += e0 + e1;
       }
     l_run = l_run * alpha + lsum;   // per-lane partial sum; the two halves are added at the end
     m_run = m_new;
