@@ -125,22 +125,54 @@ def bench_layer_c3(steps, warmup):
 
 
 def bench_hbm_kernels(steps, warmup):
+    """HBM-bound kernels: bias+residual+LayerNorm (3 x M x N x 2 bytes) at the C3 size and at a
+    size large enough to leave the launch-latency regime, and the fp16 mask -> bit-row pack."""
     from stof import fused
     from stof.ops import pack_mask_bits
-    M, N = 8192, 768
+    out = {}
     g = torch.Generator().manual_seed(0)
-    x = torch.randn(M, N, generator=g).half().cuda(); r = torch.randn(M, N, generator=g).half().cuda()
-    b = torch.randn(N, generator=g).half().cuda()
-    _, ev = time_region(lambda: fused.bias_residual_layernorm(x, b, r, b, b, 1e-12), steps, warmup)
-    ln_bytes = 3 * M * N * 2
+    for tag, M, N in (("bias_res_ln", 8192, 768), ("bias_res_ln_M131072", 131072, 768)):
+        x = torch.randn(M, N, generator=g).half().cuda(); r = torch.randn(M, N, generator=g).half().cuda()
+        b = torch.randn(N, generator=g).half().cuda()
+        _, ev = time_region(lambda: fused.bias_residual_layernorm(x, b, r, b, b, 1e-12), steps, warmup)
+        nbytes = 3 * M * N * 2
+        out[tag] = {"ms": ev, "GBs": nbytes / ev / 1e6, "frac_hbm": nbytes / ev / 1e6 / PEAK_HBM_GBS, "shape": [M, N]}
+        del x, r
+    # what a plain device copy reaches on this machine (read + write of 256 MiB each way)
+    src = torch.empty(256 << 20, dtype=torch.uint8, device="cuda").fill_(1)
+    dst = torch.empty_like(src)
+    _, evc = time_region(lambda: dst.copy_(src), 20, 5)
+    out["device_copy_256MiB"] = {"ms": evc, "GBs": 2 * src.numel() / evc / 1e6,
+                                 "frac_hbm": 2 * src.numel() / evc / 1e6 / PEAK_HBM_GBS}
+    del src, dst
     S = 4096
     m = (torch.rand(S, S, generator=g) < 0.5).half().cuda()
     _, ev2 = time_region(lambda: pack_mask_bits(m, additive=False), steps, warmup)
     pk_bytes = S * S * 2 + S * S // 8
-    return {"bias_res_ln": {"ms": ev, "GBs": ln_bytes / ev / 1e6, "frac_hbm": ln_bytes / ev / 1e6 / PEAK_HBM_GBS,
-                            "shape": [M, N]},
-            "pack_mask_bits": {"ms": ev2, "GBs": pk_bytes / ev2 / 1e6, "frac_hbm": pk_bytes / ev2 / 1e6 / PEAK_HBM_GBS,
-                               "shape": [S, S]}}
+    out["pack_mask_bits"] = {"ms": ev2, "GBs": pk_bytes / ev2 / 1e6, "frac_hbm": pk_bytes / ev2 / 1e6 / PEAK_HBM_GBS,
+                             "shape": [S, S]}
+    return out
+
+
+def bench_lut_build(with_cpu):
+    """Block LUT of the C4 mask (S 4096, 64 x 64 blocks) built on the GPU, and the reference's
+    Python double loop (restated in oracle/) on the host for the same mask at S 2048."""
+    from stof import configs, masks as pm
+    mask = configs.mask_c4(4096).float()[None].cuda()
+    pm.get_sparse_storage(mask, 64, 64)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(5):
+        pm.get_sparse_storage(mask, 64, 64)
+    torch.cuda.synchronize()
+    out = {"gpu_ms_S4096": (time.perf_counter() - t0) / 5 * 1e3}
+    if with_cpu:
+        from oracle import masks as om
+        m2 = configs.mask_c4(2048).float()[None].numpy()
+        t0 = time.perf_counter()
+        om.get_sparse_storage(m2, 64, 64)
+        out["cpu_loop_ms_S2048"] = (time.perf_counter() - t0) * 1e3
+    return out
 
 
 def main():
@@ -196,6 +228,7 @@ def main():
                                    "kernel_ms": c4b["kernel_ms"]}
         also["C3_bert_base_layer"] = bench_layer_c3(max(args.steps // 4, 20), 10)
         also["hbm_bound"] = bench_hbm_kernels(args.steps, args.warmup)
+        also["lut_build"] = bench_lut_build(not args.no_cpu)
         line["also"] = also
     print(json.dumps(line))
 

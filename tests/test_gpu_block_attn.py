@@ -188,3 +188,34 @@ def test_error_paths_raise():
     q96 = torch.randn(1, 2, 128, 96, device="cuda").half()
     with pytest.raises(StofError):
         block_attn(q96, q96, q96, lut)                         # head size 96
+
+
+def _unpack_bits(words, cols):
+    """int64 bit rows [rows, cols/64] -> bool [rows, cols] (bit t of word w = column 64w + t)."""
+    w = words.cpu().numpy().view(np.uint64)
+    t = np.arange(64, dtype=np.uint64)
+    return ((w[:, :, None] >> t[None, None, :]) & np.uint64(1)).astype(bool).reshape(w.shape[0], cols)
+
+
+@pytest.mark.parametrize("additive", [True, False])
+def test_pack_mask_bits_vector_and_scalar_paths(additive):
+    """Bit-exact against numpy; the 16-byte path (contiguous rows) and the scalar path (row
+    pitch not a multiple of 8 elements, reached through the C ABI) must agree."""
+    from stof import _lib
+    from stof.ops import pack_mask_bits
+    g = torch.Generator().manual_seed(5)
+    rows, cols = 200, 192          # 600 words: not a multiple of the 8 words a wavefront packs per pass
+    keep = torch.rand(rows, cols, generator=g) < 0.4
+    src = torch.where(keep, 0.0, -10000.0) if additive else keep.float()
+    src = src.half().cuda()
+    got = pack_mask_bits(src, additive=additive)
+    assert np.array_equal(_unpack_bits(got, cols), keep.numpy())
+    # scalar path: rows at a pitch of cols + 4 elements
+    ld = cols + 4
+    padded = torch.zeros(rows, ld, dtype=torch.float16, device="cuda")
+    padded[:, :cols] = src
+    dst = torch.zeros(rows, cols // 64, dtype=torch.int64, device="cuda")
+    rc = _lib.lib().stof_pack_mask_bits(padded.data_ptr(), dst.data_ptr(), rows, cols, ld, 1 if additive else 0, None)
+    assert rc == 0
+    torch.cuda.synchronize()
+    assert np.array_equal(_unpack_bits(dst, cols), keep.numpy())
