@@ -85,7 +85,7 @@ const char* stof_status_string(int status);
  * offsets into the (concatenated) column lists and bitmask slots.
  *
  * Supported: D == 64, block_m == block_n == 64, S % 64 == 0.  num_warps of the
- * reference launcher has no counterpart: a workgroup of four wavefronts owns two query blocks.
+ * reference launcher has no per-call counterpart: see stof_attn_set_launch_form.
  */
 int stof_block_attn_fwd(
     const void* q, const void* k, const void* v, void* out,
@@ -97,6 +97,18 @@ int stof_block_attn_fwd(
     const int64_t v_strides[3], const int64_t out_strides[3],
     int batch_size, int seq_len, int head_num, int head_size,
     int64_t lut_batch_stride, void* stream);
+
+/*
+ * Launch form of the two attention entry points, process-wide:
+ *   -1 automatic (default): chosen from the grid size per call;
+ *    0 two query blocks per workgroup, K/V tiles shared by four wavefronts (large grids);
+ *    1 one query block per workgroup, the 64 keys of every tile split over two wavefront
+ *      pairs whose partial results are merged at the end (small grids).
+ * Results are equal within rounding in every form.  This is the counterpart of the
+ * reference's kernel selection by (num_warps, BLOCK_M, BLOCK_N), block_attn_mask_cuda.cu:6064-6322,
+ * there an argument of every call.  Returns STOF_ERR_UNSUPPORTED for another value.
+ */
+int stof_attn_set_launch_form(int form);
 
 /*
  * Pack fp16 mask rows into bit rows: dst[r*(cols/64) + w] bit t = pred(src[r*ld + 64*w + t]).

@@ -92,9 +92,17 @@ struct RowList {
   int lo, hi;          // KIND != LUT: the contiguous key-block range [lo, hi]
 };
 
-template <int KIND, int ROWS>
-__global__ __launch_bounds__(128 * ROWS) void block_attn_fwd_kernel(const AttnParams p) {
-  constexpr int kDma = 4 / ROWS;   // direct-to-LDS instructions per wave and operand tile (8 over 2*ROWS waves)
+// ROWS = query blocks per workgroup, KS = key split.  Launched as <2, 1> (four waves: two query
+// blocks x two 32-query halves, every wave sees all 64 keys of a tile) or <1, 2> (four waves
+// on ONE query block: two 32-query halves x two 32-key halves of every tile, partial results
+// merged through LDS at the end).  The second form halves the work of a wave per key block,
+// so the chain of key blocks of a long LUT row finishes in half the time; it is used for
+// small grids, where that chain and not throughput sets the run time.
+template <int KIND, int ROWS, int KS>
+__global__ __launch_bounds__(128 * ROWS * KS, KS == 2 ? 5 : 4) void block_attn_fwd_kernel(const AttnParams p) {
+  static_assert(KS == 1 || ROWS == 1, "the key split serves a single query block");
+  constexpr int kDma = 4 / (ROWS * KS);   // direct-to-LDS instructions per wave and operand tile (8 per tile)
+  constexpr int kMT = 2 / KS;             // 32-key sub-tiles of a key block handled by one wave
   // Four distinct LDS objects (K and V, two buffers each): the compiler orders LDS reads
   // after in-flight direct-to-LDS loads per object, so a read of the current buffer does
   // not wait for the loads that fill the other one.
@@ -107,8 +115,9 @@ __global__ __launch_bounds__(128 * ROWS) void block_attn_fwd_kernel(const AttnPa
   const int lane = threadIdx.x & 63;
   const int j32 = lane & 31;
   const int g = lane >> 5;
-  const int rsel = wave >> 1;    // which of the pair's two query blocks this wave serves
-  const int half = wave & 1;     // which 32 queries of that block
+  const int rsel = KS == 1 ? wave >> 1 : 0;   // which of the group's query blocks this wave serves
+  const int half = wave & 1;                  // which 32 queries of that block
+  const int mt0 = KS == 1 ? 0 : wave >> 1;    // first 32-key sub-tile of this wave
 
   // Workgroups are handed to the 8 XCDs round-robin; give each XCD a contiguous range
   // of (batch, head, query-block pair) so one head's K/V is read through a single L2.
@@ -314,24 +323,24 @@ __global__ __launch_bounds__(128 * ROWS) void block_attn_fwd_kernel(const AttnPa
     }
 
     // ---- S^T = K . Q^T : sacc[mt][r] = S[query j32][key 32mt + 8(r/4) + 4g + r%4]
-    floatx16 sacc[2];
+    floatx16 sacc[kMT];
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < kMT; ++i)
 #pragma unroll
       for (int r = 0; r < 16; ++r) sacc[i][r] = 0.f;
 #pragma unroll
     for (int ks = 0; ks < 4; ++ks)
 #pragma unroll
-      for (int mt = 0; mt < 2; ++mt) {
-        const half8_t a = *reinterpret_cast<const __attribute__((address_space(3))) half8_t*>(kt + mt * 4096 + k_rd[ks]);
+      for (int mt = 0; mt < kMT; ++mt) {
+        const half8_t a = *reinterpret_cast<const __attribute__((address_space(3))) half8_t*>(kt + (mt0 + mt) * 4096 + k_rd[ks]);
         sacc[mt] = mfma32(a, qf[ks], sacc[mt]);
       }
 
     // ---- element mask of a partial tile
     if (need_mask) {
 #pragma unroll
-      for (int mt = 0; mt < 2; ++mt) {
-        const uint32_t w = (uint32_t)(bits >> (32 * mt)) >> (4 * g);
+      for (int mt = 0; mt < kMT; ++mt) {
+        const uint32_t w = (uint32_t)(bits >> (32 * (mt0 + mt))) >> (4 * g);
 #pragma unroll
         for (int r = 0; r < 16; ++r)
           if (!((w >> (8 * (r >> 2) + (r & 3))) & 1u)) sacc[mt][r] = kMasked;
@@ -344,7 +353,7 @@ __global__ __launch_bounds__(128 * ROWS) void block_attn_fwd_kernel(const AttnPa
     // normalisation by the running sum stays exact, and the O rescale becomes rare.
     float mx = sacc[0][0];
 #pragma unroll
-    for (int mt = 0; mt < 2; ++mt)
+    for (int mt = 0; mt < kMT; ++mt)
 #pragma unroll
       for (int r = 0; r < 16; ++r) mx = fmaxf(mx, sacc[mt][r]);
     mx = pair_max(mx);
@@ -354,10 +363,10 @@ __global__ __launch_bounds__(128 * ROWS) void block_attn_fwd_kernel(const AttnPa
     const float m_sub = (m_new == -INFINITY) ? 0.f : m_new;
     const float alpha = __builtin_amdgcn_exp2f((m_run - m_sub) * p.c);
     const float mc = m_sub * p.c;
-    half8_t pf[2][2];   // [key tile][half]: B operand of O^T = V^T . P^T
+    half8_t pf[kMT][2];   // [key sub-tile][half]: B operand of O^T = V^T . P^T
     float lsum = 0.f;
 #pragma unroll
-    for (int mt = 0; mt < 2; ++mt)
+    for (int mt = 0; mt < kMT; ++mt)
 #pragma unroll
       for (int r = 0; r < 16; r += 2) {
         const float e0 = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[mt][r], p.c, -mc));
@@ -380,12 +389,12 @@ __global__ __launch_bounds__(128 * ROWS) void block_attn_fwd_kernel(const AttnPa
 
     // ---- O^T += V^T . P^T
 #pragma unroll
-    for (int mt = 0; mt < 2; ++mt)
+    for (int mt = 0; mt < kMT; ++mt)
 #pragma unroll
       for (int s2 = 0; s2 < 2; ++s2)
 #pragma unroll
         for (int dt = 0; dt < 2; ++dt) {
-          const lds_byte* vp = vt + (32 * mt + 16 * s2) * 128;
+          const lds_byte* vp = vt + (32 * (mt0 + mt) + 16 * s2) * 128;
           const short4_t a0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4*)(vp + v_rd[dt][0]));
           const short4_t a1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4*)(vp + v_rd[dt][1]));
           const half8_t a = __builtin_bit_cast(half8_t, (short8_t)__builtin_shufflevector(a0, a1, 0, 1, 2, 3, 4, 5, 6, 7));
@@ -401,6 +410,35 @@ __global__ __launch_bounds__(128 * ROWS) void block_attn_fwd_kernel(const AttnPa
     if (!nxt.valid) break;
     cur = next_step();
     step(nxt, cur, (const lds_byte*)k_lds1, (const lds_byte*)v_lds1, (lds_byte*)k_lds0, (lds_byte*)v_lds0);
+  }
+
+  // ---- key split: the waves of the second key half hand their (max, sum, O) to the waves of
+  // the first through LDS (the tile buffers are free now: the last step issued no loads), lane
+  // to lane, since both hold the same queries in the same register layout.
+  if (KS == 2) {
+    float* xo = reinterpret_cast<float*>(half ? k_lds1 : k_lds0);   // 32 x 64 floats = one tile buffer
+    float* xs = reinterpret_cast<float*>(v_lds0) + 128 * half;
+    __syncthreads();
+    if (mt0 == 1) {
+#pragma unroll
+      for (int dt = 0; dt < 2; ++dt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) xo[(16 * dt + r) * 64 + lane] = oacc[dt][r];
+      xs[lane] = m_run;
+      xs[64 + lane] = l_run;
+    }
+    __syncthreads();
+    if (mt0 == 1) return;
+    const float m_b = xs[lane], l_b = xs[64 + lane];
+    const float m = fmaxf(m_run, m_b);
+    // a side that has seen no allowed key (max still -inf) contributes nothing
+    const float fa = (m_run == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f((m_run - m) * p.c);
+    const float fb = (m_b == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f((m_b - m) * p.c);
+    l_run = l_run * fa + l_b * fb;
+#pragma unroll
+    for (int dt = 0; dt < 2; ++dt)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) oacc[dt][r] = oacc[dt][r] * fa + xo[(16 * dt + r) * 64 + lane] * fb;
   }
 
   // ---- normalise and store: oacc[dt][r] = O[query j32][d = 32dt + 8(r/4) + 4g + r%4]
@@ -474,17 +512,63 @@ __global__ __launch_bounds__(256) void pack_mask_bits_kernel(const half_t* __res
   }
 }
 
-// Query blocks per workgroup.  Two rows (four waves) is what is launched: four rows (eight
-// waves) halve the L2 -> LDS traffic once more but measured no faster on MI355X (the kernel
-// is bound by VALU/MFMA issue, not by that traffic) while lengthening every workgroup's chain
-// of key blocks.
+// Launch forms.  Two query blocks per workgroup share every K/V tile between four waves and
+// halve the L2 -> LDS traffic per unit of MFMA work: the form for large grids.  (Four query
+// blocks per workgroup halve it once more but measured no faster on MI355X, the kernel being
+// bound by VALU/MFMA issue, not by that traffic.)  One query block per workgroup with the keys
+// of each tile split over two wave pairs is the form for small grids, which are bound by the
+// longest chain of key blocks: the chain runs twice as fast.
 constexpr int kRowsPerGroup = 2;
+enum { kFormAuto = -1, kFormTwoRows = 0, kFormKeySplit = 1 };
+int g_attn_form = kFormAuto;
+
+// Automatic choice: key split when the two-row grid gives a compute unit at most this many
+// workgroups AND the sequence has at least this many query blocks.  Measured on MI355X
+// (B8 H12 S1024, rows of 7..16 key blocks: 37 -> 31 us); at four workgroups per compute unit
+// or with short sequences (S 512) the two forms are within 5 % and the two-row form, which
+// moves half the bytes, is kept.
+constexpr int kKeySplitMaxGroupsPerCu = 3;
+constexpr int kKeySplitMinQueryBlocks = 16;
+
+bool use_key_split(int64_t two_row_groups, int nQ) {
+  if (g_attn_form != kFormAuto) return g_attn_form == kFormKeySplit;
+  static int cus = 0;
+  if (cus == 0) {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+      n = 256;
+    cus = n;
+  }
+  return nQ >= kKeySplitMinQueryBlocks && two_row_groups <= (int64_t)kKeySplitMaxGroupsPerCu * cus;
+}
+
+template <int KIND>
+void launch_attn(AttnParams& p, int nQ, int64_t bh, hipStream_t stream) {
+  const int64_t two_row_groups = (int64_t)((nQ + kRowsPerGroup - 1) / kRowsPerGroup) * bh;
+  if (use_key_split(two_row_groups, nQ)) {
+    p.nP = nQ;
+    p.total = (int)(nQ * bh);
+    p.chunk = (p.total + 7) / 8;
+    hipLaunchKernelGGL((block_attn_fwd_kernel<KIND, 1, 2>), dim3(p.chunk * 8), dim3(256), 0, stream, p);
+  } else {
+    p.nP = (nQ + kRowsPerGroup - 1) / kRowsPerGroup;
+    p.total = (int)two_row_groups;
+    p.chunk = (p.total + 7) / 8;
+    hipLaunchKernelGGL((block_attn_fwd_kernel<KIND, kRowsPerGroup, 1>), dim3(p.chunk * 8), dim3(128 * kRowsPerGroup), 0, stream, p);
+  }
+}
 
 bool strides_ok(const int64_t s[3]) {
   return (s[0] % 8 == 0) && (s[1] % 8 == 0) && (s[2] % 8 == 0) && s[2] >= kD && s[2] < (1 << 20);
 }
 
 }  // namespace
+
+extern "C" int stof_attn_set_launch_form(int form) {
+  if (form != kFormAuto && form != kFormTwoRows && form != kFormKeySplit) return STOF_ERR_UNSUPPORTED;
+  g_attn_form = form;
+  return STOF_OK;
+}
 
 extern "C" int stof_block_attn_fwd(
     const void* q, const void* k, const void* v, void* out,
@@ -510,9 +594,7 @@ extern "C" int stof_block_attn_fwd(
   if (!stof_aligned16(q) || !stof_aligned16(k) || !stof_aligned16(v) || !stof_aligned16(out)) return STOF_ERR_MISALIGNED;
   if (!strides_ok(q_strides) || !strides_ok(k_strides) || !strides_ok(v_strides) || !strides_ok(out_strides))
     return STOF_ERR_MISALIGNED;
-  const int nP = (nQ + kRowsPerGroup - 1) / kRowsPerGroup;
-  const int64_t total64 = (int64_t)nP * batch_size * head_num;
-  if (total64 > (int64_t)1 << 30) return STOF_ERR_BAD_SHAPE;
+  if ((int64_t)nQ * batch_size * head_num > (int64_t)1 << 30) return STOF_ERR_BAD_SHAPE;
 
   AttnParams p;
   p.q = (const half_t*)q; p.k = (const half_t*)k; p.v = (const half_t*)v; p.out = (half_t*)out;
@@ -520,13 +602,10 @@ extern "C" int stof_block_attn_fwd(
   p.pbits = part_bitmask; p.lrp = load_row_ptr; p.lci = load_col_idx;
   for (int i = 0; i < 3; ++i) { p.qs[i] = q_strides[i]; p.ks[i] = k_strides[i]; p.vs[i] = v_strides[i]; p.os[i] = out_strides[i]; }
   p.lut_bs = lut_batch_stride;
-  p.B = batch_size; p.S = seq_len; p.H = head_num; p.nQ = nQ; p.nP = nP;
-  p.total = (int)total64;
-  p.chunk = (p.total + 7) / 8;
+  p.B = batch_size; p.S = seq_len; p.H = head_num; p.nQ = nQ;
   p.c = softmax_scale * 1.4426950408889634f;
   p.row_bits = nullptr; p.words = 0; p.causal = 0; p.band = 0;
-  hipLaunchKernelGGL((block_attn_fwd_kernel<kKindLut, kRowsPerGroup>), dim3(p.chunk * 8), dim3(128 * kRowsPerGroup), 0,
-                     (hipStream_t)stream, p);
+  launch_attn<kKindLut>(p, nQ, (int64_t)batch_size * head_num, (hipStream_t)stream);
   return stof_check_launch();
 }
 
@@ -542,9 +621,8 @@ extern "C" int stof_rowwise_attn_fwd(
   if (seq_len % kBM != 0) return STOF_ERR_BAD_SHAPE;
   if (kind == STOF_ROW_SLIDING && bandwidth <= 0) return STOF_ERR_BAD_SHAPE;
   if (!stof_aligned16(q) || !stof_aligned16(k) || !stof_aligned16(v) || !stof_aligned16(out)) return STOF_ERR_MISALIGNED;
-  const int nQ = seq_len / kBM, nP = (nQ + kRowsPerGroup - 1) / kRowsPerGroup;
-  const int64_t total64 = (int64_t)nP * batch_size * head_num;
-  if (total64 > (int64_t)1 << 30) return STOF_ERR_BAD_SHAPE;
+  const int nQ = seq_len / kBM;
+  if ((int64_t)nQ * batch_size * head_num > (int64_t)1 << 30) return STOF_ERR_BAD_SHAPE;
   AttnParams p;
   p.q = (const half_t*)q; p.k = (const half_t*)k; p.v = (const half_t*)v; p.out = (half_t*)out;
   p.prp = nullptr; p.pci = nullptr; p.pbits = nullptr; p.lrp = nullptr; p.lci = nullptr;
@@ -552,15 +630,12 @@ extern "C" int stof_rowwise_attn_fwd(
   const int64_t out_s[3] = {(int64_t)seq_len * head_num * kD, kD, (int64_t)head_num * kD};   // [B,S,H*D]
   for (int i = 0; i < 3; ++i) { p.qs[i] = in_s[i]; p.ks[i] = in_s[i]; p.vs[i] = in_s[i]; p.os[i] = out_s[i]; }
   p.lut_bs = 0;
-  p.B = batch_size; p.S = seq_len; p.H = head_num; p.nQ = nQ; p.nP = nP;
-  p.total = (int)total64; p.chunk = (p.total + 7) / 8;
+  p.B = batch_size; p.S = seq_len; p.H = head_num; p.nQ = nQ;
   p.c = (1.0f / sqrtf((float)head_size)) * 1.4426950408889634f;
   p.row_bits = mask_bits; p.words = seq_len / 64; p.causal = is_causal ? 1 : 0;
   p.band = kind == STOF_ROW_SLIDING ? bandwidth : 0;
-  if (kind == STOF_ROW_MASK)
-    hipLaunchKernelGGL((block_attn_fwd_kernel<kKindBits, kRowsPerGroup>), dim3(p.chunk * 8), dim3(128 * kRowsPerGroup), 0, (hipStream_t)stream, p);
-  else
-    hipLaunchKernelGGL((block_attn_fwd_kernel<kKindPred, kRowsPerGroup>), dim3(p.chunk * 8), dim3(128 * kRowsPerGroup), 0, (hipStream_t)stream, p);
+  if (kind == STOF_ROW_MASK) launch_attn<kKindBits>(p, nQ, (int64_t)batch_size * head_num, (hipStream_t)stream);
+  else launch_attn<kKindPred>(p, nQ, (int64_t)batch_size * head_num, (hipStream_t)stream);
   return stof_check_launch();
 }
 

@@ -20,7 +20,7 @@ from . import _lib
 from ._lib import StofError, check, strides3
 
 __all__ = ["block_attn", "block_attn_mask_op", "rowwise_attn_full_op", "rowwise_attn_sliding_op",
-           "rowwise_attn_mask_op", "pack_mask_bits", "StofError"]
+           "rowwise_attn_mask_op", "pack_mask_bits", "set_attention_launch_form", "StofError"]
 
 _BITS_ATTR = "_stof_packed_bits"
 
@@ -36,6 +36,19 @@ def _ptr(t):
 def _require(cond, msg):
     if not cond:
         raise StofError(msg)
+
+
+_LAUNCH_FORMS = {"auto": -1, "two_rows": 0, "key_split": 1}
+
+
+def set_attention_launch_form(form="auto"):
+    """Process-wide launch form of the attention kernels: ``"auto"`` (by grid size),
+    ``"two_rows"`` (two query blocks per workgroup, for large grids) or ``"key_split"`` (one
+    query block per workgroup with the keys of each tile split over two wavefront pairs, for
+    small grids).  The reference selects its kernel per call with ``num_warps``
+    (src/ops/src/block_attn_mask_cuda.cu:6064-6322); results agree within rounding here."""
+    _require(form in _LAUNCH_FORMS, f"launch form must be one of {sorted(_LAUNCH_FORMS)}, got {form!r}")
+    check(_lib.lib().stof_attn_set_launch_form(_LAUNCH_FORMS[form]), "stof_attn_set_launch_form")
 
 
 def pack_mask_bits(src, additive):

@@ -64,6 +64,8 @@ def test_block_attn_argument_checks(lib):
 
 def test_other_entry_points_argument_checks(lib):
     P = 4096
+    assert lib.stof_attn_set_launch_form(7) == -3
+    assert lib.stof_attn_set_launch_form(-1) == 0
     assert lib.stof_pack_mask_bits(None, P, 64, 64, 64, 1, None) == -1
     assert lib.stof_pack_mask_bits(P, P, 64, 100, 100, 1, None) == -2
     assert lib.stof_bias_res_ln(P, None, None, None, None, P, None, None, 10, 12, 1e-5, None) == -2   # N % 8

@@ -18,6 +18,15 @@ pytestmark = pytest.mark.gpu
 ATOL, RTOL = 2e-3, 1e-2
 
 
+@pytest.fixture(autouse=True, params=["two_rows", "key_split"])
+def launch_form(request):
+    """Every test of this module runs once per launch form of the kernel."""
+    from stof.ops import set_attention_launch_form
+    set_attention_launch_form(request.param)
+    yield request.param
+    set_attention_launch_form("auto")
+
+
 def _close(got, want, what=""):
     got = got.float().cpu(); want = want.float().cpu()
     err = (got - want).abs()

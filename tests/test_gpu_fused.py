@@ -89,8 +89,16 @@ def test_fused_op_errors():
 
 # ---- row-wise attention front-ends ---------------------------------------------------------------
 
+@pytest.fixture(params=["two_rows", "key_split"])
+def launch_form(request):
+    from stof.ops import set_attention_launch_form
+    set_attention_launch_form(request.param)
+    yield request.param
+    set_attention_launch_form("auto")
+
+
 @pytest.mark.parametrize("B,H,S", [(2, 12, 256), (1, 3, 128), (1, 12, 576)])
-def test_rowwise_ops(B, H, S):
+def test_rowwise_ops(B, H, S, launch_form):
     cfg = configs.AttnConfig("t", B, H, S)
     q, k, v = configs.qkv(cfg, seed=22, device="cuda")
     qc, kc, vc = q.cpu().float(), k.cpu().float(), v.cpu().float()
