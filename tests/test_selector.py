@@ -1,0 +1,53 @@
+"""Host logic of the operator / launch-form selector (reference: select_operator,
+src/benchmk_attn_unified.py:100-163).  The rule is fixed, so the expected answers are derived by
+hand from the workload sizes: two-row workgroups = ceil(S/128) * B * H over 256 compute units."""
+import pytest
+import torch
+
+from stof import configs, masks as pm, selector
+
+
+def _lut(mask2d):
+    return pm.get_sparse_storage(mask2d.float()[None], 64, 64)
+
+
+@pytest.mark.parametrize("name,cfg,mask_fn,form,groups", [
+    ("C1", configs.AttnConfig("C1", 1, 12, 512), configs.mask_c1, "two_rows", 48),      # S 512: 8 query blocks
+    ("C2", configs.C2, configs.mask_c2, "key_split", 768),                               # 3.0 per CU, 16 query blocks
+    ("C4", configs.C4, configs.mask_c4, "two_rows", 1024),                               # 4.0 per CU
+    ("C5", configs.AttnConfig("C5", 4, 16, 2048), configs.mask_c5, "two_rows", 1024),
+])
+def test_launch_form_of_baseline_workloads(name, cfg, mask_fn, form, groups):
+    lut = _lut(mask_fn(cfg.seq))
+    sel = selector.select_operator(selector.GPUParams(), lut[6], cfg.batch, cfg.seq, cfg.heads)
+    assert sel.operator == "block-wise"
+    assert sel.launch_form == form
+    assert sel.groups_per_cu == pytest.approx(groups / 256)
+    full, part = configs.BLOCK_COUNTS[name]
+    assert sel.rho == pytest.approx((full + part) / (cfg.seq // 64) ** 2)
+    assert str(sel) == f"block-wise {form} m64n64"
+
+
+def test_dense_and_causal_masks_go_row_wise():
+    gpu = selector.GPUParams()
+    s = 512
+    dense = torch.ones(s, s)
+    assert str(selector.select_operator(gpu, _lut(dense)[6], 2, s, 12)) == "row-wise"
+    causal = torch.tril(torch.ones(s, s))
+    # 36 of 64 tiles: sparse against the square, dense against the triangle the causal predicate visits
+    assert selector.select_operator(gpu, _lut(causal)[6], 2, s, 12).operator == "block-wise"
+    assert selector.select_operator(gpu, _lut(causal)[6], 2, s, 12, is_causal=True).operator == "row-wise"
+    # a banded causal mask stays block-wise either way
+    band = configs.mask_c5(2048)
+    assert selector.select_operator(gpu, _lut(band)[6], 1, 2048, 4, is_causal=True).operator == "block-wise"
+
+
+def test_per_sample_row_pointers_and_errors():
+    mask, _ = configs.mask_c3(4, 512, 256, seed=0)
+    lut = pm.get_sparse_storage_batched(mask.float(), 64, 64)
+    sel = selector.select_operator(selector.GPUParams(), lut[6], 4, 512, 12)
+    assert sel.operator in ("block-wise", "row-wise") and sel.launch_form == "two_rows"
+    with pytest.raises(ValueError):
+        selector.select_operator(selector.GPUParams(), lut[6], 4, 500, 12)
+    with pytest.raises(ValueError):
+        selector.GPUParams("A100")
