@@ -182,6 +182,172 @@ __global__ __launch_bounds__(256) void gemm_bias_act_kernel(const GemmParams p) 
 }
 
 // ------------------------------------------------------------------------------------------
+// Wide form of the same GEMM: tile 256 (tokens) x 128 (features) x 32 (K), 4 waves as 2 x 2,
+// each 128 tokens x 64 features = 4 x 2 MFMA tiles.  A wave reads 6 fragments for 8 MFMAs per
+// k-step (0.75 KB of LDS per MFMA instead of 1 KB) and a workgroup brings in 24 KB per 2.1
+// MFLOP (85 FLOP per byte over the L2 -> LDS path instead of 64).  The K loop is a ring of NS
+// stages filled by direct-to-LDS loads and is software pipelined inside the wave.
+// ------------------------------------------------------------------------------------------
+constexpr int kWTok = 256;
+constexpr int kWFeat = 128;
+
+// 64-byte rows: chunk c of row r sits at position c ^ ((r >> 2) & 3); 16 rows fill 1 KB.
+__device__ __forceinline__ int swz4(int row) { return (row >> 2) & 3; }
+
+// s_waitcnt immediate that waits for the vector-memory counter only (lgkmcnt 15, expcnt 7)
+constexpr int vmcnt_imm(int n) { return (n & 15) | ((n >> 4) << 14) | 0x0F70; }
+
+template <int ACT, int NS>
+__global__ __launch_bounds__(256, NS <= 3 ? 2 : 1) void gemm_bias_act_wide_kernel(const GemmParams p) {
+  constexpr int kK = 32;
+  constexpr int kATile = kWTok * kK * 2, kWTile = kWFeat * kK * 2;   // 16 KB, 8 KB
+  // Ring of NS stages: NS tiles are in flight or in use at any time, so a tile has NS - 1 tile
+  // times to arrive.  (The fragment reads below are asm, so the compiler does not order them
+  // against the direct-to-LDS loads and one array per operand is enough.)
+  __shared__ __attribute__((aligned(1024))) unsigned char a_lds[NS * kATile];
+  __shared__ __attribute__((aligned(1024))) unsigned char w_lds[NS * kWTile];
+
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
+  const int j32 = lane & 31, g = lane >> 5;
+  const int wf = wave >> 1, wt = wave & 1;   // feature half (64), token half (128)
+
+  const int tm = blockIdx.x % p.tiles_m;
+  const int tn = blockIdx.x / p.tiles_m;
+  const int m0 = tm * kWTok, n0 = tn * kWFeat;
+
+  // Loads: one instruction = 16 rows of 64 B.  A tile: 16 instructions (4 per wave), W tile: 8
+  // (2 per wave).  Rows past the edge re-read the last row.  Addresses are a wave-uniform tile
+  // base (advanced along K in scalar registers) plus a 32-bit per-lane byte offset.
+  const int drow = lane >> 2;
+  uint32_t a_off[4], w_off[2];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int trow = 16 * (4 * wave + i) + drow;
+    const int chunk = (lane & 3) ^ swz4(trow);
+    a_off[i] = (uint32_t)min(trow, p.M - 1 - m0) * (uint32_t)(p.lda * 2) + 16 * chunk;
+  }
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int trow = 16 * (2 * wave + i) + drow;
+    const int chunk = (lane & 3) ^ swz4(trow);
+    w_off[i] = (uint32_t)min(trow, p.N - 1 - n0) * (uint32_t)(p.K * 2) + 16 * chunk;
+  }
+  const char* a_base = reinterpret_cast<const char*>(p.A + (int64_t)m0 * p.lda);
+  const char* w_base = reinterpret_cast<const char*>(p.W + (int64_t)n0 * p.K);
+  auto issue = [&](int kt, int stage) {
+    const char* ab = a_base + kt * (kK * 2);
+    const char* wbase = w_base + kt * (kK * 2);
+    lds_byte* ad = (lds_byte*)a_lds + stage * kATile;
+    lds_byte* wd = (lds_byte*)w_lds + stage * kWTile;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      __builtin_amdgcn_global_load_lds((gptr_t*)(ab + a_off[i]), (__attribute__((address_space(3))) void*)(ad + (4 * wave + i) * 1024), 16, 0, 0);
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+      __builtin_amdgcn_global_load_lds((gptr_t*)(wbase + w_off[i]), (__attribute__((address_space(3))) void*)(wd + (2 * wave + i) * 1024), 16, 0, 0);
+  };
+  // fragment read: row (32*t + j32), chunk 2*ks + g of 4, row pitch 64 B
+  int rd[2];
+#pragma unroll
+  for (int ks = 0; ks < 2; ++ks) rd[ks] = j32 * 64 + (((2 * ks + g) ^ swz4(j32)) << 4);
+
+  floatx16 acc[2][4];   // [feature tile ni][token tile mi]
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+  // Fragment reads are written as asm: the compiler orders LDS reads it can see after every
+  // direct-to-LDS load it cannot prove disjoint, which drains the ring.  The ring's own
+  // counter waits cover that dependency; the LDS counter is waited on by hand, fenced so that
+  // nothing that uses a fragment can be scheduled above its wait.
+  auto frags = [&](uint32_t wa, uint32_t aa, half8_t (&wbk)[2], half8_t (&xak)[4]) {
+    asm volatile(
+        "ds_read_b128 %0, %6\n\tds_read_b128 %1, %6 offset:2048\n\t"
+        "ds_read_b128 %2, %7\n\tds_read_b128 %3, %7 offset:2048\n\t"
+        "ds_read_b128 %4, %7 offset:4096\n\tds_read_b128 %5, %7 offset:6144"
+        : "=&v"(wbk[0]), "=&v"(wbk[1]), "=&v"(xak[0]), "=&v"(xak[1]), "=&v"(xak[2]), "=&v"(xak[3])
+        : "v"(wa), "v"(aa));
+  };
+  auto lds_wait = [&](int outstanding) {   // 0 or 6 fragment reads may remain in flight
+    __builtin_amdgcn_sched_barrier(0);
+    if (outstanding == 0) __builtin_amdgcn_s_waitcnt(0xC07F);   // lgkmcnt(0)
+    else __builtin_amdgcn_s_waitcnt(0xC67F);                    // lgkmcnt(6)
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  auto mfmas = [&](const half8_t (&wbk)[2], const half8_t (&xak)[4]) {
+#pragma unroll
+    for (int mi = 0; mi < 4; ++mi)
+#pragma unroll
+      for (int ni = 0; ni < 2; ++ni) acc[ni][mi] = mfma32(wbk[ni], xak[mi], acc[ni][mi]);
+  };
+  auto wg_barrier = [&]() {
+    // bare barrier: the fences of __syncthreads() would drain the loads that must stay in flight
+    __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  const uint32_t w_rd = (uint32_t)(uintptr_t)(lds_byte*)w_lds + (uint32_t)(64 * wf) * 64;
+  const uint32_t a_rd = (uint32_t)(uintptr_t)(lds_byte*)a_lds + (uint32_t)(128 * wt) * 64;
+  half8_t xa0[4], wb0[2], xa1[4], wb1[2];   // fragments of k-step 0 / k-step 1 of a tile
+
+  const int nk = p.K / kK;
+#pragma unroll
+  for (int s0 = 0; s0 < NS; ++s0)
+    if (s0 < nk) issue(s0, s0);
+  if (nk >= NS) __builtin_amdgcn_s_waitcnt(vmcnt_imm(6 * (NS - 1)));   // tile 0 landed
+  else __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
+  wg_barrier();
+  frags(w_rd + rd[0], a_rd + rd[0], wb0, xa0);
+  // Tile t: the reads of its second k-step go out before the MFMAs of its first; then tile
+  // t+1 is awaited, the barrier lets tile t's stage be refilled with tile t+NS, and the first
+  // fragments of tile t+1 are read while the MFMAs of tile t's second k-step execute.
+  int cs = 0;   // stage of tile t
+  for (int t = 0; t < nk; ++t) {
+    const int ns = (cs + 1 == NS) ? 0 : cs + 1;
+    frags(w_rd + cs * kWTile + rd[1], a_rd + cs * kATile + rd[1], wb1, xa1);
+    lds_wait(6);
+    mfmas(wb0, xa0);
+    lds_wait(0);
+    if (t + 1 < nk) {
+      // tiles t+1 .. t+NS-1 are outstanding; all but the first may stay in flight
+      if (t + NS - 1 < nk) __builtin_amdgcn_s_waitcnt(vmcnt_imm(6 * (NS - 2)));
+      else __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
+      wg_barrier();
+      if (t + NS < nk) issue(t + NS, cs);
+      frags(w_rd + ns * kWTile + rd[0], a_rd + ns * kATile + rd[0], wb0, xa0);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    mfmas(wb1, xa1);
+    cs = ns;
+  }
+
+  // epilogue: acc[ni][mi][r] = C[m0 + 128wt + 32mi + j32][n0 + 64wf + 32ni + 8(r/4) + 4g + r%4]
+#pragma unroll
+  for (int mi = 0; mi < 4; ++mi) {
+    const int m = m0 + 128 * wt + 32 * mi + j32;
+    if (m >= p.M) continue;
+    half_t* crow = p.C + (int64_t)m * p.ldc;
+#pragma unroll
+    for (int ni = 0; ni < 2; ++ni)
+#pragma unroll
+      for (int q4 = 0; q4 < 4; ++q4) {
+        const int n = n0 + 64 * wf + 32 * ni + 8 * q4 + 4 * g;
+        if (n >= p.N) continue;          // N % 8 == 0: a group of 4 is inside or outside as a whole
+        half4_t bv = {(half_t)0.f, (half_t)0.f, (half_t)0.f, (half_t)0.f};
+        if (p.bias) bv = *reinterpret_cast<const half4_t*>(p.bias + n);
+        half4_t o;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) o[e] = (half_t)activate<ACT>(acc[ni][mi][4 * q4 + e] + (float)bv[e]);
+        *reinterpret_cast<half4_t*>(crow + n) = o;
+      }
+  }
+}
+
+// ------------------------------------------------------------------------------------------
 // C[M,N] = LN(A @ Wt^T + bias + residual) * gamma + beta, N = 256 * NC, one workgroup of 8
 // waves per 64 token rows; wave w owns features [32*NC*w, 32*NC*(w+1)).  K tile = 32.
 // ------------------------------------------------------------------------------------------
@@ -193,9 +359,6 @@ struct LnGemmParams {
 
 constexpr int kLM = 64;    // token rows per workgroup
 constexpr int kLK = 32;    // K per tile: rows of 64 B, 4 chunks of 16 B
-
-// 64-byte rows: chunk c of row r sits at position c ^ ((r >> 2) & 3); 16 rows fill 1 KB.
-__device__ __forceinline__ int swz4(int row) { return (row >> 2) & 3; }
 
 template <int NC>
 __global__ __launch_bounds__(512) void gemm_bias_res_ln_kernel(const LnGemmParams p) {
@@ -353,6 +516,14 @@ __global__ __launch_bounds__(512) void gemm_bias_res_ln_kernel(const LnGemmParam
   }
 }
 
+// Which form runs: the wide one when its grid has at least this many workgroups (three per
+// compute unit of an MI355X).  Measured: 10-15 % faster there (BERT-large layer shapes at 8192
+// tokens: 686 vs 610, 655 vs 561, 765 vs 729 TFLOP/s), equal at 768 workgroups with K = 768,
+// slower below (its 256-token tiles leave compute units idle on small grids).  Three ring
+// stages: deeper rings (one workgroup per compute unit) measured no faster.
+constexpr int kWideStages = 3;
+constexpr int kWideMinGroups = 768;
+
 }  // namespace
 
 extern "C" int stof_gemm_bias_act(const void* A, const void* Wt, const void* bias, void* C,
@@ -367,9 +538,22 @@ extern "C" int stof_gemm_bias_act(const void* A, const void* Wt, const void* bia
   GemmParams p;
   p.A = (const half_t*)A; p.W = (const half_t*)Wt; p.bias = (const half_t*)bias; p.C = (half_t*)C;
   p.M = (int)M; p.N = (int)N; p.K = (int)K; p.lda = (int)lda; p.ldc = (int)ldc;
+  hipStream_t st = (hipStream_t)stream;
+  const int64_t wide_groups = ((M + kWTok - 1) / kWTok) * ((N + kWFeat - 1) / kWFeat);
+  if (wide_groups >= kWideMinGroups) {
+    p.tiles_m = (int)((M + kWTok - 1) / kWTok); p.tiles_n = (int)((N + kWFeat - 1) / kWFeat);
+    const dim3 grid((unsigned)(p.tiles_m * p.tiles_n)), block(256);
+    switch (act) {
+      case STOF_ACT_NONE: hipLaunchKernelGGL((gemm_bias_act_wide_kernel<STOF_ACT_NONE, kWideStages>), grid, block, 0, st, p); break;
+      case STOF_ACT_GELU_ERF: hipLaunchKernelGGL((gemm_bias_act_wide_kernel<STOF_ACT_GELU_ERF, kWideStages>), grid, block, 0, st, p); break;
+      case STOF_ACT_GELU_TANH: hipLaunchKernelGGL((gemm_bias_act_wide_kernel<STOF_ACT_GELU_TANH, kWideStages>), grid, block, 0, st, p); break;
+      case STOF_ACT_RELU: hipLaunchKernelGGL((gemm_bias_act_wide_kernel<STOF_ACT_RELU, kWideStages>), grid, block, 0, st, p); break;
+      default: return STOF_ERR_UNSUPPORTED;
+    }
+    return stof_check_launch();
+  }
   p.tiles_m = (int)((M + kGT - 1) / kGT); p.tiles_n = (int)((N + kGT - 1) / kGT);
   const dim3 grid((unsigned)(p.tiles_m * p.tiles_n)), block(256);
-  hipStream_t st = (hipStream_t)stream;
   switch (act) {
     case STOF_ACT_NONE: hipLaunchKernelGGL(gemm_bias_act_kernel<STOF_ACT_NONE>, grid, block, 0, st, p); break;
     case STOF_ACT_GELU_ERF: hipLaunchKernelGGL(gemm_bias_act_kernel<STOF_ACT_GELU_ERF>, grid, block, 0, st, p); break;

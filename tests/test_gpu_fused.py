@@ -28,7 +28,11 @@ def _rand(*shape, seed=0, scale=1.0):
 
 # ---- GEMM + bias + activation -----------------------------------------------------------------
 
-@pytest.mark.parametrize("M,N,K", [(8192, 3072, 768), (300, 768, 3072), (64, 2304, 768), (1, 8, 64), (129, 136, 128)])
+# (8192, 3072, 768), (8155, 3080, 64) and (8292, 3072, 192) run the wide 256 x 128 form (grids of 768+
+# workgroups): full tiles, ragged token / feature edges with fewer K tiles than ring stages, and a
+# ragged token edge with a K loop that wraps the ring; the others run the 128 x 128 form.
+@pytest.mark.parametrize("M,N,K", [(8192, 3072, 768), (8155, 3080, 64), (8292, 3072, 192), (300, 768, 3072), (64, 2304, 768),
+                                   (1, 8, 64), (129, 136, 128)])
 @pytest.mark.parametrize("act", ["none", "gelu", "gelu_tanh", "relu"])
 def test_gemm_bias_act(M, N, K, act):
     print(f"gemm M{M} N{N} K{K} {act}", flush=True)
@@ -43,6 +47,10 @@ def test_gemm_strided_rows_and_no_bias():
     W = _rand(128, 72, seed=5, scale=0.1)
     got = fused.gemm_bias_act(xs, fused.pack_weight(W.cuda()), None, "none")
     _close(got, x[:, :128].float() @ W.float(), "strided")
+    big = _rand(8192, 320, seed=15)               # wide form, row pitch 320, K = 256
+    Wb = _rand(256, 3072, seed=16, scale=0.05)
+    _close(fused.gemm_bias_act(big.cuda()[:, :256], fused.pack_weight(Wb.cuda()), None, "none"),
+           big[:, :256].float() @ Wb.float(), "strided, wide form")
     ident = torch.eye(64).half()                  # closed form: W = I returns the input
     _close(fused.gemm_bias_act(x.cuda()[:, :64].contiguous(), ident.cuda(), None, "none"), x[:, :64], "identity")
 
