@@ -404,12 +404,14 @@ __global__ __launch_bounds__(128 * ROWS * KS, KS == 2 ? 5 : 4) void block_attn_f
 
   Step cur = next_step();
   if (cur.valid) issue_tile(cur.col, (lds_byte*)k_lds0, (lds_byte*)v_lds0);
-  while (cur.valid) {
+  while (cur.valid) {   // single exit: an early exit between the two steps makes the compiler copy the accumulators
     Step nxt = next_step();
     step(cur, nxt, (const lds_byte*)k_lds0, (const lds_byte*)v_lds0, (lds_byte*)k_lds1, (lds_byte*)v_lds1);
-    if (!nxt.valid) break;
-    cur = next_step();
-    step(nxt, cur, (const lds_byte*)k_lds1, (const lds_byte*)v_lds1, (lds_byte*)k_lds0, (lds_byte*)v_lds0);
+    cur = nxt;
+    if (nxt.valid) {
+      cur = next_step();
+      step(nxt, cur, (const lds_byte*)k_lds1, (const lds_byte*)v_lds1, (lds_byte*)k_lds0, (lds_byte*)v_lds0);
+    }
   }
 
   // ---- key split: the waves of the second key half hand their (max, sum, O) to the waves of

@@ -152,11 +152,12 @@ __global__ __launch_bounds__(256) void gemm_bias_act_kernel(const GemmParams p) 
     __syncthreads();
     if (kt + 1 < nk) issue(kt + 1, (lds_byte*)a_lds1, (lds_byte*)w_lds1);
     compute((const lds_byte*)a_lds0, (const lds_byte*)w_lds0);
-    if (kt + 1 >= nk) break;
-    __builtin_amdgcn_s_waitcnt(0x0F70);
-    __syncthreads();
-    if (kt + 2 < nk) issue(kt + 2, (lds_byte*)a_lds0, (lds_byte*)w_lds0);
-    compute((const lds_byte*)a_lds1, (const lds_byte*)w_lds1);
+    if (kt + 1 < nk) {   // (no early exit from the loop: a second exit makes the compiler copy the accumulators)
+      __builtin_amdgcn_s_waitcnt(0x0F70);
+      __syncthreads();
+      if (kt + 2 < nk) issue(kt + 2, (lds_byte*)a_lds0, (lds_byte*)w_lds0);
+      compute((const lds_byte*)a_lds1, (const lds_byte*)w_lds1);
+    }
   }
 
   // epilogue: acc[ni][mi][r] = C[m0 + 64wm + 32mi + j32][n0 + 64wn + 32ni + 8(r/4) + 4g + r%4]
@@ -433,11 +434,12 @@ __global__ __launch_bounds__(512) void gemm_bias_res_ln_kernel(const LnGemmParam
     __syncthreads();
     if (kt + 1 < nk) issue(kt + 1, (lds_byte*)w_lds1, (lds_byte*)a_lds1);
     compute((const lds_byte*)w_lds0, (const lds_byte*)a_lds0);
-    if (kt + 1 >= nk) break;
-    __builtin_amdgcn_s_waitcnt(0x0F70);
-    __syncthreads();
-    if (kt + 2 < nk) issue(kt + 2, (lds_byte*)w_lds0, (lds_byte*)a_lds0);
-    compute((const lds_byte*)w_lds1, (const lds_byte*)a_lds1);
+    if (kt + 1 < nk) {   // (no early exit from the loop: a second exit makes the compiler copy the accumulators)
+      __builtin_amdgcn_s_waitcnt(0x0F70);
+      __syncthreads();
+      if (kt + 2 < nk) issue(kt + 2, (lds_byte*)w_lds0, (lds_byte*)a_lds0);
+      compute((const lds_byte*)w_lds1, (const lds_byte*)a_lds1);
+    }
   }
 
   // ---- epilogue.  acc[ni][mi][r] = X[m0 + 32mi + j32][nb + 32ni + 8(r/4) + 4g + r%4],
