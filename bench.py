@@ -14,8 +14,9 @@ the roofline figure uses.  One JSON line is printed:
   roofline     the attention kernel against the MI355X dense fp16 MFMA peak (2.5 PFLOP/s)
   cpu_baseline the reference's PyTorch-native dense attention (restated in oracle/) timed on
                this machine's host cores on the same workload, in the same unit
-  also         the other single-GPU workloads: C4 (S4096 long-sequence MHA), the C3 BERT-base
-               encoder layer (fused vs PyTorch-ROCm eager, ms) and the HBM-bound kernels
+  also         the other workloads: C1 (S512, with the host fp32 reference), C4 (S4096 long-sequence
+               MHA), the C3 BERT-base encoder layer and the C5 24-layer stack (fused vs PyTorch-ROCm
+               eager, ms, per-stage breakdown for C3), the HBM-bound kernels and the LUT build
 """
 import argparse
 import json
@@ -116,12 +117,55 @@ def bench_layer_c3(steps, warmup):
         out[fusion + "_ms"], _ = time_region(lambda: layer(x, lut), steps, warmup)
     with torch.no_grad():
         out["eager_ms"], _ = time_region(lambda: eager_layer(x, w, maskg, cfg.heads, cfg.eps), max(steps // 4, 5), 5)
+    layer = EncoderLayer(w, cfg.heads, eps=cfg.eps, ln_fusion="split")
+    out["stages_ms"] = {name: time_region(fn, steps, warmup)[1] for name, fn in layer.stages(x, lut)}
+    out["layer_ms_without_qkv_gemm"] = sum(v for k, v in out["stages_ms"].items() if k != "qkv_gemm")
     best = min(out["fused_ms"], out["split_ms"])
     out["layer_ms"] = best
     out["speedup_vs_eager"] = out["eager_ms"] / best
     flop = 2 * cfg.batch * cfg.seq * cfg.hidden * (3 * cfg.hidden + cfg.hidden + 2 * cfg.ffn)
     out["gemm_tflops_at_layer_ms"] = flop / best / 1e9
     return out
+
+
+def bench_c1(steps, warmup, with_cpu):
+    """C1 (B1 H12 S512, causal window 128 + first 64 tokens global): the GPU kernel on the fp16
+    inputs and the reference's dense attention in fp32 on the host, as the config specifies."""
+    from stof import configs
+    cfg = configs.AttnConfig("C1", 1, 12, 512)
+    r = bench_attn(cfg, configs.mask_c1, steps, warmup)
+    out = {"gpu_kernel_ms": r["kernel_ms"], "gpu_tflops": r["tflops_kernel"], "active_blocks": r["active_blocks"]}
+    if with_cpu:
+        c = cpu_baseline_attn(cfg, configs.mask_c1, r["active_blocks"], budget_s=3.0, max_iters=50)
+        out["cpu_fp32_ms"] = c["ms_per_step"]; out["cpu_tflops"] = c["value"]; out["cpu_cores"] = c["cores"]
+    return out
+
+
+def bench_stack_c5(steps, warmup):
+    """C5: 24 post-LN encoder layers, hidden 1024, 16 heads, FFN 4096, B4 S2048, causal window
+    256 + first 64 tokens global; whole stack, fused vs PyTorch-ROCm eager."""
+    from stof import configs, masks as pm
+    from stof.layer import EncoderStack, eager_layer
+    cfg = configs.C5
+    ws = [{k: v.cuda() for k, v in configs.layer_weights(cfg.hidden, cfg.ffn, seed=i).items()} for i in range(cfg.layers)]
+    x = configs.layer_input(cfg, seed=1, device="cuda")
+    mask = configs.mask_c5(cfg.seq)
+    lut = pm.get_sparse_storage(mask.float()[None].cuda(), 64, 64)[1:]
+    stack = EncoderStack(ws, cfg.heads, eps=cfg.eps)
+    stack(x, lut)
+    ms, _ = time_region(lambda: stack(x, lut), steps, warmup)
+    maskg = mask.half()[None].cuda()
+
+    def eager():
+        h = x
+        for w in ws:
+            h = eager_layer(h, w, maskg, cfg.heads, cfg.eps)
+        return h
+    with torch.no_grad():
+        eager_ms, _ = time_region(eager, max(steps // 2, 3), 2)
+    gemm_flop = 2 * cfg.batch * cfg.seq * cfg.hidden * (3 * cfg.hidden + cfg.hidden + 2 * cfg.ffn) * cfg.layers
+    return {"stack_ms": ms, "ms_per_layer": ms / cfg.layers, "eager_ms": eager_ms, "speedup_vs_eager": eager_ms / ms,
+            "gemm_tflops_at_stack_ms": gemm_flop / ms / 1e9, "layers": cfg.layers}
 
 
 def bench_hbm_kernels(steps, warmup):
@@ -226,7 +270,9 @@ def main():
         c4b = bench_attn(big, configs.mask_c4, max(args.steps // 4, 10), 5)
         also["C4_mask_B16_H16"] = {"tflops": c4b["tflops_kernel"], "frac_mfma_peak": c4b["tflops_kernel"] / PEAK_FP16_TFLOPS,
                                    "kernel_ms": c4b["kernel_ms"]}
+        also["C1_mha_S512"] = bench_c1(args.steps, args.warmup, not args.no_cpu)
         also["C3_bert_base_layer"] = bench_layer_c3(max(args.steps // 4, 20), 10)
+        also["C5_stack_24_layers"] = bench_stack_c5(max(args.steps // 20, 5), 2)
         also["hbm_bound"] = bench_hbm_kernels(args.steps, args.warmup)
         also["lut_build"] = bench_lut_build(not args.no_cpu)
         line["also"] = also

@@ -42,8 +42,9 @@ class EncoderLayer:
     def _fuse(self, M):
         if self.ln_fusion in ("fused", "split"):
             return self.ln_fusion == "fused"
-        # One workgroup per 64 rows: below ~2 workgroups per CU the fused kernel cannot fill
-        # the 256 CUs, and at hidden 1024 its register budget is exhausted.
+        # One workgroup per 64 rows streams the whole weight matrix: below ~2 workgroups per CU
+        # the fused kernel cannot fill the 256 CUs and the tiled GEMM + LayerNorm kernel is
+        # faster (measured at M = 8192 for hidden 768 and 1024).
         return self.hidden <= 768 and M >= 64 * 256
 
     def _gemm_ln(self, x, Wt, bias, residual, gamma, beta):
@@ -65,6 +66,26 @@ class EncoderLayer:
         return self._gemm_ln(f, self.W2, self.b2, h, self.g2, self.be2)
 
     __call__ = forward
+
+    def stages(self, x, lut, block=64):
+        """The five launches of ``forward`` as (name, thunk) pairs on precomputed inputs, so each
+        can be timed on its own (the reference's layer has no QKV projection,
+        src/benchmk_end2end.py:37: its figure is the sum without "qkv_gemm")."""
+        B, S, D = x.shape
+        H = self.n_heads
+        hd = D // H
+        qkv = fused.gemm_bias_act(x, self.Wqkv, self.bqkv, "none")
+        q, k, v = (qkv[..., t * D:(t + 1) * D].view(B, S, H, hd).permute(0, 2, 1, 3) for t in range(3))
+        attn = block_attn(q, k, v, lut, block, block, out_layout="bshd")
+        h = self._gemm_ln(attn, self.Wo, self.bo, x, self.g1, self.be1)
+        f = fused.gemm_bias_act(h, self.W1, self.b1, self.act)
+        return [
+            ("qkv_gemm", lambda: fused.gemm_bias_act(x, self.Wqkv, self.bqkv, "none")),
+            ("attention", lambda: block_attn(q, k, v, lut, block, block, out_layout="bshd")),
+            ("out_proj_ln", lambda: self._gemm_ln(attn, self.Wo, self.bo, x, self.g1, self.be1)),
+            ("ffn1_gelu", lambda: fused.gemm_bias_act(h, self.W1, self.b1, self.act)),
+            ("ffn2_ln", lambda: self._gemm_ln(f, self.W2, self.b2, h, self.g2, self.be2)),
+        ]
 
 
 class EncoderStack:
