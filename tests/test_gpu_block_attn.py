@@ -166,6 +166,27 @@ def test_random_block_masks(seed):
     _close(got, torch.from_numpy(blk), f"random seed {seed} (block oracle)")
 
 
+@pytest.mark.parametrize("S", [64, 192])
+def test_single_and_odd_query_block_counts(S):
+    """One query block, and a block count that leaves the last two-row workgroup half empty."""
+    g = torch.Generator().manual_seed(S)
+    mask = (torch.rand(S, S, generator=g) < 0.6).float()
+    mask[:, :64] = 1                                  # a full tile in every row
+    q, k, v = _inputs(2, 3, S, seed=8)
+    _close(_run(q, k, v, mask), _oracle(q, k, v, mask), f"S {S}")
+
+
+def test_long_sequence_walks_several_column_windows():
+    """S 8192 = 128 key blocks: the kernel walks a LUT row in windows of 64 key blocks, so rows
+    here span two windows, with partial tiles in both and rows that skip the first window."""
+    S = 8192
+    i = torch.arange(S)[:, None]; j = torch.arange(S)[None, :]
+    mask = (((i - j) >= 0) & ((i - j) < 300)) | ((j <= i) & ((j // 64) % 37 == 3)) | ((i < 64) & (j >= 4500) & (j < 4700))
+    q, k, v = _inputs(1, 2, S, seed=9)
+    got = _run(q, k, v, mask.float())
+    _close(got, _oracle(q, k, v, mask.float()), "S 8192")
+
+
 def test_large_logits_no_overflow():
     """|score| of several hundred: the max-subtracted softmax must stay finite."""
     q, k, v = _inputs(1, 2, 256, seed=6, scale=6.0)
