@@ -224,7 +224,9 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--no-extras", action="store_true", help="skip C4 / C3 layer / HBM-bound kernels")
+    ap.add_argument("--no-extras", action="store_true", help="skip everything but the C2 attention step")
+    ap.add_argument("--extras", default="c1,c4,c4big,c3,c5,hbm,lut",
+                    help="comma-separated subset of the extra workloads to run (for profiling one kind of kernel)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run one plain device copy of 256 MiB, so that a counter run of this "
@@ -263,18 +265,26 @@ def main():
         line["cpu_baseline"] = cpu_baseline_attn(configs.C2, configs.mask_c2, c2["active_blocks"])
     if not args.no_extras:
         also = {}
-        c4 = bench_attn(configs.C4, configs.mask_c4, args.steps, args.warmup)
-        also["C4_mha_S4096"] = {"tflops": c4["tflops_kernel"], "frac_mfma_peak": c4["tflops_kernel"] / PEAK_FP16_TFLOPS,
-                                "kernel_ms": c4["kernel_ms"], "active_blocks": c4["active_blocks"]}
-        big = configs.AttnConfig("C4x8", 16, 16, 4096)
-        c4b = bench_attn(big, configs.mask_c4, max(args.steps // 4, 10), 5)
-        also["C4_mask_B16_H16"] = {"tflops": c4b["tflops_kernel"], "frac_mfma_peak": c4b["tflops_kernel"] / PEAK_FP16_TFLOPS,
-                                   "kernel_ms": c4b["kernel_ms"]}
-        also["C1_mha_S512"] = bench_c1(args.steps, args.warmup, not args.no_cpu)
-        also["C3_bert_base_layer"] = bench_layer_c3(max(args.steps // 4, 20), 10)
-        also["C5_stack_24_layers"] = bench_stack_c5(max(args.steps // 20, 5), 2)
-        also["hbm_bound"] = bench_hbm_kernels(args.steps, args.warmup)
-        also["lut_build"] = bench_lut_build(not args.no_cpu)
+        want = set(args.extras.split(","))
+        if "c4" in want:
+            c4 = bench_attn(configs.C4, configs.mask_c4, args.steps, args.warmup)
+            also["C4_mha_S4096"] = {"tflops": c4["tflops_kernel"], "frac_mfma_peak": c4["tflops_kernel"] / PEAK_FP16_TFLOPS,
+                                    "kernel_ms": c4["kernel_ms"], "active_blocks": c4["active_blocks"]}
+        if "c4big" in want:
+            big = configs.AttnConfig("C4x8", 16, 16, 4096)
+            c4b = bench_attn(big, configs.mask_c4, max(args.steps // 4, 10), 5)
+            also["C4_mask_B16_H16"] = {"tflops": c4b["tflops_kernel"], "frac_mfma_peak": c4b["tflops_kernel"] / PEAK_FP16_TFLOPS,
+                                       "kernel_ms": c4b["kernel_ms"]}
+        if "c1" in want:
+            also["C1_mha_S512"] = bench_c1(args.steps, args.warmup, not args.no_cpu)
+        if "c3" in want:
+            also["C3_bert_base_layer"] = bench_layer_c3(max(args.steps // 4, 20), 10)
+        if "c5" in want:
+            also["C5_stack_24_layers"] = bench_stack_c5(max(args.steps // 20, 5), 2)
+        if "hbm" in want:
+            also["hbm_bound"] = bench_hbm_kernels(args.steps, args.warmup)
+        if "lut" in want:
+            also["lut_build"] = bench_lut_build(not args.no_cpu)
         line["also"] = also
     print(json.dumps(line))
 
