@@ -84,8 +84,9 @@ const char* stof_status_string(int status);
  * sample b uses row pointers at offset b*lut_batch_stride, whose values are absolute
  * offsets into the (concatenated) column lists and bitmask slots.
  *
- * Supported: D == 64, block_m == block_n == 64, S % 64 == 0.  num_warps of the
- * reference launcher has no per-call counterpart: see stof_attn_set_launch_form.
+ * Supported: D == 64, block_m == block_n == 64, S % 64 == 0 (the Python operator re-tiles LUTs
+ * built with other block sizes to 64 x 64 before it calls this).  num_warps of the reference
+ * launcher has no per-call counterpart: see stof_attn_set_launch_form.
  */
 int stof_block_attn_fwd(
     const void* q, const void* k, const void* v, void* out,

@@ -117,6 +117,34 @@ def _check_lut_order(lrp, lci, prp, pci, n_cols):
         pass
 
 
+_LUT64_ATTR = "_stof_lut_at_64"
+
+
+def _lut_at_64(lut, S, block_m, block_n):
+    """The same mask described with 64 x 64 blocks, for a LUT built with another block size
+    (the reference's kernels cover BLOCK_M / BLOCK_N of 16..128,
+    src/ops/src/block_attn_mask_cuda.cu:6064-6322; the kernel here has one tile shape).  The
+    LUT is expanded to the dense 0/1 mask it encodes and classified again; the attention
+    result depends on the mask only, so this changes nothing but the tiling.  Done once per
+    LUT (kept on the LOAD column tensor, keyed by the tensors' content versions)."""
+    from . import masks as pm
+    frp, fci, prp, pci, pbm, lrp, lci = lut
+    key = (lci._version, pci._version, lrp._version, prp._version, fci._version, frp._version, pbm._version, block_m, block_n)
+    cached = getattr(lci, _LUT64_ATTR, None)
+    if cached is not None and cached[0] == key:
+        return cached[1]
+    _require(lrp.dim() == 1, "per-sample LUTs are supported with 64 x 64 blocks only")
+    _require(tuple(pbm.shape[-2:]) == (block_m, block_n) or int(prp.reshape(-1)[-1]) == 0,
+             f"part_block_mask must hold {block_m} x {block_n} blocks")
+    dense = pm.expand_sparse_storage((None, frp, fci, prp, pci, pbm, lrp, lci), S, block_m, block_n)
+    lut64 = tuple(pm.get_sparse_storage(dense[None], 64, 64)[1:])
+    try:
+        setattr(lci, _LUT64_ATTR, (key, lut64))
+    except AttributeError:
+        pass
+    return lut64
+
+
 def _check_i32(name, t, device):
     _require(t.dtype == torch.int32, f"{name} must be int32, got {t.dtype}")
     _require(t.device == device, f"{name} is on {t.device}, expected {device}")
@@ -155,6 +183,10 @@ def block_attn(q, k, v, lut, block_m=64, block_n=64, out=None, out_layout="bhsd"
                  f"row pointers must have {nq + 1} entries for seq_len {S}, block_m {block_m}")
         lut_bs = 0
     _check_lut_order(lrp, lci, prp, pci, S // block_n)
+    if (block_m, block_n) != (64, 64):
+        _require(S % 64 == 0, f"seq_len {S} must be a multiple of 64")
+        frp, fci, prp, pci, pbm, lrp, lci = _lut_at_64((frp, fci, prp, pci, pbm, lrp, lci), S, block_m, block_n)
+        block_m = block_n = 64
     bits = _packed_partial_bits(pbm)
     if out is None:
         if out_layout == "bhsd":
