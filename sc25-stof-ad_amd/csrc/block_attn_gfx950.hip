@@ -180,13 +180,15 @@ __global__ __launch_bounds__(128 * ROWS * KS, KS == 2 ? 5 : 4) void block_attn_f
   // DMA: a tile is 8 instructions of 1 KB (8 rows of 128 B); wave w issues instructions
   // kDma*w .. kDma*w + kDma - 1 for K and for V.  Lane l lands at (row 8*ii + l/8, chunk
   // position l%8) and therefore fetches global chunk (l%8) ^ swz(row).
-  int k_src[kDma], v_src[kDma];
+  // Per-lane BYTE offsets inside a tile, unsigned 32-bit: the load then takes the tile's
+  // wave-uniform base in scalar registers and this as its vector offset.
+  uint32_t k_src[kDma], v_src[kDma];
 #pragma unroll
   for (int i = 0; i < kDma; ++i) {
     const int trow = 8 * (kDma * wave + i) + (lane >> 3);
     const int chunk = (lane & 7) ^ swz(trow);
-    k_src[i] = trow * (int)p.ks[2] + 8 * chunk;
-    v_src[i] = trow * (int)p.vs[2] + 8 * chunk;
+    k_src[i] = (uint32_t)trow * (uint32_t)(p.ks[2] * 2) + 16 * chunk;
+    v_src[i] = (uint32_t)trow * (uint32_t)(p.vs[2] * 2) + 16 * chunk;
   }
   // K fragment (A operand of S^T): row = key 32*mt + j32, chunk 2*ks + g.
   int k_rd[4];
@@ -218,8 +220,8 @@ __global__ __launch_bounds__(128 * ROWS * KS, KS == 2 ? 5 : 4) void block_attn_f
   float l_run = 0.f;
 
   auto issue_tile = [&](int col, lds_byte* kdst, lds_byte* vdst) {
-    const half_t* kt = kb + (int64_t)col * kBN * p.ks[2];
-    const half_t* vt = vb + (int64_t)col * kBN * p.vs[2];
+    const char* kt = reinterpret_cast<const char*>(kb + (int64_t)col * kBN * p.ks[2]);
+    const char* vt = reinterpret_cast<const char*>(vb + (int64_t)col * kBN * p.vs[2]);
     lds_byte* kd = kdst + (kDma * wave) * 1024;
     lds_byte* vd = vdst + (kDma * wave) * 1024;
 #pragma unroll
