@@ -168,6 +168,27 @@ def bench_stack_c5(steps, warmup):
             "gemm_tflops_at_stack_ms": gemm_flop / ms / 1e9, "layers": cfg.layers}
 
 
+def bench_dense_vs_sdpa(steps, warmup):
+    """The same kernel on unmasked and causal attention (row-wise front-end: key blocks from index
+    arithmetic, no LUT) next to PyTorch-ROCm's fused scaled_dot_product_attention, B16 H16 S4096:
+    what the tile engine reaches without mask irregularity, and what the vendor path reaches."""
+    import torch.nn.functional as F
+    from stof import configs
+    from stof.ops import rowwise_attn_full_op
+    cfg = configs.AttnConfig("dense", 16, 16, 4096)
+    q, k, v = configs.qkv(cfg, seed=0, device="cuda")
+    n = cfg.seq // 64
+    out = {}
+    for causal in (False, True):
+        blocks = n * (n + 1) // 2 if causal else n * n
+        flop = FLOP_PER_BLOCK * cfg.batch * cfg.heads * blocks
+        _, ms = time_region(lambda: rowwise_attn_full_op(q, k, v, causal), steps, warmup)
+        _, ms_ref = time_region(lambda: F.scaled_dot_product_attention(q, k, v, is_causal=causal), steps, warmup)
+        out["causal" if causal else "full"] = {"kernel_ms": ms, "tflops": flop / ms / 1e9, "frac_mfma_peak": flop / ms / 1e9 / PEAK_FP16_TFLOPS,
+                                               "torch_sdpa_ms": ms_ref, "torch_sdpa_tflops": flop / ms_ref / 1e9}
+    return out
+
+
 def bench_hbm_kernels(steps, warmup):
     """HBM-bound kernels: bias+residual+LayerNorm (3 x M x N x 2 bytes) at the C3 size and at a
     size large enough to leave the launch-latency regime, and the fp16 mask -> bit-row pack."""
@@ -225,7 +246,7 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-extras", action="store_true", help="skip everything but the C2 attention step")
-    ap.add_argument("--extras", default="c1,c4,c4big,c3,c5,hbm,lut",
+    ap.add_argument("--extras", default="c1,c4,c4big,dense,c3,c5,hbm,lut",
                     help="comma-separated subset of the extra workloads to run (for profiling one kind of kernel)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--copy-probe", action="store_true",
@@ -275,6 +296,8 @@ def main():
             c4b = bench_attn(big, configs.mask_c4, max(args.steps // 4, 10), 5)
             also["C4_mask_B16_H16"] = {"tflops": c4b["tflops_kernel"], "frac_mfma_peak": c4b["tflops_kernel"] / PEAK_FP16_TFLOPS,
                                        "kernel_ms": c4b["kernel_ms"]}
+        if "dense" in want:
+            also["dense_S4096_B16_H16_vs_torch_sdpa"] = bench_dense_vs_sdpa(max(args.steps // 10, 10), 3)
         if "c1" in want:
             also["C1_mha_S512"] = bench_c1(args.steps, args.warmup, not args.no_cpu)
         if "c3" in want:
