@@ -4,12 +4,14 @@
 // (src/ops/src/block_attn_mask_cuda.cu:269-6322) with one kernel designed around the
 // CDNA4 wavefront:
 //
-//  * a workgroup of four 64-lane wavefronts owns TWO adjacent 64-row query blocks (two LUT
-//    rows); each wave keeps 32 queries in registers.  The two rows' key-block lists are
-//    merged on the fly: a key block wanted by both rows is brought into LDS once and used
-//    by all four waves, one wanted by a single row is skipped by the other row's waves.
-//    This halves the L2 -> LDS traffic per unit of MFMA work, which is what bounds the
-//    kernel at head size 64.  S, P and O never touch LDS;
+//  * a wave keeps 32 queries in registers; S, P and O never touch LDS.  A workgroup of four
+//    64-lane wavefronts runs in one of two forms.  Large grids: it owns TWO adjacent 64-row
+//    query blocks (two LUT rows) whose key-block lists are merged on the fly; a key block
+//    wanted by both rows is brought into LDS once and used by all four waves, one wanted by a
+//    single row is skipped by the other row's waves.  This halves the L2 -> LDS traffic per
+//    unit of MFMA work.  Small grids: it owns ONE query block and the two wave pairs take
+//    the two 32-key halves of every tile, so the chain of key blocks of a long row, which
+//    sets the run time there, takes half as long; partial results are merged through LDS;
 //  * K/V tiles travel HBM/L2 -> LDS with the asynchronous direct-to-LDS loads
 //    (global_load_lds_dwordx4), double buffered: the loads of block t+1 are issued before
 //    the math of block t, no VGPRs are used for staging and one barrier per block suffices;
