@@ -41,6 +41,7 @@ constexpr int kBN = 64;       // keys per block
 constexpr int kTile = kBN * kD * 2;   // bytes of one K or V tile in LDS (8 KB, unpadded)
 constexpr float kMasked = -INFINITY;  // score given to a masked element
 constexpr float kLazy = 8.0f;         // log2 slack before the running max is raised
+constexpr int kPrioStep = 6;          // key blocks of remaining chain per issue-priority level
 
 typedef __attribute__((address_space(3))) unsigned char lds_byte;
 typedef short short4_t __attribute__((ext_vector_type(4)));
@@ -101,17 +102,12 @@ struct RowList {
 // so the chain of key blocks of a long LUT row finishes in half the time; it is used for
 // small grids, where that chain and not throughput sets the run time.
 template <int KIND, int ROWS, int KS>
-__global__ __launch_bounds__(128 * ROWS * KS, KS == 2 ? 5 : 4) void block_attn_fwd_kernel(const AttnParams p) {
+__device__ __forceinline__ void attn_group(const AttnParams& p, const int bh, const int pair,
+                                           unsigned char* k_lds0, unsigned char* k_lds1,
+                                           unsigned char* v_lds0, unsigned char* v_lds1) {
   static_assert(KS == 1 || ROWS == 1, "the key split serves a single query block");
   constexpr int kDma = 4 / (ROWS * KS);   // direct-to-LDS instructions per wave and operand tile (8 per tile)
   constexpr int kMT = 2 / KS;             // 32-key sub-tiles of a key block handled by one wave
-  // Four distinct LDS objects (K and V, two buffers each): the compiler orders LDS reads
-  // after in-flight direct-to-LDS loads per object, so a read of the current buffer does
-  // not wait for the loads that fill the other one.
-  __shared__ __attribute__((aligned(1024))) unsigned char k_lds0[kTile];
-  __shared__ __attribute__((aligned(1024))) unsigned char k_lds1[kTile];
-  __shared__ __attribute__((aligned(1024))) unsigned char v_lds0[kTile];
-  __shared__ __attribute__((aligned(1024))) unsigned char v_lds1[kTile];
 
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int lane = threadIdx.x & 63;
@@ -121,18 +117,6 @@ __global__ __launch_bounds__(128 * ROWS * KS, KS == 2 ? 5 : 4) void block_attn_f
   const int half = wave & 1;                  // which 32 queries of that block
   const int mt0 = KS == 1 ? 0 : wave >> 1;    // first 32-key sub-tile of this wave
 
-  // Workgroups are handed to the 8 XCDs round-robin; give each XCD a contiguous range
-  // of (batch, head, query-block pair) so one head's K/V is read through a single L2.
-  const int wg = blockIdx.x;
-  const int vid = (wg & 7) * p.chunk + (wg >> 3);
-  if (vid >= p.total) return;
-  const int bh = vid / p.nP;
-  // Row length usually grows (causal) or is flat along the sequence.  Workgroups are placed
-  // on CUs round-robin, so consecutive heads walk the sequence in opposite directions: a CU
-  // that receives the longest rows of one head receives the shortest rows of the next.
-  const int pidx = vid - bh * p.nP;
-  const int zig = ((pidx + bh) & 1) ? (pidx >> 1) : p.nP - 1 - (pidx >> 1);   // long, short, long, ...
-  const int pair = zig;
   const int b = bh / p.H;
   const int h = bh - b * p.H;
   const int qi = ROWS * pair + rsel;               // this wave's query block
@@ -168,15 +152,36 @@ __global__ __launch_bounds__(128 * ROWS * KS, KS == 2 ? 5 : 4) void block_attn_f
     }
   }
 
+  // LUT entries of the current window of 64 key blocks: lane l holds entry ptr + l of each row's
+  // LOAD list and of this wave's PART list.  Every list read of a window goes out before the
+  // first is waited for, and window 0 is requested here, AHEAD of the Q loads: the memory
+  // counter retires in order, so the wait for these (L2-resident) entries does not also wait
+  // for Q (HBM), whose latency then overlaps the walk set-up and the first K/V loads.
+  int win_e[ROWS], win_pe = 0x7fffffff;
+  auto fetch_window = [&]() {
+    win_pe = 0x7fffffff;
+#pragma unroll
+    for (int r = 0; r < ROWS; ++r) {
+      win_e[r] = 0x7fffffff;
+      if (KIND == kKindLut) {
+        if (row[r].ptr + lane < row[r].n) win_e[r] = p.lci[row[r].t0 + row[r].ptr + lane];
+        if (r == rsel && row[r].pptr + lane < row[r].np) win_pe = p.pci[row[r].p0 + row[r].pptr + lane];
+      }
+    }
+  };
+  fetch_window();
+  __builtin_amdgcn_sched_barrier(0);
+
   // Q^T as the B operand: lane (n = query j32, k-group g) holds 8 consecutive d per k-step.
+  // (A query block past the end - odd block count, last group - reads the last real block
+  // instead: its row lists are empty and nothing of it is stored.)
   half8_t qf[4];
+  {
+    const half_t* qsrc = q_valid ? qb : qb - (int64_t)kBM * p.qs[2];
 #pragma unroll
-  for (int ks = 0; ks < 4; ++ks) {
-    if (q_valid) qf[ks] = *reinterpret_cast<const half8_t*>(qb + (int64_t)j32 * p.qs[2] + 16 * ks + 8 * g);
-    else
-#pragma unroll
-      for (int e = 0; e < 8; ++e) qf[ks][e] = (half_t)0.f;
+    for (int ks = 0; ks < 4; ++ks) qf[ks] = *reinterpret_cast<const half8_t*>(qsrc + (int64_t)j32 * p.qs[2] + 16 * ks + 8 * g);
   }
+  __builtin_amdgcn_sched_barrier(0);
 
   // ---- per-lane constants of the data movement
   // DMA: a tile is 8 instructions of 1 KB (8 rows of 128 B); wave w issues instructions
@@ -213,6 +218,12 @@ __global__ __launch_bounds__(128 * ROWS * KS, KS == 2 ? 5 : 4) void block_attn_f
       }
   }
 
+  // Key blocks this wave still has to visit (the longer of the group's rows: a lower bound of
+  // the merged walk).  It sets the wave's issue priority at every step - see step().
+  int steps_left = 0;
+#pragma unroll
+  for (int r = 0; r < ROWS; ++r) steps_left = max(steps_left, KIND == kKindLut ? row[r].n : row[r].hi - row[r].lo + 1);
+
   floatx16 oacc[2];   // [d tile]: O^T for this wave's 32 queries
 #pragma unroll
   for (int i = 0; i < 2; ++i)
@@ -241,25 +252,21 @@ __global__ __launch_bounds__(128 * ROWS * KS, KS == 2 ? 5 : 4) void block_attn_f
   // offset of the window plus the population count of the PART set below the block.
   struct Step { int col; int mine; int slot; bool valid; };
   const int n_win = (p.nQ + 63) >> 6;
-  int win = -1;
+  int win = 0;   // window 0 is consumed right below, outside the walk's loop
   uint64_t set_union = 0, set_mine = 0, set_part = 0;
   int part_base = 0;
-  auto load_window = [&](int w) {
+  auto consume_window = [&](int w) {
     set_union = 0; set_mine = 0; set_part = 0;
 #pragma unroll
     for (int r = 0; r < ROWS; ++r) {
       uint64_t m = 0;
       if (KIND == kKindLut) {
-        int e = 0x7fffffff;
-        if (row[r].ptr + lane < row[r].n) e = p.lci[row[r].t0 + row[r].ptr + lane];
-        const int cnt = __builtin_popcountll(__ballot(e < 64 * (w + 1)));
-        for (int j = 0; j < cnt; ++j) m |= 1ull << (__builtin_amdgcn_readlane(e, j) - 64 * w);
+        const int cnt = __builtin_popcountll(__ballot(win_e[r] < 64 * (w + 1)));
+        for (int j = 0; j < cnt; ++j) m |= 1ull << (__builtin_amdgcn_readlane(win_e[r], j) - 64 * w);
         row[r].ptr += cnt;
         if (r == rsel) {
-          int pe = 0x7fffffff;
-          if (row[r].pptr + lane < row[r].np) pe = p.pci[row[r].p0 + row[r].pptr + lane];
-          const int pcnt = __builtin_popcountll(__ballot(pe < 64 * (w + 1)));
-          for (int j = 0; j < pcnt; ++j) set_part |= 1ull << (__builtin_amdgcn_readlane(pe, j) - 64 * w);
+          const int pcnt = __builtin_popcountll(__ballot(win_pe < 64 * (w + 1)));
+          for (int j = 0; j < pcnt; ++j) set_part |= 1ull << (__builtin_amdgcn_readlane(win_pe, j) - 64 * w);
           part_base = row[r].p0 + row[r].pptr;
           row[r].pptr += pcnt;
         }
@@ -271,11 +278,13 @@ __global__ __launch_bounds__(128 * ROWS * KS, KS == 2 ? 5 : 4) void block_attn_f
       if (r == rsel) set_mine = m;
     }
   };
+  consume_window(0);
   auto next_step = [&]() -> Step {
     Step s; s.col = 0; s.mine = 0; s.slot = -1; s.valid = false;
     while (set_union == 0) {
       if (++win >= n_win) return s;
-      load_window(win);
+      fetch_window();
+      consume_window(win);
     }
     const int bit = __builtin_ctzll(set_union);
     set_union &= set_union - 1;
@@ -291,6 +300,18 @@ __global__ __launch_bounds__(128 * ROWS * KS, KS == 2 ? 5 : 4) void block_attn_f
   auto step = [&](const Step cur, const Step nxt, const lds_byte* kt, const lds_byte* vt, lds_byte* kn, lds_byte* vn) {
     // The row mask of a partial tile is fetched first so that its latency hides behind
     // the wait below and no register-returning load is pending across the DMA issue.
+    // Longest remaining chain first.  Among waves of equal priority a SIMD issues from the
+    // oldest, which starves the youngest workgroup of a compute unit until the others are done
+    // and leaves it to finish a long chain alone (measured: the last of four equal chains had
+    // done 6 of 21 steps when the third finished).  Priority by remaining length makes the
+    // chains of a SIMD end together.
+    {
+      const int left = steps_left--;
+      if (left >= 3 * kPrioStep) __builtin_amdgcn_s_setprio(3);
+      else if (left >= 2 * kPrioStep) __builtin_amdgcn_s_setprio(2);
+      else if (left >= kPrioStep) __builtin_amdgcn_s_setprio(1);
+      else __builtin_amdgcn_s_setprio(0);
+    }
     uint64_t bits = ~0ull;
     if (KIND == kKindLut) {
       if (cur.slot >= 0) bits = p.pbits[(int64_t)cur.slot * kBM + 32 * half + j32];
@@ -463,6 +484,39 @@ __global__ __launch_bounds__(128 * ROWS * KS, KS == 2 ? 5 : 4) void block_attn_f
     }
 }
 
+// Workgroups are handed to the 8 XCDs round-robin; give each XCD a contiguous range of
+// (batch, head, group) so one head's K/V is read through a single L2.
+__device__ __forceinline__ int xcd_contiguous_id(const AttnParams& p) {
+  const int wg = blockIdx.x;
+  return (wg & 7) * p.chunk + (wg >> 3);
+}
+
+// Row length usually grows (causal) or is flat along the sequence.  Workgroups are placed on
+// CUs round-robin, so consecutive heads walk the sequence in opposite directions: a CU that
+// receives the longest rows of one head receives the shortest rows of the next.
+__device__ __forceinline__ int zigzag(int pidx, int bh, int n) {
+  return ((pidx + bh) & 1) ? (pidx >> 1) : n - 1 - (pidx >> 1);   // long, short, long, ...
+}
+
+// Four distinct LDS objects (K and V, two buffers each): the compiler orders LDS reads after
+// in-flight direct-to-LDS loads per object, so a read of the current buffer does not wait for
+// the loads that fill the other one.
+#define STOF_ATTN_LDS_TILES                                                     \
+  __shared__ __attribute__((aligned(1024))) unsigned char k_lds0[kTile];        \
+  __shared__ __attribute__((aligned(1024))) unsigned char k_lds1[kTile];        \
+  __shared__ __attribute__((aligned(1024))) unsigned char v_lds0[kTile];        \
+  __shared__ __attribute__((aligned(1024))) unsigned char v_lds1[kTile]
+
+template <int KIND, int ROWS, int KS>
+__global__ __launch_bounds__(128 * ROWS * KS, 4) void block_attn_fwd_kernel(const AttnParams p) {
+  STOF_ATTN_LDS_TILES;
+  const int vid = xcd_contiguous_id(p);
+  if (vid >= p.total) return;
+  const int bh = vid / p.nP;
+  const int pair = zigzag(vid - bh * p.nP, bh, p.nP);
+  attn_group<KIND, ROWS, KS>(p, bh, pair, k_lds0, k_lds1, v_lds0, v_lds1);
+}
+
 // dst[r*(cols/64)+w] bit t = pred(src[r*ld + 64w + t]).
 // Vector form: a lane loads 8 elements (16 B) and forms one byte of the word; the 8 lanes of a
 // word merge their bytes with three lane exchanges and the first of them stores 8 B.  A
@@ -536,8 +590,8 @@ int g_attn_form = kFormAuto;
 constexpr int kKeySplitMaxGroupsPerCu = 3;
 constexpr int kKeySplitMinQueryBlocks = 16;
 
-bool use_key_split(int64_t two_row_groups, int nQ) {
-  if (g_attn_form != kFormAuto) return g_attn_form == kFormKeySplit;
+int pick_form(int64_t two_row_groups, int nQ) {
+  if (g_attn_form != kFormAuto) return g_attn_form;
   static int cus = 0;
   if (cus == 0) {
     int dev = 0, n = 0;
@@ -545,13 +599,14 @@ bool use_key_split(int64_t two_row_groups, int nQ) {
       n = 256;
     cus = n;
   }
-  return nQ >= kKeySplitMinQueryBlocks && two_row_groups <= (int64_t)kKeySplitMaxGroupsPerCu * cus;
+  return (nQ >= kKeySplitMinQueryBlocks && two_row_groups <= (int64_t)kKeySplitMaxGroupsPerCu * cus) ? kFormKeySplit : kFormTwoRows;
 }
 
 template <int KIND>
 void launch_attn(AttnParams& p, int nQ, int64_t bh, hipStream_t stream) {
   const int64_t two_row_groups = (int64_t)((nQ + kRowsPerGroup - 1) / kRowsPerGroup) * bh;
-  if (use_key_split(two_row_groups, nQ)) {
+  const int form = pick_form(two_row_groups, nQ);
+  if (form == kFormKeySplit) {
     p.nP = nQ;
     p.total = (int)(nQ * bh);
     p.chunk = (p.total + 7) / 8;
