@@ -582,12 +582,13 @@ constexpr int kRowsPerGroup = 2;
 enum { kFormAuto = -1, kFormTwoRows = 0, kFormKeySplit = 1 };
 int g_attn_form = kFormAuto;
 
-// Automatic choice: key split when the two-row grid gives a compute unit at most this many
-// workgroups AND the sequence has at least this many query blocks.  Measured on MI355X
-// (B8 H12 S1024, rows of 7..16 key blocks: 37 -> 31 us); at four workgroups per compute unit
-// or with short sequences (S 512) the two forms are within 5 % and the two-row form, which
-// moves half the bytes, is kept.
-constexpr int kKeySplitMaxGroupsPerCu = 3;
+// Automatic choice: key split when the sequence has at least kKeySplitMinQueryBlocks query
+// blocks AND the two-row grid gives a compute unit at most kKeySplitMaxGroupsPerCu workgroups.
+// Four workgroups are resident per compute unit (LDS), and the key split doubles the count:
+// up to two two-row groups per compute unit it still runs as a single round with every chain
+// half as long (B2 H12 S2048 causal: 44 -> 34 us, B4 H12 S1024 sparse: 25 -> 23 us), beyond
+// that it needs a second, partly filled round and loses (three per compute unit: -3 % .. +15 %).
+constexpr int kKeySplitMaxGroupsPerCu = 2;
 constexpr int kKeySplitMinQueryBlocks = 16;
 
 int pick_form(int64_t two_row_groups, int nQ) {

@@ -518,13 +518,16 @@ __global__ __launch_bounds__(512) void gemm_bias_res_ln_kernel(const LnGemmParam
   }
 }
 
-// Which form runs: the wide one when its grid has at least this many workgroups (three per
-// compute unit of an MI355X).  Measured: 10-15 % faster there (BERT-large layer shapes at 8192
-// tokens: 686 vs 610, 655 vs 561, 765 vs 729 TFLOP/s), equal at 768 workgroups with K = 768,
-// slower below (its 256-token tiles leave compute units idle on small grids).  Three ring
-// stages: deeper rings (one workgroup per compute unit) measured no faster.
+// Which form runs: the wide one when its grid has at least kWideMinGroups workgroups (three per
+// compute unit of an MI355X) and K is at least kWideMinK.  Measured at settled clocks, 8192
+// tokens: N 3072 K 1024 721 vs 673 TFLOP/s, N 4096 K 1024 706 vs 648, N 1024 K 4096 882 vs 830,
+// 8192^3 951 vs 864; with K 768 (N 3072: 564 vs 598) its longer ring fill and epilogue per
+// workgroup are not paid back, and on smaller grids its 256-token tiles leave compute units
+// idle.  Three ring stages: deeper rings (one workgroup per compute unit) measured no faster;
+// a 256 x 256 tile with eight waves gained 3-9 % only from N 4096 up and is not built.
 constexpr int kWideStages = 3;
 constexpr int kWideMinGroups = 768;
+constexpr int kWideMinK = 1024;
 
 }  // namespace
 
@@ -542,7 +545,7 @@ extern "C" int stof_gemm_bias_act(const void* A, const void* Wt, const void* bia
   p.M = (int)M; p.N = (int)N; p.K = (int)K; p.lda = (int)lda; p.ldc = (int)ldc;
   hipStream_t st = (hipStream_t)stream;
   const int64_t wide_groups = ((M + kWTok - 1) / kWTok) * ((N + kWFeat - 1) / kWFeat);
-  if (wide_groups >= kWideMinGroups) {
+  if (wide_groups >= kWideMinGroups && K >= kWideMinK) {
     p.tiles_m = (int)((M + kWTok - 1) / kWTok); p.tiles_n = (int)((N + kWFeat - 1) / kWFeat);
     const dim3 grid((unsigned)(p.tiles_m * p.tiles_n)), block(256);
     switch (act) {

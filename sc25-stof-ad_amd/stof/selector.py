@@ -46,7 +46,7 @@ class GPUParams:
         self.lds_per_group = 4 * BLOCK * 64 * 2      # K and V tiles, double buffered: 32 KB
         self.waves_per_group = 4
         # launch-form rule (kKeySplitMaxGroupsPerCu / kKeySplitMinQueryBlocks in the kernel source)
-        self.key_split_max_groups_per_cu = 3
+        self.key_split_max_groups_per_cu = 2
         self.key_split_min_query_blocks = 16
 
 
@@ -91,7 +91,8 @@ def phase2_selection(gpu, seq_len, batch_size, head_num):
     if nq >= gpu.key_split_min_query_blocks and groups <= gpu.key_split_max_groups_per_cu * gpu.cu_count:
         return ("key_split", per_cu,
                 f"{per_cu:.2f} two-row workgroups per compute unit (<= {gpu.key_split_max_groups_per_cu}, "
-                f"{resident} fit): run time is set by the longest chain of key blocks, which the key split halves")
+                f"{resident} fit, so twice as many still run as one round): run time is set by the longest chain "
+                f"of key blocks, which the key split halves")
     if nq < gpu.key_split_min_query_blocks:
         why = f"chains of at most {nq} key blocks are too short for the split to pay"
     else:

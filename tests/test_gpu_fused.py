@@ -28,11 +28,12 @@ def _rand(*shape, seed=0, scale=1.0):
 
 # ---- GEMM + bias + activation -----------------------------------------------------------------
 
-# (8192, 3072, 768), (8155, 3080, 64) and (8292, 3072, 192) run the wide 256 x 128 form (grids of 768+
-# workgroups): full tiles, ragged token / feature edges with fewer K tiles than ring stages, and a
-# ragged token edge with a K loop that wraps the ring; the others run the 128 x 128 form.
-@pytest.mark.parametrize("M,N,K", [(8192, 3072, 768), (8155, 3080, 64), (8292, 3072, 192), (300, 768, 3072), (64, 2304, 768),
-                                   (1, 8, 64), (129, 136, 128)])
+# (8192, 3072, 1024), (8155, 3080, 1024) and (8292, 3072, 1088) run the wide 256 x 128 form (grids of
+# 768+ workgroups, K >= 1024): full tiles, ragged token / feature edges, and a K loop whose length
+# is not a multiple of the ring depth; (8192, 3072, 768) has the grid but not the K and, like the
+# others, runs the 128 x 128 form.
+@pytest.mark.parametrize("M,N,K", [(8192, 3072, 1024), (8155, 3080, 1024), (8292, 3072, 1088), (8192, 3072, 768),
+                                   (300, 768, 3072), (64, 2304, 768), (1, 8, 64), (129, 136, 128)])
 @pytest.mark.parametrize("act", ["none", "gelu", "gelu_tanh", "relu"])
 def test_gemm_bias_act(M, N, K, act):
     print(f"gemm M{M} N{N} K{K} {act}", flush=True)
@@ -47,10 +48,10 @@ def test_gemm_strided_rows_and_no_bias():
     W = _rand(128, 72, seed=5, scale=0.1)
     got = fused.gemm_bias_act(xs, fused.pack_weight(W.cuda()), None, "none")
     _close(got, x[:, :128].float() @ W.float(), "strided")
-    big = _rand(8192, 320, seed=15)               # wide form, row pitch 320, K = 256
-    Wb = _rand(256, 3072, seed=16, scale=0.05)
-    _close(fused.gemm_bias_act(big.cuda()[:, :256], fused.pack_weight(Wb.cuda()), None, "none"),
-           big[:, :256].float() @ Wb.float(), "strided, wide form")
+    big = _rand(8192, 1088, seed=15)              # wide form, row pitch 1088, K = 1024
+    Wb = _rand(1024, 3072, seed=16, scale=0.05)
+    _close(fused.gemm_bias_act(big.cuda()[:, :1024], fused.pack_weight(Wb.cuda()), None, "none"),
+           big[:, :1024].float() @ Wb.float(), "strided, wide form")
     ident = torch.eye(64).half()                  # closed form: W = I returns the input
     _close(fused.gemm_bias_act(x.cuda()[:, :64].contiguous(), ident.cuda(), None, "none"), x[:, :64], "identity")
 

@@ -13,7 +13,8 @@ def _lut(mask2d):
 
 @pytest.mark.parametrize("name,cfg,mask_fn,form,groups", [
     ("C1", configs.AttnConfig("C1", 1, 12, 512), configs.mask_c1, "two_rows", 48),      # S 512: 8 query blocks
-    ("C2", configs.C2, configs.mask_c2, "key_split", 768),                               # 3.0 per CU, 16 query blocks
+    ("C2", configs.C2, configs.mask_c2, "two_rows", 768),                                # 3.0 per CU: the split would need two rounds
+    ("C2/B4", configs.AttnConfig("C2b4", 4, 12, 1024), configs.mask_c2, "key_split", 384),  # 1.5 per CU, 16 query blocks
     ("C4", configs.C4, configs.mask_c4, "two_rows", 1024),                               # 4.0 per CU
     ("C5", configs.AttnConfig("C5", 4, 16, 2048), configs.mask_c5, "two_rows", 1024),
 ])
@@ -23,7 +24,7 @@ def test_launch_form_of_baseline_workloads(name, cfg, mask_fn, form, groups):
     assert sel.operator == "block-wise"
     assert sel.launch_form == form
     assert sel.groups_per_cu == pytest.approx(groups / 256)
-    full, part = configs.BLOCK_COUNTS[name]
+    full, part = configs.BLOCK_COUNTS[name.split("/")[0]]
     assert sel.rho == pytest.approx((full + part) / (cfg.seq // 64) ** 2)
     assert str(sel) == f"block-wise {form} m64n64"
 
