@@ -139,6 +139,28 @@ def bench_layer_c3(steps, warmup):
     return out
 
 
+def bench_small_batch_layer(steps, warmup):
+    """BERT-base layer at B1 S512 (the C1 mask): five short kernels, so issuing the launches
+    costs as much as running them; eager launches vs one HIP-graph replay vs PyTorch eager."""
+    from stof import configs, masks as pm
+    from stof.layer import CapturedForward, EncoderLayer, eager_layer
+    cfg = configs.LayerConfig("C1-layer", 1, 512, 768, 12, 3072, 1)
+    w = {k: v.cuda() for k, v in configs.layer_weights(cfg.hidden, cfg.ffn, seed=0).items()}
+    x = configs.layer_input(cfg, seed=1, device="cuda")
+    mask = configs.mask_c1(cfg.seq)[None]
+    lut = pm.get_sparse_storage(mask.float().cuda(), 64, 64)[1:]
+    layer = EncoderLayer(w, cfg.heads, eps=cfg.eps)
+    run = CapturedForward(layer, x, lut)
+    out = {}
+    out["launched_ms"], _ = time_region(lambda: layer(x, lut), steps, warmup)
+    out["graph_replay_ms"], _ = time_region(lambda: run.graph.replay(), steps, warmup)
+    maskg = mask.cuda().half()
+    with torch.no_grad():
+        out["eager_ms"], _ = time_region(lambda: eager_layer(x, w, maskg, cfg.heads, cfg.eps), steps, warmup)
+    out["speedup_vs_eager"] = out["eager_ms"] / min(out["launched_ms"], out["graph_replay_ms"])
+    return out
+
+
 def bench_c1(steps, warmup, with_cpu):
     """C1 (B1 H12 S512, causal window 128 + first 64 tokens global): the GPU kernel on the fp16
     inputs and the reference's dense attention in fp32 on the host, as the config specifies."""
@@ -258,7 +280,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=2000,
                     help="untimed steps before the timed ones; the default (about 70 ms of load) lets the clocks settle")
     ap.add_argument("--no-extras", action="store_true", help="skip everything but the C2 attention step")
-    ap.add_argument("--extras", default="c1,c4,c4big,dense,c3,c5,hbm,lut",
+    ap.add_argument("--extras", default="c1,c4,c4big,dense,c3,c3small,c5,hbm,lut",
                     help="comma-separated subset of the extra workloads to run (for profiling one kind of kernel)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--copy-probe", action="store_true",
@@ -314,6 +336,8 @@ def main():
             also["C1_mha_S512"] = bench_c1(args.steps, args.warmup, not args.no_cpu)
         if "c3" in want:
             also["C3_bert_base_layer"] = bench_layer_c3(max(args.steps // 4, 20), 10)
+        if "c3small" in want:
+            also["bert_base_layer_B1_S512"] = bench_small_batch_layer(max(args.steps // 4, 20), 20)
         if "c5" in want:
             also["C5_stack_24_layers"] = bench_stack_c5(max(args.steps // 20, 5), 2)
         if "hbm" in want:

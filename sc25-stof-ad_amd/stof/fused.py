@@ -25,8 +25,14 @@ ACT = {"none": 0, "gelu": 1, "gelu_erf": 1, "gelu_tanh": 2, "relu": 3}
 _PACK_ATTR = "_stof_packed_nk"
 
 
-def _stream():
-    return torch.cuda.current_stream().cuda_stream
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
+def _stream(t):
+    """Raw handle of torch's current stream on the device of tensor ``t``."""
+    if _raw_stream is not None and t.device.index is not None:
+        return _raw_stream(t.device.index)
+    return torch.cuda.current_stream(t.device).cuda_stream
 
 
 def _require(cond, msg):
@@ -76,7 +82,7 @@ def bias_residual_layernorm(x, bias, residual, gamma, beta, eps=1e-5, return_sta
         mean = torch.empty(M, dtype=torch.float32, device=x.device)
         rstd = torch.empty(M, dtype=torch.float32, device=x.device)
     check(_lib.lib().stof_bias_res_ln(x.data_ptr(), _p(bias), _p(residual), _p(gamma), _p(beta),
-                                      y.data_ptr(), _p(mean), _p(rstd), M, N, float(eps), _stream()),
+                                      y.data_ptr(), _p(mean), _p(rstd), M, N, float(eps), _stream(y)),
           "stof_bias_res_ln")
     return (y, mean, rstd) if return_stats else y
 
@@ -104,7 +110,7 @@ def gemm_bias_act(x, Wt, bias=None, act="none", out=None):
     o2 = out.view(-1, N)
     _require(o2.shape[0] == M and o2.stride(1) == 1, "out must be [..., N] with contiguous rows")
     check(_lib.lib().stof_gemm_bias_act(x2.data_ptr(), Wt.data_ptr(), _p(bias), o2.data_ptr(),
-                                        M, N, K, x2.stride(0), o2.stride(0), ACT[act], _stream()),
+                                        M, N, K, x2.stride(0), o2.stride(0), ACT[act], _stream(o2)),
           "stof_gemm_bias_act")
     return out
 
@@ -122,7 +128,7 @@ def gemm_bias_residual_layernorm(x, Wt, bias, residual, gamma, beta, eps=1e-5, o
     if out is None:
         out = torch.empty(x.shape[:-1] + (N,), dtype=torch.float16, device=x.device)
     check(_lib.lib().stof_gemm_bias_res_ln(x.data_ptr(), Wt.data_ptr(), _p(bias), _p(residual),
-                                           _p(gamma), _p(beta), out.data_ptr(), M, N, K, float(eps), _stream()),
+                                           _p(gamma), _p(beta), out.data_ptr(), M, N, K, float(eps), _stream(out)),
           "stof_gemm_bias_res_ln")
     return out
 

@@ -25,8 +25,14 @@ __all__ = ["block_attn", "block_attn_mask_op", "rowwise_attn_full_op", "rowwise_
 _BITS_ATTR = "_stof_packed_bits"
 
 
-def _stream():
-    return torch.cuda.current_stream().cuda_stream
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
+def _stream(device=None):
+    """Raw handle of torch's current stream on ``device`` (a torch.device) or the current device."""
+    if _raw_stream is not None and device is not None and device.index is not None:
+        return _raw_stream(device.index)
+    return torch.cuda.current_stream(device).cuda_stream
 
 
 def _ptr(t):
@@ -62,7 +68,7 @@ def pack_mask_bits(src, additive):
     rows = src.numel() // cols
     dst = torch.empty(src.shape[:-1] + (cols // 64,), dtype=torch.int64, device=src.device)
     check(_lib.lib().stof_pack_mask_bits(src.data_ptr(), dst.data_ptr(), rows, cols, cols,
-                                         1 if additive else 0, _stream()), "stof_pack_mask_bits")
+                                         1 if additive else 0, _stream(src.device)), "stof_pack_mask_bits")
     return dst
 
 
@@ -145,6 +151,49 @@ def _lut_at_64(lut, S, block_m, block_n):
     return lut64
 
 
+_LUT_READY_ATTR = "_stof_lut_ready"
+
+
+def _prepared_lut(lut, B, S, block_m, block_n, dev):
+    """Validate a LUT and turn it into the seven pointers ``stof_block_attn_fwd`` takes plus the
+    per-sample row-pointer stride.  The work (dtype / device / shape / ordering checks, bit
+    packing of the partial blocks, re-tiling to 64 x 64) is done once per LUT: the result is
+    kept on the LOAD column tensor, keyed by the identity and content version of all seven
+    tensors, the problem size and the device, and it holds the tensors it points into."""
+    lci = lut[6]
+    key = (B, S, block_m, block_n, dev) + tuple((id(t), t._version) for t in lut)
+    cached = getattr(lci, _LUT_READY_ATTR, None)
+    if cached is not None and cached[0] == key:
+        return cached[1], cached[2]
+    frp, fci, prp, pci, pbm, lrp, lci = lut
+    frp = _check_i32("full_row_ptr", frp, dev); fci = _check_i32("full_col_idx", fci, dev)
+    prp = _check_i32("part_row_ptr", prp, dev); pci = _check_i32("part_col_idx", pci, dev)
+    lrp = _check_i32("load_row_ptr", lrp, dev); lci_c = _check_i32("load_col_idx", lci, dev)
+    _require(pbm.dtype == torch.float16 and pbm.device == dev, "part_block_mask must be fp16 on q's device")
+    _require(S % block_m == 0 and S % block_n == 0, f"seq_len {S} not divisible by block {block_m}x{block_n}")
+    nq = S // block_m
+    if lrp.dim() == 2:
+        _require(lrp.shape == (B, nq + 1) and frp.shape == lrp.shape and prp.shape == lrp.shape,
+                 f"per-sample row pointers must be [{B}, {nq + 1}]")
+        lut_bs = nq + 1
+    else:
+        _require(lrp.numel() == nq + 1 and frp.numel() == nq + 1 and prp.numel() == nq + 1,
+                 f"row pointers must have {nq + 1} entries for seq_len {S}, block_m {block_m}")
+        lut_bs = 0
+    _check_lut_order(lrp, lci_c, prp, pci, S // block_n)
+    if (block_m, block_n) != (64, 64):
+        _require(S % 64 == 0, f"seq_len {S} must be a multiple of 64")
+        frp, fci, prp, pci, pbm, lrp, lci_c = _lut_at_64((frp, fci, prp, pci, pbm, lrp, lci_c), S, block_m, block_n)
+    bits = _packed_partial_bits(pbm)
+    keep = (frp, fci, prp, pci, bits, lrp, lci_c)
+    ptrs = tuple(_ptr(t) for t in keep)
+    try:
+        setattr(lci, _LUT_READY_ATTR, (key, ptrs, lut_bs, keep, tuple(lut)))   # holds what the key and the pointers refer to
+    except AttributeError:
+        pass
+    return ptrs, lut_bs
+
+
 def _check_i32(name, t, device):
     _require(t.dtype == torch.int32, f"{name} must be int32, got {t.dtype}")
     _require(t.device == device, f"{name} is on {t.device}, expected {device}")
@@ -159,35 +208,15 @@ def block_attn(q, k, v, lut, block_m=64, block_n=64, out=None, out_layout="bhsd"
     per sample).  Returns ``out``: ``[B,H,S,D]`` (``out_layout='bhsd'``) or ``[B,S,H*D]``
     (``'bshd'``); ``out`` may be ``q`` itself.
     """
-    frp, fci, prp, pci, pbm, lrp, lci = lut
     _require(q.is_cuda, "q must be a CUDA tensor (this path has no CPU implementation)")
+    dev = q.device
     for name, t in (("q", q), ("k", k), ("v", v)):
         _require(t.dtype == torch.float16, f"{name} must be float16, got {t.dtype}")
         _require(t.dim() == 4 and t.stride(3) == 1, f"{name} must be [B,H,S,D] with contiguous D")
-        _require(t.device == q.device, f"{name} is on a different device than q")
+        _require(t is q or t.device == dev, f"{name} is on a different device than q")
     _require(k.shape == q.shape and v.shape == q.shape, "q, k, v must have the same shape")
     B, H, S, D = q.shape
-    dev = q.device
-    frp = _check_i32("full_row_ptr", frp, dev); fci = _check_i32("full_col_idx", fci, dev)
-    prp = _check_i32("part_row_ptr", prp, dev); pci = _check_i32("part_col_idx", pci, dev)
-    lrp = _check_i32("load_row_ptr", lrp, dev); lci = _check_i32("load_col_idx", lci, dev)
-    _require(pbm.dtype == torch.float16 and pbm.device == dev, "part_block_mask must be fp16 on q's device")
-    _require(S % block_m == 0 and S % block_n == 0, f"seq_len {S} not divisible by block {block_m}x{block_n}")
-    nq = S // block_m
-    if lrp.dim() == 2:
-        _require(lrp.shape == (B, nq + 1) and frp.shape == lrp.shape and prp.shape == lrp.shape,
-                 f"per-sample row pointers must be [{B}, {nq + 1}]")
-        lut_bs = nq + 1
-    else:
-        _require(lrp.numel() == nq + 1 and frp.numel() == nq + 1 and prp.numel() == nq + 1,
-                 f"row pointers must have {nq + 1} entries for seq_len {S}, block_m {block_m}")
-        lut_bs = 0
-    _check_lut_order(lrp, lci, prp, pci, S // block_n)
-    if (block_m, block_n) != (64, 64):
-        _require(S % 64 == 0, f"seq_len {S} must be a multiple of 64")
-        frp, fci, prp, pci, pbm, lrp, lci = _lut_at_64((frp, fci, prp, pci, pbm, lrp, lci), S, block_m, block_n)
-        block_m = block_n = 64
-    bits = _packed_partial_bits(pbm)
+    lut_ptrs, lut_bs = _prepared_lut(lut, B, S, block_m, block_n, dev)
     if out is None:
         if out_layout == "bhsd":
             out = torch.empty((B, H, S, D), dtype=torch.float16, device=dev)
@@ -205,10 +234,9 @@ def block_attn(q, k, v, lut, block_m=64, block_n=64, out=None, out_layout="bhsd"
     scale = softmax_scale if softmax_scale is not None else 1.0 / math.sqrt(D)
     check(_lib.lib().stof_block_attn_fwd(
         q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(),
-        _ptr(frp), _ptr(fci), _ptr(prp), _ptr(pci), _ptr(bits), _ptr(lrp), _ptr(lci),
-        block_m, block_n, scale,
+        *lut_ptrs, 64, 64, scale,
         strides3(q), strides3(k), strides3(v), ostr,
-        B, S, H, D, lut_bs, _stream()), "stof_block_attn_fwd")
+        B, S, H, D, lut_bs, _stream(dev)), "stof_block_attn_fwd")
     return out
 
 
@@ -259,7 +287,7 @@ def _rowwise(kind, q, k, v, is_causal, bandwidth, row_mask):
     check(_lib.lib().stof_rowwise_attn_fwd(
         q.data_ptr(), k.data_ptr(), v.data_ptr(), result.data_ptr(),
         kind, 1 if is_causal else 0, int(bandwidth), _ptr(bits),
-        B, S, H, D, _stream()), "stof_rowwise_attn_fwd")
+        B, S, H, D, _stream(q.device)), "stof_rowwise_attn_fwd")
     return result
 
 

@@ -7,7 +7,7 @@ import torch
 from oracle import attention as oa
 from oracle import encoder as oe
 from stof import configs, fused, masks as pm
-from stof.layer import EncoderLayer, EncoderStack
+from stof.layer import CapturedForward, EncoderLayer, EncoderStack
 from stof.ops import (rowwise_attn_full_op, rowwise_attn_sliding_op, rowwise_attn_mask_op, StofError)
 
 pytestmark = pytest.mark.gpu
@@ -158,3 +158,25 @@ def test_encoder_stack_two_layers_c5_shape_reduced():
     for w in ws:
         want = oe.bert_layer(want, w, mask.float(), H, eps=1e-12)
     _close(got, want, "stack", atol=6e-3)
+
+
+def test_captured_stack_replays_match_eager_launches():
+    """A two-layer stack recorded into a HIP graph: every replay (different inputs, eager work
+    and synchronisation between replays) must reproduce the eagerly launched stack bit for bit."""
+    B, S, D, H, F = 1, 512, 768, 12, 3072
+    ws = [configs.layer_weights(D, F, seed=s) for s in (3, 4)]
+    mask = configs.mask_c1(S)[None]
+    lut = pm.get_sparse_storage(mask.float().cuda(), 64, 64)[1:]
+    stack = EncoderStack([{k: v.cuda() for k, v in w.items()} for w in ws], H, eps=1e-12)
+    xs = [configs.layer_input(configs.LayerConfig("t", B, S, D, H, F, 2), seed=s).cuda() for s in (5, 6, 7, 8)]
+    run = CapturedForward(stack, xs[0], lut)
+    for i, x in enumerate(xs):
+        print(f"graph replay {i}", flush=True)
+        want = stack(x, lut)                       # eager launches between the replays
+        torch.cuda.synchronize()
+        got = run(x).clone()
+        torch.cuda.synchronize()
+        assert torch.equal(got, want), f"replay {i} differs from the eager result"
+    want0 = oe.bert_layer(oe.bert_layer(xs[0].cpu(), ws[0], mask.float(), H, eps=1e-12), ws[1], mask.float(), H, eps=1e-12)
+    _close(run(xs[0]), want0, "captured stack vs oracle", atol=6e-3)
+
