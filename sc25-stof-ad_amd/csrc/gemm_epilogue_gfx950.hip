@@ -183,13 +183,18 @@ __global__ __launch_bounds__(256) void gemm_bias_act_kernel(const GemmParams p) 
 }
 
 // ------------------------------------------------------------------------------------------
-// Wide form of the same GEMM: tile 256 (tokens) x 128 (features) x 32 (K), 4 waves as 2 x 2,
-// each 128 tokens x 64 features = 4 x 2 MFMA tiles.  A wave reads 6 fragments for 8 MFMAs per
-// k-step (0.75 KB of LDS per MFMA instead of 1 KB) and a workgroup brings in 24 KB per 2.1
-// MFLOP (85 FLOP per byte over the L2 -> LDS path instead of 64).  The K loop is a ring of NS
+// Ring forms of the same GEMM: tile (64 * MI tokens) x 128 (features) x 32 (K), 4 waves as
+// 2 x 2, each (32 * MI) tokens x 64 features = MI x 2 MFMA tiles.  The K loop is a ring of NS
 // stages filled by direct-to-LDS loads and is software pipelined inside the wave.
+//   MI = 4, NS = 3 (wide): 256-token tiles; a wave reads 6 fragments for 8 MFMAs per k-step
+//     (0.75 KB of LDS per MFMA instead of 1 KB) and a workgroup brings in 24 KB per 2.1 MFLOP
+//     (85 FLOP per byte over the L2 -> LDS path instead of 64): the form for large grids.
+//   MI = 1, NS = 4 (small): 64-token tiles, four times the workgroups of the 128 x 128 form and
+//     three tiles in flight per workgroup: the form for token counts that give the 128 x 128
+//     form less than one workgroup per two compute units, where the K loop of each workgroup
+//     runs at the latency of its loads (512 tokens, N 768, K 3072: 36 -> 23 us).
 // ------------------------------------------------------------------------------------------
-constexpr int kWTok = 256;
+constexpr int kWTok = 256;     // tokens per workgroup of the wide form (MI = 4)
 constexpr int kWFeat = 128;
 
 // 64-byte rows: chunk c of row r sits at position c ^ ((r >> 2) & 3); 16 rows fill 1 KB.
@@ -198,10 +203,13 @@ __device__ __forceinline__ int swz4(int row) { return (row >> 2) & 3; }
 // s_waitcnt immediate that waits for the vector-memory counter only (lgkmcnt 15, expcnt 7)
 constexpr int vmcnt_imm(int n) { return (n & 15) | ((n >> 4) << 14) | 0x0F70; }
 
-template <int ACT, int NS>
-__global__ __launch_bounds__(256, NS <= 3 ? 2 : 1) void gemm_bias_act_wide_kernel(const GemmParams p) {
+template <int ACT, int NS, int MI>
+__global__ __launch_bounds__(256, 2) void gemm_bias_act_ring_kernel(const GemmParams p) {
+  static_assert(MI == 1 || MI == 2 || MI == 4, "token tiles per wave");
   constexpr int kK = 32;
-  constexpr int kATile = kWTok * kK * 2, kWTile = kWFeat * kK * 2;   // 16 KB, 8 KB
+  constexpr int kTok = 64 * MI;           // tokens per workgroup: two waves of MI 32-token tiles
+  constexpr int kLoads = MI + 2;          // load instructions per wave per tile
+  constexpr int kATile = kTok * kK * 2, kWTile = kWFeat * kK * 2;   // 4 KB * MI, 8 KB
   // Ring of NS stages: NS tiles are in flight or in use at any time, so a tile has NS - 1 tile
   // times to arrive.  (The fragment reads below are asm, so the compiler does not order them
   // against the direct-to-LDS loads and one array per operand is enough.)
@@ -211,20 +219,20 @@ __global__ __launch_bounds__(256, NS <= 3 ? 2 : 1) void gemm_bias_act_wide_kerne
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int lane = threadIdx.x & 63;
   const int j32 = lane & 31, g = lane >> 5;
-  const int wf = wave >> 1, wt = wave & 1;   // feature half (64), token half (128)
+  const int wf = wave >> 1, wt = wave & 1;   // feature half (64), token half (32 * MI)
 
   const int tm = blockIdx.x % p.tiles_m;
   const int tn = blockIdx.x / p.tiles_m;
-  const int m0 = tm * kWTok, n0 = tn * kWFeat;
+  const int m0 = tm * kTok, n0 = tn * kWFeat;
 
-  // Loads: one instruction = 16 rows of 64 B.  A tile: 16 instructions (4 per wave), W tile: 8
-  // (2 per wave).  Rows past the edge re-read the last row.  Addresses are a wave-uniform tile
+  // Loads: one instruction = 16 rows of 64 B.  A tile: 4 * MI instructions (MI per wave), W
+  // tile: 8 (2 per wave).  Rows past the edge re-read the last row.  Addresses are a wave-uniform tile
   // base (advanced along K in scalar registers) plus a 32-bit per-lane byte offset.
   const int drow = lane >> 2;
-  uint32_t a_off[4], w_off[2];
+  uint32_t a_off[MI], w_off[2];
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int trow = 16 * (4 * wave + i) + drow;
+  for (int i = 0; i < MI; ++i) {
+    const int trow = 16 * (MI * wave + i) + drow;
     const int chunk = (lane & 3) ^ swz4(trow);
     a_off[i] = (uint32_t)min(trow, p.M - 1 - m0) * (uint32_t)(p.lda * 2) + 16 * chunk;
   }
@@ -242,8 +250,8 @@ __global__ __launch_bounds__(256, NS <= 3 ? 2 : 1) void gemm_bias_act_wide_kerne
     lds_byte* ad = (lds_byte*)a_lds + stage * kATile;
     lds_byte* wd = (lds_byte*)w_lds + stage * kWTile;
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
-      __builtin_amdgcn_global_load_lds((gptr_t*)(ab + a_off[i]), (__attribute__((address_space(3))) void*)(ad + (4 * wave + i) * 1024), 16, 0, 0);
+    for (int i = 0; i < MI; ++i)
+      __builtin_amdgcn_global_load_lds((gptr_t*)(ab + a_off[i]), (__attribute__((address_space(3))) void*)(ad + (MI * wave + i) * 1024), 16, 0, 0);
 #pragma unroll
     for (int i = 0; i < 2; ++i)
       __builtin_amdgcn_global_load_lds((gptr_t*)(wbase + w_off[i]), (__attribute__((address_space(3))) void*)(wd + (2 * wave + i) * 1024), 16, 0, 0);
@@ -253,11 +261,11 @@ __global__ __launch_bounds__(256, NS <= 3 ? 2 : 1) void gemm_bias_act_wide_kerne
 #pragma unroll
   for (int ks = 0; ks < 2; ++ks) rd[ks] = j32 * 64 + (((2 * ks + g) ^ swz4(j32)) << 4);
 
-  floatx16 acc[2][4];   // [feature tile ni][token tile mi]
+  floatx16 acc[2][MI];   // [feature tile ni][token tile mi]
 #pragma unroll
   for (int i = 0; i < 2; ++i)
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
+    for (int j = 0; j < MI; ++j)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
@@ -265,23 +273,37 @@ __global__ __launch_bounds__(256, NS <= 3 ? 2 : 1) void gemm_bias_act_wide_kerne
   // direct-to-LDS load it cannot prove disjoint, which drains the ring.  The ring's own
   // counter waits cover that dependency; the LDS counter is waited on by hand, fenced so that
   // nothing that uses a fragment can be scheduled above its wait.
-  auto frags = [&](uint32_t wa, uint32_t aa, half8_t (&wbk)[2], half8_t (&xak)[4]) {
-    asm volatile(
-        "ds_read_b128 %0, %6\n\tds_read_b128 %1, %6 offset:2048\n\t"
-        "ds_read_b128 %2, %7\n\tds_read_b128 %3, %7 offset:2048\n\t"
-        "ds_read_b128 %4, %7 offset:4096\n\tds_read_b128 %5, %7 offset:6144"
-        : "=&v"(wbk[0]), "=&v"(wbk[1]), "=&v"(xak[0]), "=&v"(xak[1]), "=&v"(xak[2]), "=&v"(xak[3])
-        : "v"(wa), "v"(aa));
+  auto frags = [&](uint32_t wa, uint32_t aa, half8_t (&wbk)[2], half8_t (&xak)[MI]) {
+    if constexpr (MI == 4) {
+      asm volatile(
+          "ds_read_b128 %0, %6\n\tds_read_b128 %1, %6 offset:2048\n\t"
+          "ds_read_b128 %2, %7\n\tds_read_b128 %3, %7 offset:2048\n\t"
+          "ds_read_b128 %4, %7 offset:4096\n\tds_read_b128 %5, %7 offset:6144"
+          : "=&v"(wbk[0]), "=&v"(wbk[1]), "=&v"(xak[0]), "=&v"(xak[1]), "=&v"(xak[2]), "=&v"(xak[3])
+          : "v"(wa), "v"(aa));
+    } else if constexpr (MI == 2) {
+      asm volatile(
+          "ds_read_b128 %0, %4\n\tds_read_b128 %1, %4 offset:2048\n\t"
+          "ds_read_b128 %2, %5\n\tds_read_b128 %3, %5 offset:2048"
+          : "=&v"(wbk[0]), "=&v"(wbk[1]), "=&v"(xak[0]), "=&v"(xak[1])
+          : "v"(wa), "v"(aa));
+    } else {
+      asm volatile(
+          "ds_read_b128 %0, %3\n\tds_read_b128 %1, %3 offset:2048\n\t"
+          "ds_read_b128 %2, %4"
+          : "=&v"(wbk[0]), "=&v"(wbk[1]), "=&v"(xak[0])
+          : "v"(wa), "v"(aa));
+    }
   };
-  auto lds_wait = [&](int outstanding) {   // 0 or 6 fragment reads may remain in flight
+  auto lds_wait = [&](bool one_set_in_flight) {   // wait for all fragment reads, or all but the MI + 2 of the latest set
     __builtin_amdgcn_sched_barrier(0);
-    if (outstanding == 0) __builtin_amdgcn_s_waitcnt(0xC07F);   // lgkmcnt(0)
-    else __builtin_amdgcn_s_waitcnt(0xC67F);                    // lgkmcnt(6)
+    if (!one_set_in_flight) __builtin_amdgcn_s_waitcnt(0xC07F);   // lgkmcnt(0)
+    else __builtin_amdgcn_s_waitcnt(0xC07F | ((MI + 2) << 8));    // lgkmcnt(MI + 2)
     __builtin_amdgcn_sched_barrier(0);
   };
-  auto mfmas = [&](const half8_t (&wbk)[2], const half8_t (&xak)[4]) {
+  auto mfmas = [&](const half8_t (&wbk)[2], const half8_t (&xak)[MI]) {
 #pragma unroll
-    for (int mi = 0; mi < 4; ++mi)
+    for (int mi = 0; mi < MI; ++mi)
 #pragma unroll
       for (int ni = 0; ni < 2; ++ni) acc[ni][mi] = mfma32(wbk[ni], xak[mi], acc[ni][mi]);
   };
@@ -292,14 +314,14 @@ __global__ __launch_bounds__(256, NS <= 3 ? 2 : 1) void gemm_bias_act_wide_kerne
     __builtin_amdgcn_sched_barrier(0);
   };
   const uint32_t w_rd = (uint32_t)(uintptr_t)(lds_byte*)w_lds + (uint32_t)(64 * wf) * 64;
-  const uint32_t a_rd = (uint32_t)(uintptr_t)(lds_byte*)a_lds + (uint32_t)(128 * wt) * 64;
-  half8_t xa0[4], wb0[2], xa1[4], wb1[2];   // fragments of k-step 0 / k-step 1 of a tile
+  const uint32_t a_rd = (uint32_t)(uintptr_t)(lds_byte*)a_lds + (uint32_t)(32 * MI * wt) * 64;
+  half8_t xa0[MI], wb0[2], xa1[MI], wb1[2];   // fragments of k-step 0 / k-step 1 of a tile
 
   const int nk = p.K / kK;
 #pragma unroll
   for (int s0 = 0; s0 < NS; ++s0)
     if (s0 < nk) issue(s0, s0);
-  if (nk >= NS) __builtin_amdgcn_s_waitcnt(vmcnt_imm(6 * (NS - 1)));   // tile 0 landed
+  if (nk >= NS) __builtin_amdgcn_s_waitcnt(vmcnt_imm(kLoads * (NS - 1)));   // tile 0 landed
   else __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
   wg_barrier();
   frags(w_rd + rd[0], a_rd + rd[0], wb0, xa0);
@@ -310,12 +332,12 @@ __global__ __launch_bounds__(256, NS <= 3 ? 2 : 1) void gemm_bias_act_wide_kerne
   for (int t = 0; t < nk; ++t) {
     const int ns = (cs + 1 == NS) ? 0 : cs + 1;
     frags(w_rd + cs * kWTile + rd[1], a_rd + cs * kATile + rd[1], wb1, xa1);
-    lds_wait(6);
+    lds_wait(true);
     mfmas(wb0, xa0);
-    lds_wait(0);
+    lds_wait(false);
     if (t + 1 < nk) {
       // tiles t+1 .. t+NS-1 are outstanding; all but the first may stay in flight
-      if (t + NS - 1 < nk) __builtin_amdgcn_s_waitcnt(vmcnt_imm(6 * (NS - 2)));
+      if (t + NS - 1 < nk) __builtin_amdgcn_s_waitcnt(vmcnt_imm(kLoads * (NS - 2)));
       else __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
       wg_barrier();
       if (t + NS < nk) issue(t + NS, cs);
@@ -326,10 +348,10 @@ __global__ __launch_bounds__(256, NS <= 3 ? 2 : 1) void gemm_bias_act_wide_kerne
     cs = ns;
   }
 
-  // epilogue: acc[ni][mi][r] = C[m0 + 128wt + 32mi + j32][n0 + 64wf + 32ni + 8(r/4) + 4g + r%4]
+  // epilogue: acc[ni][mi][r] = C[m0 + 32MI*wt + 32mi + j32][n0 + 64wf + 32ni + 8(r/4) + 4g + r%4]
 #pragma unroll
-  for (int mi = 0; mi < 4; ++mi) {
-    const int m = m0 + 128 * wt + 32 * mi + j32;
+  for (int mi = 0; mi < MI; ++mi) {
+    const int m = m0 + 32 * MI * wt + 32 * mi + j32;
     if (m >= p.M) continue;
     half_t* crow = p.C + (int64_t)m * p.ldc;
 #pragma unroll
@@ -518,16 +540,39 @@ __global__ __launch_bounds__(512) void gemm_bias_res_ln_kernel(const LnGemmParam
   }
 }
 
-// Which form runs: the wide one when its grid has at least kWideMinGroups workgroups (three per
-// compute unit of an MI355X) and K is at least kWideMinK.  Measured at settled clocks, 8192
-// tokens: N 3072 K 1024 721 vs 673 TFLOP/s, N 4096 K 1024 706 vs 648, N 1024 K 4096 882 vs 830,
-// 8192^3 951 vs 864; with K 768 (N 3072: 564 vs 598) its longer ring fill and epilogue per
-// workgroup are not paid back, and on smaller grids its 256-token tiles leave compute units
-// idle.  Three ring stages: deeper rings (one workgroup per compute unit) measured no faster;
-// a 256 x 256 tile with eight waves gained 3-9 % only from N 4096 up and is not built.
+// Which form runs.
+//  * wide ring (256-token tiles, 3 stages) when its grid has at least kWideMinGroups workgroups
+//    (three per compute unit of an MI355X) and K is at least kWideMinK.  Measured at settled
+//    clocks, 8192 tokens: N 3072 K 1024 721 vs 673 TFLOP/s, N 4096 K 1024 706 vs 648, N 1024
+//    K 4096 882 vs 830, 8192^3 951 vs 864; with K 768 (N 3072: 564 vs 598) its longer ring fill
+//    and epilogue per workgroup are not paid back.  Deeper rings (one workgroup per compute
+//    unit) measured no faster; a 256 x 256 tile with eight waves gained 3-9 % only from N 4096
+//    up and is not built.
+//  * small ring (64-token tiles, 4 stages) when the 128 x 128 form would have at most
+//    kSmallMaxTiles workgroups.  GPU time, N x K of the BERT-base layer: 512 tokens 14.4 -> 8.9,
+//    14.0 -> 8.4, 14.5 -> 10.6, 36.0 -> 22.9 us; 2048 tokens x N 768: 14.2 -> 8.9, 36.9 -> 23.2 us;
+//    from 192 tiles on (4096 tokens x N 768, 2048 x N 2304) the two are within 5 % either way.
+//  * the 128 x 128 double-buffered form otherwise.
 constexpr int kWideStages = 3;
 constexpr int kWideMinGroups = 768;
 constexpr int kWideMinK = 1024;
+constexpr int kSmallStages = 4;
+constexpr int kSmallMaxTiles = 128;
+
+template <int NS, int MI>
+int launch_ring(GemmParams& p, int act, hipStream_t st) {
+  p.tiles_m = (p.M + 64 * MI - 1) / (64 * MI);
+  p.tiles_n = (p.N + kWFeat - 1) / kWFeat;
+  const dim3 grid((unsigned)(p.tiles_m * p.tiles_n)), block(256);
+  switch (act) {
+    case STOF_ACT_NONE: hipLaunchKernelGGL((gemm_bias_act_ring_kernel<STOF_ACT_NONE, NS, MI>), grid, block, 0, st, p); break;
+    case STOF_ACT_GELU_ERF: hipLaunchKernelGGL((gemm_bias_act_ring_kernel<STOF_ACT_GELU_ERF, NS, MI>), grid, block, 0, st, p); break;
+    case STOF_ACT_GELU_TANH: hipLaunchKernelGGL((gemm_bias_act_ring_kernel<STOF_ACT_GELU_TANH, NS, MI>), grid, block, 0, st, p); break;
+    case STOF_ACT_RELU: hipLaunchKernelGGL((gemm_bias_act_ring_kernel<STOF_ACT_RELU, NS, MI>), grid, block, 0, st, p); break;
+    default: return STOF_ERR_UNSUPPORTED;
+  }
+  return stof_check_launch();
+}
 
 }  // namespace
 
@@ -545,18 +590,9 @@ extern "C" int stof_gemm_bias_act(const void* A, const void* Wt, const void* bia
   p.M = (int)M; p.N = (int)N; p.K = (int)K; p.lda = (int)lda; p.ldc = (int)ldc;
   hipStream_t st = (hipStream_t)stream;
   const int64_t wide_groups = ((M + kWTok - 1) / kWTok) * ((N + kWFeat - 1) / kWFeat);
-  if (wide_groups >= kWideMinGroups && K >= kWideMinK) {
-    p.tiles_m = (int)((M + kWTok - 1) / kWTok); p.tiles_n = (int)((N + kWFeat - 1) / kWFeat);
-    const dim3 grid((unsigned)(p.tiles_m * p.tiles_n)), block(256);
-    switch (act) {
-      case STOF_ACT_NONE: hipLaunchKernelGGL((gemm_bias_act_wide_kernel<STOF_ACT_NONE, kWideStages>), grid, block, 0, st, p); break;
-      case STOF_ACT_GELU_ERF: hipLaunchKernelGGL((gemm_bias_act_wide_kernel<STOF_ACT_GELU_ERF, kWideStages>), grid, block, 0, st, p); break;
-      case STOF_ACT_GELU_TANH: hipLaunchKernelGGL((gemm_bias_act_wide_kernel<STOF_ACT_GELU_TANH, kWideStages>), grid, block, 0, st, p); break;
-      case STOF_ACT_RELU: hipLaunchKernelGGL((gemm_bias_act_wide_kernel<STOF_ACT_RELU, kWideStages>), grid, block, 0, st, p); break;
-      default: return STOF_ERR_UNSUPPORTED;
-    }
-    return stof_check_launch();
-  }
+  if (wide_groups >= kWideMinGroups && K >= kWideMinK) return launch_ring<kWideStages, 4>(p, act, st);
+  const int64_t tiles128 = ((M + kGT - 1) / kGT) * ((N + kGT - 1) / kGT);
+  if (tiles128 <= kSmallMaxTiles) return launch_ring<kSmallStages, 1>(p, act, st);
   p.tiles_m = (int)((M + kGT - 1) / kGT); p.tiles_n = (int)((N + kGT - 1) / kGT);
   const dim3 grid((unsigned)(p.tiles_m * p.tiles_n)), block(256);
   switch (act) {

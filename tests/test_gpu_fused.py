@@ -28,12 +28,16 @@ def _rand(*shape, seed=0, scale=1.0):
 
 # ---- GEMM + bias + activation -----------------------------------------------------------------
 
-# (8192, 3072, 1024), (8155, 3080, 1024) and (8292, 3072, 1088) run the wide 256 x 128 form (grids of
-# 768+ workgroups, K >= 1024): full tiles, ragged token / feature edges, and a K loop whose length
-# is not a multiple of the ring depth; (8192, 3072, 768) has the grid but not the K and, like the
-# others, runs the 128 x 128 form.
+# Three launch forms behind one entry point:
+#  wide ring (grids of 768+ workgroups of 256 x 128, K >= 1024): (8192, 3072, 1024) full tiles,
+#    (8155, 3080, 1024) ragged token / feature edges, (8292, 3072, 1088) a K loop whose length is not
+#    a multiple of the ring depth;
+#  128 x 128 double-buffered: (8192, 3072, 768) has the grid of the wide form but not the K,
+#    (2100, 2312, 192) ragged edges on both sides;
+#  small ring (at most 128 tiles of 128 x 128): (300, 768, 3072) long K loop, (64, 2304, 768),
+#    (1, 8, 64) fewer K tiles than ring stages, (129, 136, 128) ragged edges.
 @pytest.mark.parametrize("M,N,K", [(8192, 3072, 1024), (8155, 3080, 1024), (8292, 3072, 1088), (8192, 3072, 768),
-                                   (300, 768, 3072), (64, 2304, 768), (1, 8, 64), (129, 136, 128)])
+                                   (2100, 2312, 192), (300, 768, 3072), (64, 2304, 768), (1, 8, 64), (129, 136, 128)])
 @pytest.mark.parametrize("act", ["none", "gelu", "gelu_tanh", "relu"])
 def test_gemm_bias_act(M, N, K, act):
     print(f"gemm M{M} N{N} K{K} {act}", flush=True)
