@@ -586,10 +586,12 @@ int g_attn_form = kFormAuto;
 // blocks AND the two-row grid gives a compute unit at most kKeySplitMaxGroupsPerCu workgroups.
 // Four workgroups are resident per compute unit (LDS), and the key split doubles the count:
 // up to two two-row groups per compute unit it still runs as a single round with every chain
-// half as long (B2 H12 S2048 causal: 44 -> 34 us, B4 H12 S1024 sparse: 25 -> 23 us), beyond
-// that it needs a second, partly filled round and loses (three per compute unit: -3 % .. +15 %).
+// half as long (GPU time: B2 H12 S2048 causal 44 -> 34 us, B4 H12 S1024 sparse 25 -> 23 us,
+// B1 H12 S512 11.1 -> 9.6 us, B1 H12 S256 7.6 -> 6.6 us), beyond that it needs a second, partly
+// filled round and loses (three per compute unit: -3 % .. +15 %).  With two query blocks
+// (S 128) the chains are too short either way (+-5 %).
 constexpr int kKeySplitMaxGroupsPerCu = 2;
-constexpr int kKeySplitMinQueryBlocks = 16;
+constexpr int kKeySplitMinQueryBlocks = 4;
 
 int pick_form(int64_t two_row_groups, int nQ) {
   if (g_attn_form != kFormAuto) return g_attn_form;

@@ -47,7 +47,7 @@ class GPUParams:
         self.waves_per_group = 4
         # launch-form rule (kKeySplitMaxGroupsPerCu / kKeySplitMinQueryBlocks in the kernel source)
         self.key_split_max_groups_per_cu = 2
-        self.key_split_min_query_blocks = 16
+        self.key_split_min_query_blocks = 4
 
 
 @dataclass(frozen=True)

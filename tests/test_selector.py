@@ -12,7 +12,7 @@ def _lut(mask2d):
 
 
 @pytest.mark.parametrize("name,cfg,mask_fn,form,groups", [
-    ("C1", configs.AttnConfig("C1", 1, 12, 512), configs.mask_c1, "two_rows", 48),      # S 512: 8 query blocks
+    ("C1", configs.AttnConfig("C1", 1, 12, 512), configs.mask_c1, "key_split", 48),     # 0.19 per CU, 8 query blocks
     ("C2", configs.C2, configs.mask_c2, "two_rows", 768),                                # 3.0 per CU: the split would need two rounds
     ("C2/B4", configs.AttnConfig("C2b4", 4, 12, 1024), configs.mask_c2, "key_split", 384),  # 1.5 per CU, 16 query blocks
     ("C4", configs.C4, configs.mask_c4, "two_rows", 1024),                               # 4.0 per CU
@@ -47,7 +47,9 @@ def test_per_sample_row_pointers_and_errors():
     mask, _ = configs.mask_c3(4, 512, 256, seed=0)
     lut = pm.get_sparse_storage_batched(mask.float(), 64, 64)
     sel = selector.select_operator(selector.GPUParams(), lut[6], 4, 512, 12)
-    assert sel.operator in ("block-wise", "row-wise") and sel.launch_form == "two_rows"
+    assert sel.operator in ("block-wise", "row-wise") and sel.launch_form == "key_split"   # 192 groups, 8 query blocks
+    short = selector.select_operator(selector.GPUParams(), lut[6][:, :3], 4, 128, 12)        # two query blocks: never split
+    assert short.launch_form == "two_rows"
     with pytest.raises(ValueError):
         selector.select_operator(selector.GPUParams(), lut[6], 4, 500, 12)
     with pytest.raises(ValueError):
