@@ -57,6 +57,7 @@ struct AttnParams {
   int64_t lut_bs;
   int B, S, H, nQ, nP;   // nP = query-block pairs per (batch, head)
   int total, chunk;
+  int balance, cus_per_xcd;   // balance != 0: groups are dealt to compute units by row length (see balanced_group)
   float c;  // softmax_scale * log2(e)
   // row-wise front-ends (KIND != 0): key blocks come from index arithmetic, not from a LUT
   const uint64_t* row_bits; int words; int causal; int band;
@@ -95,6 +96,12 @@ struct RowList {
   int lo, hi;          // KIND != LUT: the contiguous key-block range [lo, hi]
 };
 
+// Row pointers of a group's rows when the caller of attn_group has them in registers already.
+template <int ROWS> struct RowPtrs {
+  int t0[ROWS], n[ROWS], p0[ROWS], np[ROWS];
+  bool valid;
+};
+
 // ROWS = query blocks per workgroup, KS = key split.  Launched as <2, 1> (four waves: two query
 // blocks x two 32-query halves, every wave sees all 64 keys of a tile) or <1, 2> (four waves
 // on ONE query block: two 32-query halves x two 32-key halves of every tile, partial results
@@ -102,7 +109,7 @@ struct RowList {
 // so the chain of key blocks of a long LUT row finishes in half the time; it is used for
 // small grids, where that chain and not throughput sets the run time.
 template <int KIND, int ROWS, int KS>
-__device__ __forceinline__ void attn_group(const AttnParams& p, const int bh, const int pair,
+__device__ __forceinline__ void attn_group(const AttnParams& p, const int bh, const int pair, const RowPtrs<ROWS>& pre,
                                            unsigned char* k_lds0, unsigned char* k_lds1,
                                            unsigned char* v_lds0, unsigned char* v_lds1) {
   static_assert(KS == 1 || ROWS == 1, "the key split serves a single query block");
@@ -138,10 +145,14 @@ __device__ __forceinline__ void attn_group(const AttnParams& p, const int bh, co
     row[r].lo = 0; row[r].hi = -1;
     if (qr < p.nQ) {
       if (KIND == kKindLut) {
-        row[r].t0 = __builtin_amdgcn_readfirstlane(p.lrp[lo + qr]);
-        row[r].n = __builtin_amdgcn_readfirstlane(p.lrp[lo + qr + 1]) - row[r].t0;
-        row[r].p0 = __builtin_amdgcn_readfirstlane(p.prp[lo + qr]);
-        row[r].np = __builtin_amdgcn_readfirstlane(p.prp[lo + qr + 1]) - row[r].p0;
+        if (pre.valid) {   // the placement code has read the row pointers already
+          row[r].t0 = pre.t0[r]; row[r].n = pre.n[r]; row[r].p0 = pre.p0[r]; row[r].np = pre.np[r];
+        } else {
+          row[r].t0 = __builtin_amdgcn_readfirstlane(p.lrp[lo + qr]);
+          row[r].n = __builtin_amdgcn_readfirstlane(p.lrp[lo + qr + 1]) - row[r].t0;
+          row[r].p0 = __builtin_amdgcn_readfirstlane(p.prp[lo + qr]);
+          row[r].np = __builtin_amdgcn_readfirstlane(p.prp[lo + qr + 1]) - row[r].p0;
+        }
       } else {
         // keys allowed for some query of block qr: (64qr - band, 64qr + 63] when sliding,
         // up to the diagonal block when causal, else every block
@@ -507,14 +518,92 @@ __device__ __forceinline__ int zigzag(int pidx, int bh, int n) {
   __shared__ __attribute__((aligned(1024))) unsigned char v_lds0[kTile];        \
   __shared__ __attribute__((aligned(1024))) unsigned char v_lds1[kTile]
 
+// Length-aware placement.  A mask with a few long rows (global rows, the bottom of a causal
+// mask) otherwise leaves whole compute units with nothing but long chains: measured on B8 H12
+// S1024 with two global rows, every eighth compute unit received three 16-block chains (done at
+// 33 us) while most had 21 blocks in total (done at 19 us).
+//
+// Each XCD owns `chunk / nP` whole heads, taken in sets of about one resident round of groups
+// (4 per compute unit), so that the K/V of few heads is live in the XCD's L2 at a time.  The
+// groups of a set are ordered by (rank of the group inside its own head by descending row
+// length, head) and dealt to the XCD's compute units, which the dispatcher fills round-robin, in
+// boustrophedon order: pass 0 hands units 0..n-1 the first n groups, pass 1 hands units n-1..0
+// the next n, and so on.  Sums per unit come out even and every unit starts with its longest
+// chain.  The rank is computed here from the row pointers (lane l holds group l of the head; at
+// most 32 groups), so no host pass over the LUT and no scratch memory is needed; being a
+// permutation per head it is a bijection also when every sample has its own LUT.  The row
+// pointers read for it are handed on to attn_group, which saves that a memory round trip.
+template <int KIND, int ROWS>
+__device__ __forceinline__ void balanced_group(const AttnParams& p, int& bh, int& pair, RowPtrs<ROWS>& pre) {
+  const int lane = threadIdx.x & 63;
+  const int x = blockIdx.x & 7, i = blockIdx.x >> 3;   // XCD, dispatch index inside it (i < chunk: the grid is exact)
+  const int ncu = p.cus_per_xcd;
+  const int hx = p.chunk / p.nP;                                        // heads of this XCD
+  const int hs = min(hx, max(1, (4 * ncu + p.nP - 1) / p.nP));          // heads per set
+  const int per_set = hs * p.nP;
+  const int s = i / per_set;
+  const int h0 = s * hs;
+  const int hn = min(hs, hx - h0);                                      // heads in this set
+  const int il = i - s * per_set;
+  const int pass = il / ncu, pos = il - pass * ncu;
+  const int plen = min(ncu, hn * p.nP - pass * ncu);
+  const int j = pass * ncu + ((pass & 1) ? plen - 1 - pos : pos);       // position in the set's order
+  const int rank_wanted = j / hn;
+  bh = x * hx + h0 + (j - rank_wanted * hn);
+  pre.valid = false;
+  int rp[ROWS + 1], pp[ROWS + 1];   // LOAD / PART row pointers of group `lane`: rows ROWS*lane .. and the end
+  int len = 0;
+  if (KIND == kKindLut) {
+    const int64_t lo = (int64_t)(bh / p.H) * p.lut_bs;
+#pragma unroll
+    for (int r = 0; r <= ROWS; ++r) {
+      const int qr = min(ROWS * lane + r, p.nQ);   // (lanes past the last group and a missing second row read the end pointer)
+      rp[r] = p.lrp[lo + qr];
+      pp[r] = p.prp[lo + qr];
+    }
+#pragma unroll
+    for (int r = 0; r < ROWS; ++r) len = max(len, rp[r + 1] - rp[r]);
+  } else {
+#pragma unroll
+    for (int r = 0; r < ROWS; ++r) {
+      const int qr = ROWS * lane + r;
+      const int hi = p.causal ? qr : p.nQ - 1;
+      const int first_key = (KIND == kKindPred && p.band > 0) ? 64 * qr - p.band + 1 : 0;
+      if (qr < p.nQ) len = max(len, hi - (first_key > 0 ? first_key / 64 : 0) + 1);
+    }
+  }
+  // one comparable key per group: longer first, lower index first among equals
+  const int key = lane < p.nP ? (len << 6) | (63 - lane) : -1;
+  int rank = 0;
+  for (int q = 0; q < p.nP; ++q) rank += __builtin_amdgcn_readlane(key, q) > key ? 1 : 0;
+  pair = __builtin_ctzll(__ballot(lane < p.nP && rank == rank_wanted));
+  if (KIND == kKindLut) {
+#pragma unroll
+    for (int r = 0; r < ROWS; ++r) {
+      pre.t0[r] = __builtin_amdgcn_readlane(rp[r], pair);
+      pre.n[r] = __builtin_amdgcn_readlane(rp[r + 1], pair) - pre.t0[r];
+      pre.p0[r] = __builtin_amdgcn_readlane(pp[r], pair);
+      pre.np[r] = __builtin_amdgcn_readlane(pp[r + 1], pair) - pre.p0[r];
+    }
+    pre.valid = true;
+  }
+}
+
 template <int KIND, int ROWS, int KS>
 __global__ __launch_bounds__(128 * ROWS * KS, 4) void block_attn_fwd_kernel(const AttnParams p) {
   STOF_ATTN_LDS_TILES;
-  const int vid = xcd_contiguous_id(p);
-  if (vid >= p.total) return;
-  const int bh = vid / p.nP;
-  const int pair = zigzag(vid - bh * p.nP, bh, p.nP);
-  attn_group<KIND, ROWS, KS>(p, bh, pair, k_lds0, k_lds1, v_lds0, v_lds1);
+  int bh, pair;
+  RowPtrs<ROWS> pre;
+  pre.valid = false;
+  if (p.balance) {
+    balanced_group<KIND, ROWS>(p, bh, pair, pre);
+  } else {
+    const int vid = xcd_contiguous_id(p);
+    if (vid >= p.total) return;
+    bh = vid / p.nP;
+    pair = zigzag(vid - bh * p.nP, bh, p.nP);
+  }
+  attn_group<KIND, ROWS, KS>(p, bh, pair, pre, k_lds0, k_lds1, v_lds0, v_lds1);
 }
 
 // dst[r*(cols/64)+w] bit t = pred(src[r*ld + 64w + t]).
@@ -593,8 +682,7 @@ int g_attn_form = kFormAuto;
 constexpr int kKeySplitMaxGroupsPerCu = 2;
 constexpr int kKeySplitMinQueryBlocks = 4;
 
-int pick_form(int64_t two_row_groups, int nQ) {
-  if (g_attn_form != kFormAuto) return g_attn_form;
+int compute_units() {
   static int cus = 0;
   if (cus == 0) {
     int dev = 0, n = 0;
@@ -602,7 +690,26 @@ int pick_form(int64_t two_row_groups, int nQ) {
       n = 256;
     cus = n;
   }
-  return (nQ >= kKeySplitMinQueryBlocks && two_row_groups <= (int64_t)kKeySplitMaxGroupsPerCu * cus) ? kFormKeySplit : kFormTwoRows;
+  return cus;
+}
+
+int pick_form(int64_t two_row_groups, int nQ) {
+  if (g_attn_form != kFormAuto) return g_attn_form;
+  return (nQ >= kKeySplitMinQueryBlocks && two_row_groups <= (int64_t)kKeySplitMaxGroupsPerCu * compute_units()) ? kFormKeySplit : kFormTwoRows;
+}
+
+// Length-aware placement needs whole heads per XCD and a compute-unit count that splits over
+// the 8 XCDs; it is used up to 32 groups per head (the rank of a group costs one pass over the
+// head's groups per workgroup; at 64 it costs more than it gains: B1 H16 S4096 key split +6 %).
+// Measured (two rows per workgroup, zig-zag order -> length order): B8 H12 S1024 with two global
+// rows 32.8 -> 26.3 us, the same mask at B4 24.9 -> 21.3, at B16 51.3 -> 48.3; causal B4 H12
+// S1024 / S2048 / S4096 25.0 -> 21.0, 55.1 -> 43.3, 150 -> 141; growing-band B2 H16 S4096 46.3 ->
+// 46.2, at B16 346 -> 354; dense S4096 246 -> 248; eight blocks in every row 23.8 -> 24.4.
+constexpr int kBalanceMaxGroups = 32;
+void set_balance(AttnParams& p) {
+  const int cus = compute_units();
+  p.cus_per_xcd = cus / 8;
+  p.balance = (p.total % 8 == 0 && p.chunk % p.nP == 0 && p.nP <= kBalanceMaxGroups && p.nP > 1 && cus % 8 == 0 && cus >= 8) ? 1 : 0;
 }
 
 template <int KIND>
@@ -613,11 +720,13 @@ void launch_attn(AttnParams& p, int nQ, int64_t bh, hipStream_t stream) {
     p.nP = nQ;
     p.total = (int)(nQ * bh);
     p.chunk = (p.total + 7) / 8;
+    set_balance(p);
     hipLaunchKernelGGL((block_attn_fwd_kernel<KIND, 1, 2>), dim3(p.chunk * 8), dim3(256), 0, stream, p);
   } else {
     p.nP = (nQ + kRowsPerGroup - 1) / kRowsPerGroup;
     p.total = (int)two_row_groups;
     p.chunk = (p.total + 7) / 8;
+    set_balance(p);
     hipLaunchKernelGGL((block_attn_fwd_kernel<KIND, kRowsPerGroup, 1>), dim3(p.chunk * 8), dim3(128 * kRowsPerGroup), 0, stream, p);
   }
 }

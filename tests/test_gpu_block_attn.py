@@ -166,6 +166,30 @@ def test_random_block_masks(seed):
     _close(got, torch.from_numpy(blk), f"random seed {seed} (block oracle)")
 
 
+@pytest.mark.parametrize("b,h,s,seed", [(2, 4, 1024, 20), (4, 4, 512, 21), (1, 8, 192, 22), (8, 2, 2048, 23)])
+def test_length_ordered_placement(b, h, s, seed):
+    """Batch x heads a multiple of 8: workgroups take their query blocks in descending order of
+    LUT row length (ranked inside the kernel).  Rows of very different and of equal lengths, an
+    empty row, an odd block count: every block must still be computed exactly once."""
+    rng = np.random.default_rng(seed)
+    n = s // 64
+    blk = np.zeros((n, n), dtype=bool)
+    for r in range(n):
+        cnt = int(rng.choice([0, 1, 2, n // 2, n]))        # many ties, some empty, some full rows
+        blk[r, rng.choice(n, size=cnt, replace=False)] = True
+    mask = torch.from_numpy(np.kron(blk, np.ones((64, 64), dtype=np.float32)))
+    holes = torch.from_numpy((rng.random((s, s)) < 0.9).astype(np.float32))
+    part = torch.from_numpy(np.kron(rng.random((n, n)) < 0.3, np.ones((64, 64), dtype=np.float32)))
+    mask = mask * (1 - part) + mask * part * holes          # a third of the blocks become partial
+    print(f"placement b{b} h{h} s{s} rows {blk.sum(1).tolist()}", flush=True)
+    q, k, v = _inputs(b, h, s, seed=seed)
+    got = _run(q, k, v, mask)
+    _close(got, _oracle(q, k, v, mask), "length-ordered placement")
+    per_sample = torch.stack([mask if i % 2 == 0 else torch.flip(mask, dims=(0,)) for i in range(b)])
+    lut = pm.get_sparse_storage_batched(per_sample.float().cuda(), 64, 64)[1:]
+    _close(block_attn(q, k, v, lut), _oracle(q, k, v, per_sample), "length-ordered placement, LUT per sample")
+
+
 @pytest.mark.parametrize("S", [64, 192])
 def test_single_and_odd_query_block_counts(S):
     """One query block, and a block count that leaves the last two-row workgroup half empty."""
