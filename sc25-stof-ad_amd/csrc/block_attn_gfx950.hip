@@ -30,7 +30,9 @@
 //    64-bit row mask (512 B per tile instead of the reference's 8 KB additive fp16 tile),
 //    empty tiles are never visited; the LUT row is fetched once into registers;
 //  * workgroup ids are remapped so that all query blocks of one (batch, head) run on one
-//    XCD (K/V stay in that XCD's L2) and long LUT rows start first.
+//    XCD (K/V stay in that XCD's L2), and the groups of an XCD are taken in descending order
+//    of LUT row length, ranked inside the kernel, and dealt evenly over its compute units;
+//    at every step a wave's issue priority follows the number of key blocks it has left.
 #include "stof_common.h"
 
 namespace {
