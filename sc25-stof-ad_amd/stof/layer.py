@@ -42,10 +42,17 @@ class EncoderLayer:
     def _fuse(self, M):
         if self.ln_fusion in ("fused", "split"):
             return self.ln_fusion == "fused"
-        # One workgroup per 64 rows streams the whole weight matrix: below ~2 workgroups per CU
-        # the fused kernel cannot fill the 256 CUs and the tiled GEMM + LayerNorm kernel is
-        # faster (measured at M = 8192 for hidden 768 and 1024).
-        return self.hidden <= 768 and M >= 64 * 256
+        # One workgroup per 64 rows streams the whole weight matrix, so the fused kernel needs many
+        # row blocks per compute unit (or a small matrix) to beat the tiled GEMM followed by the
+        # LayerNorm kernel.  Measured on MI355X for N = K and N = K / 4: hidden 256 fused wins from
+        # 2048 rows up (10 vs 19 us at 8192); hidden 512 from 32768 rows; hidden 768 / 1024 from
+        # 65536 rows (513 vs 640 us, 915 vs 1188 us at K = 4N), below that the split form wins
+        # (hidden 768, 8192 rows: 41 vs 28 us and 109 vs 60 us).
+        if self.hidden <= 256:
+            return True
+        if self.hidden <= 512:
+            return M >= 32768
+        return M >= 65536
 
     def _gemm_ln(self, x, Wt, bias, residual, gamma, beta):
         M = x.numel() // x.shape[-1]
