@@ -82,7 +82,8 @@ const char* stof_status_string(int status);
  * LUT arrays are int32.  With lut_batch_stride == 0 the three row-pointer arrays have
  * S/block_m + 1 entries and are shared by every (b,h) as in the reference; otherwise
  * sample b uses row pointers at offset b*lut_batch_stride, whose values are absolute
- * offsets into the (concatenated) column lists and bitmask slots.
+ * offsets into the (concatenated) column lists and bitmask slots.  A column list or the bitmask
+ * may be NULL when every row range over it is empty (no partial blocks; nothing allowed at all).
  *
  * Supported: D == 64, block_m == block_n == 64, S % 64 == 0 (the Python operator re-tiles LUTs
  * built with other block sizes to 64 x 64 before it calls this).  num_warps of the reference

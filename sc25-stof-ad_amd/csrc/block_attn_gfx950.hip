@@ -758,14 +758,14 @@ extern "C" int stof_block_attn_fwd(
   if (!q || !k || !v || !out || !full_row_ptr || !part_row_ptr || !load_row_ptr ||
       !q_strides || !k_strides || !v_strides || !out_strides)
     return STOF_ERR_NULL_POINTER;
-  // column lists / bitmask may legitimately be empty, but then must still be addressable
-  // by the kernel's scalar loads only when their row ranges are non-empty; NULL is accepted.
+  // The column lists and the bitmask may be NULL when every row range over them is empty (a
+  // mask without partial blocks; a mask that allows nothing, whose output is all zeros): the
+  // kernel reads them only inside non-empty row ranges.
   if (batch_size <= 0 || seq_len <= 0 || head_num <= 0 || head_size <= 0) return STOF_ERR_BAD_SHAPE;
   if (head_size != kD || block_m != kBM || block_n != kBN) return STOF_ERR_UNSUPPORTED;
   if (seq_len % kBM != 0) return STOF_ERR_BAD_SHAPE;
   const int nQ = seq_len / kBM;
   if (lut_batch_stride != 0 && lut_batch_stride < nQ + 1) return STOF_ERR_BAD_LUT;
-  if (!load_col_idx) return STOF_ERR_NULL_POINTER;
   if (!stof_aligned16(q) || !stof_aligned16(k) || !stof_aligned16(v) || !stof_aligned16(out)) return STOF_ERR_MISALIGNED;
   if (!strides_ok(q_strides) || !strides_ok(k_strides) || !strides_ok(v_strides) || !strides_ok(out_strides))
     return STOF_ERR_MISALIGNED;

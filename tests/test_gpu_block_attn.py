@@ -190,6 +190,14 @@ def test_length_ordered_placement(b, h, s, seed):
     _close(block_attn(q, k, v, lut), _oracle(q, k, v, per_sample), "length-ordered placement, LUT per sample")
 
 
+def test_mask_that_allows_nothing_gives_zeros():
+    """Every LUT row empty: the column lists have no entries at all (NULL at the C boundary)."""
+    for b, h, s in ((1, 2, 64), (2, 4, 256)):
+        q, k, v = _inputs(b, h, s, seed=30)
+        got = _run(q, k, v, torch.zeros(s, s))
+        assert bool((got == 0).all())
+
+
 @pytest.mark.parametrize("S", [64, 192])
 def test_single_and_odd_query_block_counts(S):
     """One query block, and a block count that leaves the last two-row workgroup half empty."""
