@@ -45,6 +45,7 @@ class GPUParams:
         self.l2_per_xcd = 4 * 1024 * 1024
         self.lds_per_group = 4 * BLOCK * 64 * 2      # K and V tiles, double buffered: 32 KB
         self.waves_per_group = 4
+        self.resident_groups_per_cu = 4   # measured: the fifth 32 KB group does not become resident
         # launch-form rule (kKeySplitMaxGroupsPerCu / kKeySplitMinQueryBlocks in the kernel source)
         self.key_split_max_groups_per_cu = 2
         self.key_split_min_query_blocks = 4
@@ -87,7 +88,7 @@ def phase2_selection(gpu, seq_len, batch_size, head_num):
     nq = seq_len // BLOCK
     groups = ((nq + 1) // 2) * batch_size * head_num
     per_cu = groups / gpu.cu_count
-    resident = min(gpu.lds_per_cu // gpu.lds_per_group, gpu.max_waves_per_simd)
+    resident = gpu.resident_groups_per_cu
     if nq >= gpu.key_split_min_query_blocks and groups <= gpu.key_split_max_groups_per_cu * gpu.cu_count:
         return ("key_split", per_cu,
                 f"{per_cu:.2f} two-row workgroups per compute unit (<= {gpu.key_split_max_groups_per_cu}, "

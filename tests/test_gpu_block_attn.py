@@ -297,3 +297,16 @@ def test_pack_mask_bits_vector_and_scalar_paths(additive):
     assert rc == 0
     torch.cuda.synchronize()
     assert np.array_equal(_unpack_bits(dst, cols), keep.numpy())
+
+
+@pytest.mark.parametrize("mask", ["causal", "bigbird", "sliding"])
+def test_example_script_runs(mask):
+    """The example that follows the reference's unified attention benchmark, end to end."""
+    import subprocess, sys, os
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    script = os.path.join(root, "sc25-stof-ad_amd", "examples", "unified_attention.py")
+    r = subprocess.run([sys.executable, script, "--mask", mask, "--batch", "2", "--heads", "4", "--seq", "512", "--iters", "5"],
+                       capture_output=True, text=True, timeout=110)
+    assert r.returncode == 0, r.stdout + r.stderr
+    line = [l for l in r.stdout.splitlines() if l.startswith("max abs difference")][0]
+    assert float(line.split(":")[1]) < 5e-3, r.stdout
