@@ -532,7 +532,7 @@ __device__ __forceinline__ int zigzag(int pidx, int bh, int n) {
 // boustrophedon order: pass 0 hands units 0..n-1 the first n groups, pass 1 hands units n-1..0
 // the next n, and so on.  Sums per unit come out even and every unit starts with its longest
 // chain.  The rank is computed here from the row pointers (lane l holds group l of the head; at
-// most 32 groups), so no host pass over the LUT and no scratch memory is needed; being a
+// most 64 groups), so no host pass over the LUT and no scratch memory is needed; being a
 // permutation per head it is a bijection also when every sample has its own LUT.  The row
 // pointers read for it are handed on to attn_group, which saves that a memory round trip.
 template <int KIND, int ROWS>
@@ -701,17 +701,20 @@ int pick_form(int64_t two_row_groups, int nQ) {
 }
 
 // Length-aware placement needs whole heads per XCD and a compute-unit count that splits over
-// the 8 XCDs; it is used up to 32 groups per head (the rank of a group costs one pass over the
-// head's groups per workgroup; at 64 it costs more than it gains: B1 H16 S4096 key split +6 %).
+// the 8 XCDs.  The rank of a group costs one pass over the head's groups per workgroup: with two
+// rows per workgroup it is used up to 64 groups per head (S 8192; one lane per group), with the
+// key split - small grids, short kernels - up to 32 (at 64: B1 H16 S4096 +6 %).
 // Measured (two rows per workgroup, zig-zag order -> length order): B8 H12 S1024 with two global
 // rows 32.8 -> 26.3 us, the same mask at B4 24.9 -> 21.3, at B16 51.3 -> 48.3; causal B4 H12
 // S1024 / S2048 / S4096 25.0 -> 21.0, 55.1 -> 43.3, 150 -> 141; growing-band B2 H16 S4096 46.3 ->
-// 46.2, at B16 346 -> 354; dense S4096 246 -> 248; eight blocks in every row 23.8 -> 24.4.
-constexpr int kBalanceMaxGroups = 32;
-void set_balance(AttnParams& p) {
+// 46.2, at B16 346 -> 354; dense S4096 246 -> 248; eight blocks in every row 23.8 -> 24.4; B2 H16
+// S8192 band + two global rows + random blocks 178 -> 159, causal 350 -> 350.
+constexpr int kBalanceMaxGroupsTwoRows = 64;
+constexpr int kBalanceMaxGroupsKeySplit = 32;
+void set_balance(AttnParams& p, int max_groups) {
   const int cus = compute_units();
   p.cus_per_xcd = cus / 8;
-  p.balance = (p.total % 8 == 0 && p.chunk % p.nP == 0 && p.nP <= kBalanceMaxGroups && p.nP > 1 && cus % 8 == 0 && cus >= 8) ? 1 : 0;
+  p.balance = (p.total % 8 == 0 && p.chunk % p.nP == 0 && p.nP <= max_groups && p.nP > 1 && cus % 8 == 0 && cus >= 8) ? 1 : 0;
 }
 
 template <int KIND>
@@ -722,13 +725,13 @@ void launch_attn(AttnParams& p, int nQ, int64_t bh, hipStream_t stream) {
     p.nP = nQ;
     p.total = (int)(nQ * bh);
     p.chunk = (p.total + 7) / 8;
-    set_balance(p);
+    set_balance(p, kBalanceMaxGroupsKeySplit);
     hipLaunchKernelGGL((block_attn_fwd_kernel<KIND, 1, 2>), dim3(p.chunk * 8), dim3(256), 0, stream, p);
   } else {
     p.nP = (nQ + kRowsPerGroup - 1) / kRowsPerGroup;
     p.total = (int)two_row_groups;
     p.chunk = (p.total + 7) / 8;
-    set_balance(p);
+    set_balance(p, kBalanceMaxGroupsTwoRows);
     hipLaunchKernelGGL((block_attn_fwd_kernel<KIND, kRowsPerGroup, 1>), dim3(p.chunk * 8), dim3(128 * kRowsPerGroup), 0, stream, p);
   }
 }

@@ -217,6 +217,11 @@ def test_long_sequence_walks_several_column_windows():
     q, k, v = _inputs(1, 2, S, seed=9)
     got = _run(q, k, v, mask.float())
     _close(got, _oracle(q, k, v, mask.float()), "S 8192")
+    # 8 heads: whole heads per XCD, so the 64 pairs of query blocks of a head are taken in length
+    # order (two rows per workgroup; with the key split 128 rows exceed the limit: plain order)
+    q, k, v = _inputs(1, 8, S, seed=10)
+    got = _run(q, k, v, mask.float())
+    _close(got, _oracle(q, k, v, mask.float()), "S 8192, 8 heads")
 
 
 @pytest.mark.parametrize("bm,bn", [(16, 16), (32, 32), (128, 128), (32, 64), (64, 16), (128, 32)])
