@@ -41,7 +41,6 @@ constexpr int kD = 64;        // head size
 constexpr int kBM = 64;       // query rows per block
 constexpr int kBN = 64;       // keys per block
 constexpr int kTile = kBN * kD * 2;   // bytes of one K or V tile in LDS (8 KB, unpadded)
-constexpr float kMasked = -INFINITY;  // score given to a masked element
 constexpr float kLazy = 8.0f;         // log2 slack before the running max is raised
 constexpr int kPrioStep = 6;          // key blocks of remaining chain per issue-priority level
 
@@ -361,28 +360,40 @@ __device__ __forceinline__ void attn_group(const AttnParams& p, const int bh, co
     }
 
     // ---- S^T = K . Q^T : sacc[mt][r] = S[query j32][key 32mt + 8(r/4) + 4g + r%4]
+    // A partial tile applies its element mask through the accumulator's INITIAL value: 0 where
+    // the key is allowed, -inf where it is not (-inf + finite = -inf), two instructions per
+    // element (sign-extended one-bit field of the inverted mask word, AND with the bit pattern
+    // of -inf) instead of test + compare + select after the product.  The two cases run their
+    // own copy of the product so that the unmasked one keeps the constant-zero accumulator input.
     floatx16 sacc[kMT];
+    auto s_product = [&]() {
 #pragma unroll
-    for (int i = 0; i < kMT; ++i)
+      for (int ks = 0; ks < 4; ++ks)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) sacc[i][r] = 0.f;
-#pragma unroll
-    for (int ks = 0; ks < 4; ++ks)
-#pragma unroll
-      for (int mt = 0; mt < kMT; ++mt) {
-        const half8_t a = *reinterpret_cast<const __attribute__((address_space(3))) half8_t*>(kt + (mt0 + mt) * 4096 + k_rd[ks]);
-        sacc[mt] = mfma32(a, qf[ks], sacc[mt]);
-      }
-
-    // ---- element mask of a partial tile
+        for (int mt = 0; mt < kMT; ++mt) {
+          const half8_t a = *reinterpret_cast<const __attribute__((address_space(3))) half8_t*>(kt + (mt0 + mt) * 4096 + k_rd[ks]);
+          sacc[mt] = mfma32(a, qf[ks], sacc[mt]);
+        }
+    };
     if (need_mask) {
 #pragma unroll
       for (int mt = 0; mt < kMT; ++mt) {
-        const uint32_t w = (uint32_t)(bits >> (32 * (mt0 + mt))) >> (4 * g);
+        const uint32_t nw = ~((uint32_t)(bits >> (32 * (mt0 + mt))) >> (4 * g));   // bit set = key masked
 #pragma unroll
-        for (int r = 0; r < 16; ++r)
-          if (!((w >> (8 * (r >> 2) + (r & 3))) & 1u)) sacc[mt][r] = kMasked;
+        for (int r = 0; r < 16; ++r) {
+          // (asm: written with the builtin, the compiler turns the pair back into and + compare + select)
+          int all;   // -1 if masked, else 0
+          asm("v_bfe_i32 %0, %1, %2, 1" : "=v"(all) : "v"(nw), "n"(8 * (r >> 2) + (r & 3)));
+          sacc[mt][r] = __builtin_bit_cast(float, (uint32_t)all & 0xFF800000u);
+        }
       }
+      s_product();
+    } else {
+#pragma unroll
+      for (int i = 0; i < kMT; ++i)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) sacc[i][r] = 0.f;
+      s_product();
     }
 
     // ---- online softmax; one query per lane (shared with the partner lane ^ 32).
