@@ -110,7 +110,8 @@ def launch_form(request):
     set_attention_launch_form("auto")
 
 
-@pytest.mark.parametrize("B,H,S", [(2, 12, 256), (1, 3, 128), (1, 12, 576)])
+# (2, 4, 1024): batch x heads a multiple of 8, so query blocks are taken in length order (8 or 16 groups)
+@pytest.mark.parametrize("B,H,S", [(2, 12, 256), (1, 3, 128), (1, 12, 576), (2, 4, 1024)])
 def test_rowwise_ops(B, H, S, launch_form):
     cfg = configs.AttnConfig("t", B, H, S)
     q, k, v = configs.qkv(cfg, seed=22, device="cuda")
