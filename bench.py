@@ -3,9 +3,10 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-extras] [--no-cpu]
 
-One "step" is one launch of block-masked multi-head attention on workload C2 (fp16,
-B8 H12 S1024 D64, banded + global + random key blocks, 129 active 64x64 blocks), inputs
-resident in HBM.  The timed region is K steps between device synchronisations; the same
+One "step" is one launch of block-masked multi-head attention on workload C4 (fp16,
+B2 H16 S4096 D64, causal sliding window of 512 plus every fourth key block, 946 active 64x64
+blocks of 4096: the largest single-GPU attention workload and the one the MFMA target is
+quoted on), inputs resident in HBM.  The timed region is K steps between device synchronisations; the same
 region is bracketed by HIP events on the launch stream for the per-launch kernel time that
 the roofline figure uses.  One JSON line is printed:
 
@@ -14,9 +15,10 @@ the roofline figure uses.  One JSON line is printed:
   roofline     the attention kernel against the MI355X dense fp16 MFMA peak (2.5 PFLOP/s)
   cpu_baseline the reference's PyTorch-native dense attention (restated in oracle/) timed on
                this machine's host cores on the same workload, in the same unit
-  also         the other workloads: C1 (S512, with the host fp32 reference), C4 (S4096 long-sequence
-               MHA), the C3 BERT-base encoder layer and the C5 24-layer stack (fused vs PyTorch-ROCm
-               eager, ms, per-stage breakdown for C3), the HBM-bound kernels and the LUT build
+  also         the other workloads: C1 (S512, with the host fp32 reference), C2 (B8 H12 S1024), the
+               C3 BERT-base encoder layer and the C5 24-layer stack (fused vs PyTorch-ROCm eager,
+               ms, per-stage breakdown for C3, output checked against the eager result), the
+               HBM-bound kernels and the LUT build
 """
 import argparse
 import json
@@ -34,9 +36,25 @@ PEAK_FP16_TFLOPS = 2500.0     # MI355X dense fp16 matrix peak (published)
 PEAK_HBM_GBS = 8000.0         # MI355X HBM3E peak (published)
 FLOP_PER_BLOCK = 4 * 64 * 64 * 64
 
-# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (two runs),
-# scaled by the same counters on a 256 MiB fill + copy in the same run (profiles/block_attn_C2_hbm_traffic.txt).
-MEASURED_TRAFFIC_BYTES = {"C2": 50.5e6}   # fetch 37.9 MB + write 12.6 MB; algorithmic minimum 50.3 MB
+# HBM bytes per launch of the headline kernel come from two counter runs of this script
+# (rocprofv3 --pmc FETCH_SIZE, then WRITE_SIZE, each scaled by the same counter on the 256 MiB
+# copy of --copy-probe); their summary is a text file under profiles/ whose line
+# "traffic_bytes_per_launch: <bytes>" is read here, so the figure reported is the one the
+# committed profile holds and names its source.
+TRAFFIC_PROFILE = os.path.join("profiles", "block_attn_C4_hbm_traffic.txt")
+
+
+def measured_traffic():
+    """(bytes per launch, source) from the committed counter summary, or (None, reason)."""
+    path = os.path.join(ROOT, TRAFFIC_PROFILE)
+    try:
+        with open(path) as f:
+            for line in f:
+                if line.startswith("traffic_bytes_per_launch:"):
+                    return float(line.split(":", 1)[1].split()[0]), TRAFFIC_PROFILE
+    except OSError:
+        pass
+    return None, f"{TRAFFIC_PROFILE} not found or without a traffic_bytes_per_launch line"
 
 
 def attn_setup(cfg, mask_fn, device):
@@ -87,7 +105,7 @@ def bench_attn(cfg, mask_fn, steps, warmup, settle_ms=SETTLE_MS):
             "tflops_wall": flop / wall_ms / 1e9, "tflops_kernel": flop / ev_ms / 1e9}
 
 
-def cpu_baseline_attn(cfg, mask_fn, n_active, budget_s=12.0, max_iters=20):
+def cpu_baseline_attn(cfg, mask_fn, n_active, budget_s=12.0, max_iters=20, min_iters=3):
     """The reference's dense PyTorch attention (oracle.attention.torch_attn_std) in fp32 on the
     host cores; bounded sample of whole-workload iterations."""
     from oracle import attention as oa
@@ -100,15 +118,31 @@ def cpu_baseline_attn(cfg, mask_fn, n_active, budget_s=12.0, max_iters=20):
     mask = mask_fn(cfg.seq).float()[None]
     oa.torch_attn_std(q, k, v, mask)           # warm-up
     iters, t0 = 0, time.perf_counter()
-    while iters < max_iters and (time.perf_counter() - t0) < budget_s:
+    while iters < min_iters or (iters < max_iters and (time.perf_counter() - t0) < budget_s):
         oa.torch_attn_std(q, k, v, mask)
         iters += 1
     dt = (time.perf_counter() - t0) / iters
     flop = FLOP_PER_BLOCK * cfg.batch * cfg.heads * n_active
     return {"value": flop / dt / 1e12, "unit": "TFLOP/s", "cores": cores, "kind": "port",
             "ms_per_step": dt * 1e3,
-            "sample": f"{iters} full passes of the {cfg.name} workload (dense fp32 softmax(QK^T/8 - 10000(1-M))V, "
-                      f"B{cfg.batch} H{cfg.heads} S{cfg.seq} D64), active-block FLOPs / time"}
+            "sample": f"1 warm-up + {iters} timed full passes of the {cfg.name} workload (dense fp32 "
+                      f"softmax(QK^T/8 - 10000(1-M))V, B{cfg.batch} H{cfg.heads} S{cfg.seq} D64, scores materialised), "
+                      f"active-block FLOPs / time"}
+
+
+def output_check(got, want_eager, valid=None, bound=5e-2):
+    """The timed path's output against PyTorch-ROCm's eager fp16 result on the same inputs: a
+    guard against timing a path that computes something else, not the parity test (the
+    eager layer rounds to fp16 at more points than the fused one; parity against the oracle
+    is asserted in tests/).  Rows a padding mask leaves without keys are excluded."""
+    d = (got.float() - want_eager.float()).abs()
+    if valid is not None:
+        d = d[valid]
+    m = float(d.max())
+    ok = bool(torch.isfinite(got.float()).all()) and m <= bound
+    if not ok:
+        raise RuntimeError(f"bench output check failed: max |fused - eager| = {m:.3e} (bound {bound})")
+    return {"max_abs_diff_vs_eager": m, "bound": bound, "ok": ok}
 
 
 def bench_layer_c3(steps, warmup):
@@ -118,20 +152,25 @@ def bench_layer_c3(steps, warmup):
     cfg = configs.C3
     w = {k: v.cuda() for k, v in configs.layer_weights(cfg.hidden, cfg.ffn, seed=0).items()}
     x = configs.layer_input(cfg, seed=1, device="cuda")
-    mask, _ = configs.mask_c3(cfg.batch, cfg.seq, 256, seed=0)
+    mask, L = configs.mask_c3(cfg.batch, cfg.seq, 256, seed=0)
     maskg = mask.cuda().half()
     lut = pm.get_sparse_storage_batched(mask.float().cuda(), 64, 64)[1:]
     out = {}
-    for fusion in ("fused", "split"):
+    for fusion in ("auto", "fused", "split"):
         layer = EncoderLayer(w, cfg.heads, eps=cfg.eps, ln_fusion=fusion)
-        layer(x, lut)
+        y = layer(x, lut)
         out[fusion + "_ms"], _ = time_region(lambda: layer(x, lut), steps, warmup)
+        if fusion == "auto":
+            out["auto_runs"] = "fused" if layer._fuse(cfg.batch * cfg.seq) else "split"
+            y_auto = y
     with torch.no_grad():
+        y_eager = eager_layer(x, w, maskg, cfg.heads, cfg.eps)
         out["eager_ms"], _ = time_region(lambda: eager_layer(x, w, maskg, cfg.heads, cfg.eps), max(steps // 4, 5), 5)
-    layer = EncoderLayer(w, cfg.heads, eps=cfg.eps, ln_fusion="split")
+    out["output_check"] = output_check(y_auto, y_eager, valid=(torch.arange(cfg.seq)[None, :] < L[:, None]).cuda())
+    layer = EncoderLayer(w, cfg.heads, eps=cfg.eps, ln_fusion="auto")
     out["stages_ms"] = {name: time_region(fn, steps, warmup)[1] for name, fn in layer.stages(x, lut)}
     out["layer_ms_without_qkv_gemm"] = sum(v for k, v in out["stages_ms"].items() if k != "qkv_gemm")
-    best = min(out["fused_ms"], out["split_ms"])
+    best = out["auto_ms"]                      # what ln_fusion="auto", the default, runs
     out["layer_ms"] = best
     out["speedup_vs_eager"] = out["eager_ms"] / best
     flop = 2 * cfg.batch * cfg.seq * cfg.hidden * (3 * cfg.hidden + cfg.hidden + 2 * cfg.ffn)
@@ -199,7 +238,7 @@ def bench_stack_c5(steps, warmup):
     mask = configs.mask_c5(cfg.seq)
     lut = pm.get_sparse_storage(mask.float()[None].cuda(), 64, 64)[1:]
     stack = EncoderStack(ws, cfg.heads, eps=cfg.eps)
-    stack(x, lut)
+    y = stack(x, lut)
     ms, _ = time_region(lambda: stack(x, lut), steps, warmup)
     maskg = mask.half()[None].cuda()
 
@@ -209,10 +248,11 @@ def bench_stack_c5(steps, warmup):
             h = eager_layer(h, w, maskg, cfg.heads, cfg.eps)
         return h
     with torch.no_grad():
+        check = output_check(y, eager(), bound=1e-1)     # 24 chained fp16 layers on both sides
         eager_ms, _ = time_region(eager, max(steps // 2, 3), 2)
     gemm_flop = 2 * cfg.batch * cfg.seq * cfg.hidden * (3 * cfg.hidden + cfg.hidden + 2 * cfg.ffn) * cfg.layers
     return {"stack_ms": ms, "ms_per_layer": ms / cfg.layers, "eager_ms": eager_ms, "speedup_vs_eager": eager_ms / ms,
-            "gemm_tflops_at_stack_ms": gemm_flop / ms / 1e9, "layers": cfg.layers}
+            "gemm_tflops_at_stack_ms": gemm_flop / ms / 1e9, "layers": cfg.layers, "output_check": check}
 
 
 def bench_dense_vs_sdpa(steps, warmup):
@@ -293,8 +333,8 @@ def main():
     ap.add_argument("--steps", type=int, default=2000)
     ap.add_argument("--warmup", type=int, default=2000,
                     help="untimed steps before the timed ones; the default (about 70 ms of load) lets the clocks settle")
-    ap.add_argument("--no-extras", action="store_true", help="skip everything but the C2 attention step")
-    ap.add_argument("--extras", default="c1,c4,c4big,dense,c3,c3small,c5,hbm,lut",
+    ap.add_argument("--no-extras", action="store_true", help="skip everything but the C4 attention step")
+    ap.add_argument("--extras", default="c1,c2,c4big,dense,c3,c3small,c5,hbm,lut",
                     help="comma-separated subset of the extra workloads to run (for profiling one kind of kernel)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--copy-probe", action="store_true",
@@ -316,29 +356,31 @@ def main():
         dst = torch.empty_like(src)
         dst.copy_(src)
         torch.cuda.synchronize()
-    c2 = bench_attn(configs.C2, configs.mask_c2, args.steps, args.warmup, settle_ms=0)   # exactly W warm-up steps, then K timed
+    c4 = bench_attn(configs.C4, configs.mask_c4, args.steps, args.warmup, settle_ms=0)   # exactly W warm-up steps, then K timed
+    traffic, traffic_source = measured_traffic()
     line = {
         "metric": "masked-MHA TFLOP/s (active blocks) + encoder-layer ms, fp16, 1xMI355X",
-        "value": c2["tflops_wall"], "unit": "TFLOP/s",
-        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": c2["wall_ms"],
+        "value": c4["tflops_wall"], "unit": "TFLOP/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": c4["wall_ms"],
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f16", "data": "synthetic",
-        "config": {"workload": "C2: block-masked MHA, B8 H12 S1024 D64, band 3 + 2 global + 3 random key blocks "
-                               "per 64-row query block", "active_blocks": c2["active_blocks"], "block": 64,
-                   "flop_per_step": c2["flop"]},
-        "roofline": {"bound": "mfma", "achieved": c2["tflops_kernel"], "peak": PEAK_FP16_TFLOPS, "unit": "TFLOP/s",
-                     "frac": c2["tflops_kernel"] / PEAK_FP16_TFLOPS, "traffic": MEASURED_TRAFFIC_BYTES["C2"],
-                     "kernel": "block_attn_fwd_kernel", "kernel_ms": c2["kernel_ms"]},
+        "config": {"workload": "C4: long-sequence block-masked MHA, B2 H16 S4096 D64, causal sliding window of 512 + "
+                               "every 4th key block, 64 x 64 blocks", "active_blocks": c4["active_blocks"],
+                   "blocks_total": (configs.C4.seq // 64) ** 2, "block": 64, "flop_per_step": c4["flop"]},
+        "roofline": {"bound": "mfma", "achieved": c4["tflops_kernel"], "peak": PEAK_FP16_TFLOPS, "unit": "TFLOP/s",
+                     "frac": c4["tflops_kernel"] / PEAK_FP16_TFLOPS, "traffic": traffic, "traffic_source": traffic_source,
+                     "algorithmic_bytes": 4 * configs.C4.batch * configs.C4.heads * configs.C4.seq * 64 * 2,
+                     "kernel": "block_attn_fwd_kernel", "kernel_ms": c4["kernel_ms"]},
     }
     if not args.no_cpu:
-        line["cpu_baseline"] = cpu_baseline_attn(configs.C2, configs.mask_c2, c2["active_blocks"])
+        line["cpu_baseline"] = cpu_baseline_attn(configs.C4, configs.mask_c4, c4["active_blocks"])
     if not args.no_extras:
         also = {}
         want = set(args.extras.split(","))
-        if "c4" in want:
-            c4 = bench_attn(configs.C4, configs.mask_c4, args.steps, args.warmup)
-            also["C4_mha_S4096"] = {"tflops": c4["tflops_kernel"], "frac_mfma_peak": c4["tflops_kernel"] / PEAK_FP16_TFLOPS,
-                                    "kernel_ms": c4["kernel_ms"], "active_blocks": c4["active_blocks"]}
+        if "c2" in want:
+            c2 = bench_attn(configs.C2, configs.mask_c2, args.steps, args.warmup)
+            also["C2_mha_S1024"] = {"tflops": c2["tflops_kernel"], "frac_mfma_peak": c2["tflops_kernel"] / PEAK_FP16_TFLOPS,
+                                    "kernel_ms": c2["kernel_ms"], "active_blocks": c2["active_blocks"]}
         if "c4big" in want:
             big = configs.AttnConfig("C4x8", 16, 16, 4096)
             c4b = bench_attn(big, configs.mask_c4, max(args.steps // 4, 10), 5)

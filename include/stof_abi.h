@@ -40,7 +40,7 @@
 extern "C" {
 #endif
 
-#define STOF_ABI_VERSION 1
+#define STOF_ABI_VERSION 2
 
 enum {
   STOF_OK = 0,
@@ -54,6 +54,9 @@ enum {
 
 /* activation selector of stof_gemm_bias_act */
 enum { STOF_ACT_NONE = 0, STOF_ACT_GELU_ERF = 1, STOF_ACT_GELU_TANH = 2, STOF_ACT_RELU = 3 };
+
+/* launch form of the attention entry points */
+enum { STOF_FORM_DEFAULT = -1, STOF_FORM_TWO_ROWS = 0, STOF_FORM_KEY_SPLIT = 1 };
 
 /* rowwise front-end selector of stof_rowwise_attn_fwd */
 enum { STOF_ROW_FULL = 0, STOF_ROW_SLIDING = 1, STOF_ROW_MASK = 2 };
@@ -86,8 +89,18 @@ const char* stof_status_string(int status);
  * may be NULL when every row range over it is empty (no partial blocks; nothing allowed at all).
  *
  * Supported: D == 64, block_m == block_n == 64, S % 64 == 0 (the Python operator re-tiles LUTs
- * built with other block sizes to 64 x 64 before it calls this).  num_warps of the reference
- * launcher has no per-call counterpart: see stof_attn_set_launch_form.
+ * built with other block sizes to 64 x 64 before it calls this).
+ *
+ * launch_form is the per-call counterpart of the reference launcher's num_warps (its kernel
+ * selection by (num_warps, BLOCK_M, BLOCK_N), block_attn_mask_cuda.cu:6064-6322):
+ *   STOF_FORM_DEFAULT (-1) the process default (automatic by grid size unless
+ *                          stof_attn_set_launch_form changed it);
+ *   STOF_FORM_TWO_ROWS (0) two query blocks per workgroup, K/V tiles shared by four wavefronts
+ *                          (large grids);
+ *   STOF_FORM_KEY_SPLIT (1) one query block per workgroup, the 64 keys of every tile split over
+ *                          two wavefront pairs whose partial results are merged at the end
+ *                          (small grids).
+ * Results are equal within rounding in every form; another value returns STOF_ERR_UNSUPPORTED.
  */
 int stof_block_attn_fwd(
     const void* q, const void* k, const void* v, void* out,
@@ -98,17 +111,13 @@ int stof_block_attn_fwd(
     const int64_t q_strides[3], const int64_t k_strides[3],
     const int64_t v_strides[3], const int64_t out_strides[3],
     int batch_size, int seq_len, int head_num, int head_size,
-    int64_t lut_batch_stride, void* stream);
+    int64_t lut_batch_stride, int launch_form, void* stream);
 
 /*
- * Launch form of the two attention entry points, process-wide:
- *   -1 automatic (default): chosen from the grid size per call;
- *    0 two query blocks per workgroup, K/V tiles shared by four wavefronts (large grids);
- *    1 one query block per workgroup, the 64 keys of every tile split over two wavefront
- *      pairs whose partial results are merged at the end (small grids).
- * Results are equal within rounding in every form.  This is the counterpart of the
- * reference's kernel selection by (num_warps, BLOCK_M, BLOCK_N), block_attn_mask_cuda.cu:6064-6322,
- * there an argument of every call.  Returns STOF_ERR_UNSUPPORTED for another value.
+ * Process-wide default launch form, used by calls that pass STOF_FORM_DEFAULT: -1 automatic
+ * (the initial state), 0 / 1 as above.  A convenience for harnesses that sweep the forms
+ * without touching their call sites; calls that name a form are not affected by it.
+ * Returns STOF_ERR_UNSUPPORTED for another value.
  */
 int stof_attn_set_launch_form(int form);
 
@@ -130,11 +139,12 @@ int stof_pack_mask_bits(const void* src, uint64_t* dst, int64_t rows, int64_t co
  *   kind STOF_ROW_MASK:    additionally bit j of mask_bits[i*(S/64) + j/64] set
  * Unlike the reference kernels the softmax is max-subtracted (no overflow) and rows
  * without an allowed key produce zeros.  q, k, v contiguous [B,H,S,D], D == 64, S % 64 == 0.
+ * launch_form as for stof_block_attn_fwd.
  */
 int stof_rowwise_attn_fwd(
     const void* q, const void* k, const void* v, void* out,
     int kind, int is_causal, int bandwidth, const uint64_t* mask_bits,
-    int batch_size, int seq_len, int head_num, int head_size, void* stream);
+    int batch_size, int seq_len, int head_num, int head_size, int launch_form, void* stream);
 
 /*
  * y[m,:] = LayerNorm(x[m,:] + bias[:] + residual[m,:]) * gamma + beta     (fp32 statistics)

@@ -26,6 +26,13 @@ import torch.nn.functional as F
 from .attention import dense_masked_attention
 
 
+def _r16(t, on):
+    """Round to fp16 and back: where the fp16 eager path of the reference (every tensor of
+    src/benchmk_end2end.py:31-88 is fp16 on the GPU) and the five kernels of the product store
+    a tensor between two operators."""
+    return t.to(torch.float16).to(t.dtype) if on else t
+
+
 def new_gelu(x):
     """src/benchmk_end2end.py:25-26 (tanh approximation)."""
     return 0.5 * x * (1.0 + torch.tanh(math.sqrt(2.0 / math.pi) * (x + 0.044715 * torch.pow(x, 3.0))))
@@ -84,9 +91,11 @@ def gemm_bias_act(x, W, bias, act="none", dtype=torch.float32):
     return y
 
 
-def gemm_bias_residual_layernorm(x, W, bias, residual, gamma, beta, eps=1e-5, dtype=torch.float32):
-    """src/benchmk_end2end.py:73-76 / :83-86: LN(x@W + bias + residual; gamma, beta)."""
-    y = torch.matmul(x.to(dtype), W.to(dtype)) + bias.to(dtype) + residual.to(dtype)
+def gemm_bias_residual_layernorm(x, W, bias, residual, gamma, beta, eps=1e-5, dtype=torch.float32, round_product=False):
+    """src/benchmk_end2end.py:73-76 / :83-86: LN(x@W + bias + residual; gamma, beta).
+    ``round_product`` rounds x@W to fp16 first, as the reference's fp16 ``torch.matmul`` does
+    (:73, :83) and as a GEMM kernel followed by a separate LayerNorm kernel does."""
+    y = _r16(torch.matmul(x.to(dtype), W.to(dtype)), round_product) + bias.to(dtype) + residual.to(dtype)
     return layer_norm(y, gamma.to(dtype), beta.to(dtype), eps)
 
 
@@ -95,8 +104,14 @@ def transpose_for_scores(x, n_heads, head_size):
     return x.view(x.shape[:-1] + (n_heads, head_size)).permute(0, 2, 1, 3)
 
 
-def bert_layer(x, p, mask, n_heads, eps=1e-5, gelu="erf", dtype=torch.float32):
+def bert_layer(x, p, mask, n_heads, eps=1e-5, gelu="erf", dtype=torch.float32, round_fp16=False):
     """One post-LayerNorm encoder layer, src/benchmk_end2end.py:31-88.
+
+    ``round_fp16=True`` rounds the tensors that cross an operator boundary (qkv, the attention
+    result, the first LayerNorm's output, the FFN activation, the layer output) to fp16, as
+    the reference's fp16 eager layer does at the same points; all arithmetic inside an
+    operator stays in ``dtype``.  ``round_fp16="split"`` additionally rounds the two products
+    that feed a LayerNorm (the eager layer's fp16 matmul outputs, :73 and :83).  ``gelu``: "erf" (:81), "tanh" (new_gelu, :25-26) or "relu" (:206).
 
     ``p`` is a dict of weights in the reference's [in, out] orientation:
     W_qkv [D,3D] (or None: then p['qkv_act'] [B,S,3D] plays the reference's
@@ -111,13 +126,16 @@ def bert_layer(x, p, mask, n_heads, eps=1e-5, gelu="erf", dtype=torch.float32):
         qkv = torch.matmul(x, p["W_qkv"].to(dtype)) + p["b_qkv"].to(dtype)
     else:
         qkv = p["qkv_act"].to(dtype) + p["b_qkv"].to(dtype)
+    qkv = _r16(qkv, round_fp16)
     q, k, v = qkv.chunk(3, dim=-1)
     q = transpose_for_scores(q, n_heads, hd)
     k = transpose_for_scores(k, n_heads, hd)
     v = transpose_for_scores(v, n_heads, hd)
     h = dense_masked_attention(q, k, v, mask, dtype)
-    h = h.permute(0, 2, 1, 3).contiguous().view(x.shape)
-    h = gemm_bias_residual_layernorm(h, p["W_o"], p["b_o"], x, p["g1"], p["be1"], eps, dtype)
+    h = _r16(h.permute(0, 2, 1, 3).contiguous().view(x.shape), round_fp16)
+    rp = round_fp16 == "split"
+    h = _r16(gemm_bias_residual_layernorm(h, p["W_o"], p["b_o"], x, p["g1"], p["be1"], eps, dtype, rp), round_fp16)
     r = h
-    h = gemm_bias_act(h, p["W_1"], p["b_1"], "gelu" if gelu == "erf" else "gelu_tanh", dtype)
-    return gemm_bias_residual_layernorm(h, p["W_2"], p["b_2"], r, p["g2"], p["be2"], eps, dtype)
+    act = {"erf": "gelu", "tanh": "gelu_tanh", "relu": "relu"}[gelu]
+    h = _r16(gemm_bias_act(h, p["W_1"], p["b_1"], act, dtype), round_fp16)
+    return _r16(gemm_bias_residual_layernorm(h, p["W_2"], p["b_2"], r, p["g2"], p["be2"], eps, dtype, rp), round_fp16)

@@ -706,8 +706,9 @@ int compute_units() {
   return cus;
 }
 
-int pick_form(int64_t two_row_groups, int nQ) {
-  if (g_attn_form != kFormAuto) return g_attn_form;
+int pick_form(int requested, int64_t two_row_groups, int nQ) {
+  if (requested != kFormAuto) return requested;          // the caller's choice for this call
+  if (g_attn_form != kFormAuto) return g_attn_form;      // the process-wide default
   return (nQ >= kKeySplitMinQueryBlocks && two_row_groups <= (int64_t)kKeySplitMaxGroupsPerCu * compute_units()) ? kFormKeySplit : kFormTwoRows;
 }
 
@@ -729,9 +730,9 @@ void set_balance(AttnParams& p, int max_groups) {
 }
 
 template <int KIND>
-void launch_attn(AttnParams& p, int nQ, int64_t bh, hipStream_t stream) {
+void launch_attn(AttnParams& p, int nQ, int64_t bh, int requested_form, hipStream_t stream) {
   const int64_t two_row_groups = (int64_t)((nQ + kRowsPerGroup - 1) / kRowsPerGroup) * bh;
-  const int form = pick_form(two_row_groups, nQ);
+  const int form = pick_form(requested_form, two_row_groups, nQ);
   if (form == kFormKeySplit) {
     p.nP = nQ;
     p.total = (int)(nQ * bh);
@@ -768,7 +769,8 @@ extern "C" int stof_block_attn_fwd(
     const int64_t q_strides[3], const int64_t k_strides[3],
     const int64_t v_strides[3], const int64_t out_strides[3],
     int batch_size, int seq_len, int head_num, int head_size,
-    int64_t lut_batch_stride, void* stream) {
+    int64_t lut_batch_stride, int launch_form, void* stream) {
+  if (launch_form != kFormAuto && launch_form != kFormTwoRows && launch_form != kFormKeySplit) return STOF_ERR_UNSUPPORTED;
   if (!q || !k || !v || !out || !full_row_ptr || !part_row_ptr || !load_row_ptr ||
       !q_strides || !k_strides || !v_strides || !out_strides)
     return STOF_ERR_NULL_POINTER;
@@ -794,14 +796,15 @@ extern "C" int stof_block_attn_fwd(
   p.B = batch_size; p.S = seq_len; p.H = head_num; p.nQ = nQ;
   p.c = softmax_scale * 1.4426950408889634f;
   p.row_bits = nullptr; p.words = 0; p.causal = 0; p.band = 0;
-  launch_attn<kKindLut>(p, nQ, (int64_t)batch_size * head_num, (hipStream_t)stream);
+  launch_attn<kKindLut>(p, nQ, (int64_t)batch_size * head_num, launch_form, (hipStream_t)stream);
   return stof_check_launch();
 }
 
 extern "C" int stof_rowwise_attn_fwd(
     const void* q, const void* k, const void* v, void* out,
     int kind, int is_causal, int bandwidth, const uint64_t* mask_bits,
-    int batch_size, int seq_len, int head_num, int head_size, void* stream) {
+    int batch_size, int seq_len, int head_num, int head_size, int launch_form, void* stream) {
+  if (launch_form != kFormAuto && launch_form != kFormTwoRows && launch_form != kFormKeySplit) return STOF_ERR_UNSUPPORTED;
   if (!q || !k || !v || !out) return STOF_ERR_NULL_POINTER;
   if (kind != STOF_ROW_FULL && kind != STOF_ROW_SLIDING && kind != STOF_ROW_MASK) return STOF_ERR_UNSUPPORTED;
   if (kind == STOF_ROW_MASK && !mask_bits) return STOF_ERR_NULL_POINTER;
@@ -823,8 +826,8 @@ extern "C" int stof_rowwise_attn_fwd(
   p.c = (1.0f / sqrtf((float)head_size)) * 1.4426950408889634f;
   p.row_bits = mask_bits; p.words = seq_len / 64; p.causal = is_causal ? 1 : 0;
   p.band = kind == STOF_ROW_SLIDING ? bandwidth : 0;
-  if (kind == STOF_ROW_MASK) launch_attn<kKindBits>(p, nQ, (int64_t)batch_size * head_num, (hipStream_t)stream);
-  else launch_attn<kKindPred>(p, nQ, (int64_t)batch_size * head_num, (hipStream_t)stream);
+  if (kind == STOF_ROW_MASK) launch_attn<kKindBits>(p, nQ, (int64_t)batch_size * head_num, launch_form, (hipStream_t)stream);
+  else launch_attn<kKindPred>(p, nQ, (int64_t)batch_size * head_num, launch_form, (hipStream_t)stream);
   return stof_check_launch();
 }
 

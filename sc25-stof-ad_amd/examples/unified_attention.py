@@ -19,7 +19,7 @@ from ops.package_op import block_attn_mask_op, rowwise_attn_full_op            #
 from util.masks import (generate_bigbird_mask, generate_causal_mask, generate_dilated_mask,  # noqa: E402
                         generate_longformer_mask, generate_sliding_mask, get_sparse_storage)
 from util.utils import time_stamp_cudasync, torch_cuda_identify                 # noqa: E402
-from stof.selector import GPUParams, select_operator                            # noqa: E402
+from stof.selector import GPUParams, apply, select_operator                     # noqa: E402
 
 
 def dense_attention(q, k, v, mask):
@@ -63,18 +63,19 @@ def main():
     nnz, *lut = get_sparse_storage(mask, 64, 64)          # nnz: the reference's figure, non-zeros of [B,S,S] over S*S in per cent
     active = int(lut[5][-1])                               # last LOAD row pointer = active 64 x 64 blocks
     choice = select_operator(GPUParams("MI355X"), lut[5], args.batch, args.seq, args.heads,
-                             is_causal=args.mask == "causal")
+                             is_causal=args.mask == "causal", lut=lut)
     print(f"mask {args.mask}: nnz figure {float(nnz):.1f}, {active} of {(args.seq // 64) ** 2} blocks active; "
           f"selector: {choice} ({choice.reason})")
 
     want = dense_attention(q, k, v, mask[:1])
-    if choice.operator == "row-wise" and args.mask == "causal":
-        run = lambda: rowwise_attn_full_op(q, k, v, True)                      # [B,S,H*D]
-        got = run().view(args.batch, args.seq, args.heads, 64).permute(0, 2, 1, 3)
-    else:
-        out = torch.empty_like(q)
-        run = lambda: block_attn_mask_op(out.copy_(q), k, v, *lut, 64, 64, 4)   # the op writes into its first argument
-        got = run()
+    # the selected operator in the selected launch form; [B,S,H*D] like the reference's row-wise operators
+    run = lambda: apply(choice, q, k, v, lut, is_causal=args.mask == "causal")
+    got = run().view(args.batch, args.seq, args.heads, 64).permute(0, 2, 1, 3)
+    # the reference-named operators give the same numbers (the block op writes into its first argument)
+    same = block_attn_mask_op(q.clone(), k, v, *lut, 64, 64, 4)
+    if args.mask == "causal":
+        same = rowwise_attn_full_op(q, k, v, True).view(args.batch, args.seq, args.heads, 64).permute(0, 2, 1, 3)
+    assert (same.float() - got.float()).abs().max().item() < 2e-3
     err = (got.float() - want).abs().max().item()
     print(f"max abs difference from dense fp32 attention: {err:.2e}")
 

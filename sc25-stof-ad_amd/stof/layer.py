@@ -28,7 +28,11 @@ class EncoderLayer:
         W_2 [F,D], b_2, g2, be2 in the reference's [in, out] orientation, fp16 on the GPU."""
         self.n_heads = n_heads
         self.eps = eps
-        self.act = "gelu" if gelu == "erf" else "gelu_tanh"
+        # FFN activation: erf GELU (BERT, src/benchmk_end2end.py:81), tanh GELU (GPT, :25-26,144), ReLU (T5, :206)
+        acts = {"erf": "gelu", "gelu": "gelu", "tanh": "gelu_tanh", "gelu_tanh": "gelu_tanh", "relu": "relu"}
+        if gelu not in acts:
+            raise ValueError(f"activation must be one of {sorted(acts)}, got {gelu!r}")
+        self.act = acts[gelu]
         self.ln_fusion = ln_fusion
         w = weights
         self.Wqkv = w["W_qkv"].t().contiguous(); self.bqkv = w["b_qkv"].contiguous()

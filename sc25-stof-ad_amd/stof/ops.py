@@ -19,7 +19,7 @@ from torch.autograd import Function
 from . import _lib
 from ._lib import StofError, check, strides3
 
-__all__ = ["block_attn", "block_attn_mask_op", "rowwise_attn_full_op", "rowwise_attn_sliding_op",
+__all__ = ["block_attn", "rowwise_attn", "block_attn_mask_op", "rowwise_attn_full_op", "rowwise_attn_sliding_op",
            "rowwise_attn_mask_op", "pack_mask_bits", "set_attention_launch_form", "StofError"]
 
 _BITS_ATTR = "_stof_packed_bits"
@@ -44,16 +44,24 @@ def _require(cond, msg):
         raise StofError(msg)
 
 
-_LAUNCH_FORMS = {"auto": -1, "two_rows": 0, "key_split": 1}
+_LAUNCH_FORMS = {None: -1, "default": -1, "auto": -1, "two_rows": 0, "key_split": 1}
+
+
+def _form(launch_form):
+    _require(launch_form in _LAUNCH_FORMS,
+             f"launch form must be one of 'default', 'two_rows', 'key_split', got {launch_form!r}")
+    return _LAUNCH_FORMS[launch_form]
 
 
 def set_attention_launch_form(form="auto"):
-    """Process-wide launch form of the attention kernels: ``"auto"`` (by grid size),
-    ``"two_rows"`` (two query blocks per workgroup, for large grids) or ``"key_split"`` (one
-    query block per workgroup with the keys of each tile split over two wavefront pairs, for
-    small grids).  The reference selects its kernel per call with ``num_warps``
-    (src/ops/src/block_attn_mask_cuda.cu:6064-6322); results agree within rounding here."""
-    _require(form in _LAUNCH_FORMS, f"launch form must be one of {sorted(_LAUNCH_FORMS)}, got {form!r}")
+    """Process-wide DEFAULT launch form of the attention kernels, used by calls that do not
+    name one: ``"auto"`` (by grid size), ``"two_rows"`` (two query blocks per workgroup, for
+    large grids) or ``"key_split"`` (one query block per workgroup with the keys of each tile
+    split over two wavefront pairs, for small grids).  The reference selects its kernel per
+    call with ``num_warps`` (src/ops/src/block_attn_mask_cuda.cu:6064-6322); the per-call
+    counterpart here is the ``launch_form`` argument of ``block_attn`` and of the row-wise
+    operators' functional form.  Results agree within rounding in every form."""
+    _require(form in ("auto", "two_rows", "key_split"), f"launch form must be 'auto', 'two_rows' or 'key_split', got {form!r}")
     check(_lib.lib().stof_attn_set_launch_form(_LAUNCH_FORMS[form]), "stof_attn_set_launch_form")
 
 
@@ -72,11 +80,29 @@ def pack_mask_bits(src, additive):
     return dst
 
 
+def _content_key(t):
+    """What the per-tensor caches are keyed on: the storage address and PyTorch's in-place
+    version counter.  A write that goes around PyTorch (another library through ``data_ptr``,
+    DLPack, numpy-shared memory) changes neither: such callers pass ``revalidate=True``."""
+    return (t.data_ptr(), t._version)
+
+
+def _drop_caches(lut):
+    for t in lut:
+        for attr in (_BITS_ATTR, _LUT_OK_ATTR, _LUT64_ATTR, _LUT_READY_ATTR):
+            if hasattr(t, attr):
+                try:
+                    delattr(t, attr)
+                except AttributeError:
+                    pass
+
+
 def _packed_partial_bits(part_block_mask):
     """Bit rows of the LUT's partial blocks, packed once per tensor object and content
     version and kept on the tensor itself."""
+    key = _content_key(part_block_mask)
     cached = getattr(part_block_mask, _BITS_ATTR, None)
-    if cached is not None and cached[0] == part_block_mask._version:
+    if cached is not None and cached[0] == key:
         return cached[1]
     pbm = part_block_mask
     _require(pbm.dim() == 3, "part_block_mask must be [n_part, BLOCK_M, BLOCK_N]")
@@ -86,7 +112,7 @@ def _packed_partial_bits(part_block_mask):
     _require(bool(ok), "part_block_mask must hold only 0 and -10000 (get_sparse_storage's encoding)")
     bits = pack_mask_bits(pbm, additive=True)
     try:
-        setattr(part_block_mask, _BITS_ATTR, (part_block_mask._version, bits))
+        setattr(part_block_mask, _BITS_ATTR, (key, bits))
     except AttributeError:
         pass
     return bits
@@ -99,7 +125,7 @@ def _check_lut_order(lrp, lci, prp, pci, n_cols):
     """The kernel walks each row's LOAD and PART lists as ascending sets (that is how
     get_sparse_storage emits them); verify once per column-list tensor and content version."""
     cached = getattr(lci, _LUT_OK_ATTR, None)
-    key = (lci._version, pci._version, lrp._version, prp._version)
+    key = tuple(_content_key(t) for t in (lci, pci, lrp, prp))
     if cached == key:
         return
     for name, rp, ci in (("load", lrp, lci), ("part", prp, pci)):
@@ -135,7 +161,7 @@ def _lut_at_64(lut, S, block_m, block_n):
     LUT (kept on the LOAD column tensor, keyed by the tensors' content versions)."""
     from . import masks as pm
     frp, fci, prp, pci, pbm, lrp, lci = lut
-    key = (lci._version, pci._version, lrp._version, prp._version, fci._version, frp._version, pbm._version, block_m, block_n)
+    key = tuple(_content_key(t) for t in lut) + (block_m, block_n)
     cached = getattr(lci, _LUT64_ATTR, None)
     if cached is not None and cached[0] == key:
         return cached[1]
@@ -161,7 +187,7 @@ def _prepared_lut(lut, B, S, block_m, block_n, dev):
     kept on the LOAD column tensor, keyed by the identity and content version of all seven
     tensors, the problem size and the device, and it holds the tensors it points into."""
     lci = lut[6]
-    key = (B, S, block_m, block_n, dev) + tuple((id(t), t._version) for t in lut)
+    key = (B, S, block_m, block_n, dev) + tuple((id(t),) + _content_key(t) for t in lut)
     cached = getattr(lci, _LUT_READY_ATTR, None)
     if cached is not None and cached[0] == key:
         return cached[1], cached[2]
@@ -200,13 +226,20 @@ def _check_i32(name, t, device):
     return t.contiguous()
 
 
-def block_attn(q, k, v, lut, block_m=64, block_n=64, out=None, out_layout="bhsd", softmax_scale=None):
+def block_attn(q, k, v, lut, block_m=64, block_n=64, out=None, out_layout="bhsd", softmax_scale=None,
+               launch_form=None, revalidate=False):
     """Block-masked attention.  q, k, v: fp16 views ``[B,H,S,D]`` with unit stride in D (any
     other strides).  ``lut`` = (full_row_ptr, full_col_idx, part_row_ptr, part_col_idx,
     part_block_mask, load_row_ptr, load_col_idx) as returned by ``get_sparse_storage`` (the
     leading ``nnz`` dropped) or by ``get_sparse_storage_batched`` (2-D row pointers: one LUT
     per sample).  Returns ``out``: ``[B,H,S,D]`` (``out_layout='bhsd'``) or ``[B,S,H*D]``
     (``'bshd'``); ``out`` may be ``q`` itself.
+
+    ``launch_form``: ``None`` / ``"default"`` (the process default, automatic by grid size
+    unless ``set_attention_launch_form`` changed it), ``"two_rows"`` or ``"key_split"`` - the
+    per-call counterpart of the reference's ``num_warps``.  ``revalidate=True`` discards what
+    is cached for this LUT (validation, packed bit rows, re-tiling) and prepares it again: for
+    LUT buffers rewritten behind PyTorch's back, which the caches cannot see.
     """
     _require(q.is_cuda, "q must be a CUDA tensor (this path has no CPU implementation)")
     dev = q.device
@@ -216,6 +249,9 @@ def block_attn(q, k, v, lut, block_m=64, block_n=64, out=None, out_layout="bhsd"
         _require(t is q or t.device == dev, f"{name} is on a different device than q")
     _require(k.shape == q.shape and v.shape == q.shape, "q, k, v must have the same shape")
     B, H, S, D = q.shape
+    form = _form(launch_form)
+    if revalidate:
+        _drop_caches(lut)
     lut_ptrs, lut_bs = _prepared_lut(lut, B, S, block_m, block_n, dev)
     if out is None:
         if out_layout == "bhsd":
@@ -236,7 +272,7 @@ def block_attn(q, k, v, lut, block_m=64, block_n=64, out=None, out_layout="bhsd"
         q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(),
         *lut_ptrs, 64, 64, scale,
         strides3(q), strides3(k), strides3(v), ostr,
-        B, S, H, D, lut_bs, _stream(dev)), "stof_block_attn_fwd")
+        B, S, H, D, lut_bs, form, _stream(dev)), "stof_block_attn_fwd")
     return out
 
 
@@ -265,7 +301,7 @@ class Block_Attn_Mask(Function):
         return q
 
 
-def _rowwise(kind, q, k, v, is_causal, bandwidth, row_mask):
+def _rowwise(kind, q, k, v, is_causal, bandwidth, row_mask, launch_form=None):
     _require(q.is_cuda, "q must be a CUDA tensor (this path has no CPU implementation)")
     for name, t in (("q", q), ("k", k), ("v", v)):
         _require(t.dtype == torch.float16, f"{name} must be float16, got {t.dtype}")
@@ -276,19 +312,27 @@ def _rowwise(kind, q, k, v, is_causal, bandwidth, row_mask):
     if kind == 2:
         _require(row_mask.shape[-2:] == (S, S), f"row_mask must be [{S},{S}]")
         cached = getattr(row_mask, _BITS_ATTR, None)
-        if cached is not None and cached[0] == row_mask._version:
+        if cached is not None and cached[0] == _content_key(row_mask):
             bits = cached[1]
         else:
             bits = pack_mask_bits(row_mask.to(torch.float16).reshape(S, S), additive=False)
             try:
-                setattr(row_mask, _BITS_ATTR, (row_mask._version, bits))
+                setattr(row_mask, _BITS_ATTR, (_content_key(row_mask), bits))
             except AttributeError:
                 pass
     check(_lib.lib().stof_rowwise_attn_fwd(
         q.data_ptr(), k.data_ptr(), v.data_ptr(), result.data_ptr(),
         kind, 1 if is_causal else 0, int(bandwidth), _ptr(bits),
-        B, S, H, D, _stream(q.device)), "stof_rowwise_attn_fwd")
+        B, S, H, D, _form(launch_form), _stream(q.device)), "stof_rowwise_attn_fwd")
     return result
+
+
+def rowwise_attn(kind, q, k, v, is_causal=False, bandwidth=0, row_mask=None, launch_form=None):
+    """Functional form of the three row-wise operators with the launch form as an argument:
+    ``kind`` "full" | "sliding" | "mask"; returns ``[B, S, H*D]``."""
+    kinds = {"full": 0, "sliding": 1, "mask": 2}
+    _require(kind in kinds, f"kind must be one of {sorted(kinds)}, got {kind!r}")
+    return _rowwise(kinds[kind], q, k, v, is_causal, bandwidth, row_mask, launch_form)
 
 
 class RowWise_Attn_Full(Function):

@@ -16,8 +16,8 @@ Mirrors the interface of the reference's two-phase selector
   the choice is between two query blocks per workgroup (K/V tiles shared, half the L2 -> LDS
   traffic) and the key split (one query block per workgroup, half-length chains), by how
   many workgroups a compute unit receives and how long the chains can be.  The same rule is
-  built into ``stof_block_attn_fwd``; this module states it, explains it and lets a caller
-  apply it explicitly through ``apply``.
+  built into ``stof_block_attn_fwd`` (its default); this module states it, explains it and
+  ``apply`` runs the chosen operator with the chosen form as a per-call argument.
 
 No measurement, search or autotuning takes place.
 """
@@ -72,15 +72,37 @@ def _active_blocks(load_row_ptr):
     return int(last)
 
 
-def phase1_decision(load_row_ptr, seq_len, is_causal=False, dense_tau=0.9):
+def phase1_decision(load_row_ptr, seq_len, is_causal=False, dense_tau=0.9, lut=None):
     """True -> block-wise (LUT) operator, False -> row-wise (predicate) operator.
 
     ``rho`` is the share of 64 x 64 tiles the LUT lists; the row-wise operators would visit
     every tile (the lower triangle when causal).  Block-wise unless the LUT lists at least
-    ``dense_tau`` of those."""
+    ``dense_tau`` of those.  With the whole ``lut`` given (the seven tensors of
+    ``get_sparse_storage``) the answer is exact instead of a density estimate: row-wise only if
+    the LUT IS the predicate's pattern - every tile of the square listed and none partial
+    (dense), or exactly the lower triangle listed, only the diagonal tiles partial and each of
+    them the 64 x 64 lower triangle (causal) - so that ``rowwise_attn_full_op`` computes the
+    same function; any other nearly-dense mask stays on the LUT, which keeps its partial tiles."""
     nq = seq_len // BLOCK
     visited = nq * (nq + 1) // 2 if is_causal else nq * nq
-    return _active_blocks(load_row_ptr) < dense_tau * visited
+    if lut is None:
+        return _active_blocks(load_row_ptr) < dense_tau * visited
+    import torch
+    frp, fci, prp, pci, pbm, lrp, lci = lut
+    if lrp.dim() == 2:
+        if lrp.shape[0] > 1:
+            return True                              # per-sample masks: no single predicate
+        lrp, prp = lrp[0], prp[0]
+    rows = (lrp[1:] - lrp[:-1]).tolist()
+    parts = (prp[1:] - prp[:-1]).tolist()
+    if not is_causal:
+        return not (rows == [nq] * nq and parts == [0] * nq)
+    if rows != list(range(1, nq + 1)) or parts != [1] * nq or tuple(pbm.shape) != (nq, BLOCK, BLOCK):
+        return True
+    if pci.tolist() != list(range(nq)):
+        return True
+    tri = torch.tril(torch.ones(BLOCK, BLOCK, device=pbm.device)) > 0
+    return not bool(((pbm == 0) == tri[None]).all())
 
 
 def phase2_selection(gpu, seq_len, batch_size, head_num):
@@ -101,23 +123,32 @@ def phase2_selection(gpu, seq_len, batch_size, head_num):
     return ("two_rows", per_cu, why)
 
 
-def select_operator(gpu_params, load_row_ptr, batch_size, seq_len, head_num, is_causal=False):
+def select_operator(gpu_params, load_row_ptr, batch_size, seq_len, head_num, is_causal=False, lut=None):
     """Reference: select_operator(gpu_params, load_row_ptr, batch_size, seq_len, head_num),
     benchmk_attn_unified.py:157-163, which returns ``"block-wise warp{w}m{m}n{n}"`` or
-    ``"row-wise"``; ``str()`` of the result here has the same two shapes."""
+    ``"row-wise"``; ``str()`` of the result here has the same two shapes.  Pass the whole
+    ``lut`` as well to have "row-wise" returned only when the dense / causal row-wise operator
+    computes exactly the LUT's mask (see ``phase1_decision``)."""
     if seq_len % BLOCK:
         raise ValueError(f"seq_len ({seq_len}) must be a multiple of {BLOCK}")
     nq = seq_len // BLOCK
     rho = _active_blocks(load_row_ptr) / float(nq * nq)
     form, per_cu, why = phase2_selection(gpu_params, seq_len, batch_size, head_num)
-    if phase1_decision(load_row_ptr, seq_len, is_causal):
+    if phase1_decision(load_row_ptr, seq_len, is_causal, lut=lut):
         return Selection("block-wise", form, BLOCK, BLOCK, rho, per_cu, why)
     return Selection("row-wise", form, BLOCK, BLOCK, rho, per_cu,
                      "the LUT lists nearly every tile the index predicate visits; " + why)
 
 
-def apply(selection):
-    """Force the selected launch form for the calls that follow (``"auto"`` applies the same
-    rule inside the library)."""
-    from .ops import set_attention_launch_form
-    set_attention_launch_form(selection.launch_form)
+def apply(selection, q, k, v, lut=None, is_causal=False, out_layout="bshd"):
+    """Run the selected operator in the selected launch form (passed per call, no process
+    state involved) and return its result: ``[B,S,H*D]`` (``out_layout="bshd"``, the layout
+    of the reference's row-wise operators) or ``[B,H,S,D]`` (``"bhsd"``, block-wise only).
+    ``lut``: the seven LUT tensors, needed for "block-wise"."""
+    from .ops import block_attn, rowwise_attn
+    if selection.operator == "row-wise":
+        return rowwise_attn("full", q, k, v, is_causal, launch_form=selection.launch_form)
+    if lut is None:
+        raise ValueError("the block-wise operator needs the LUT")
+    return block_attn(q, k, v, lut, selection.block_m, selection.block_n, out_layout=out_layout,
+                      launch_form=selection.launch_form)

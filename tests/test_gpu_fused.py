@@ -87,7 +87,9 @@ def test_reference_named_fused_ops():
     a = _rand(2, 128, 256, seed=16); b = _rand(256, 1024, seed=17, scale=0.05); d = _rand(1024, 256, seed=18, scale=0.05)
     bb = _rand(1024, seed=19, scale=0.5)
     got = fused.triton_matmul_batch(a.cuda(), b.cuda(), d.cuda(), bb.cuda())
-    _close(got, oe.matmul_gelu_matmul(a, b, d, bb), "matmul_batch", atol=4e-3)
+    want = oe.matmul_gelu_matmul(a, b, d, bb)        # the oracle stores the intermediate in fp16, as gemm_gemm.py:152 does
+    print(f"matmul_batch max abs err {float((got.float().cpu() - want).abs().max()):.2e}", flush=True)
+    _close(got, want, "matmul_batch")
 
 
 def test_fused_op_errors():
@@ -134,21 +136,62 @@ def test_rowwise_ops(B, H, S, launch_form):
 
 
 # ---- encoder layer -----------------------------------------------------------------------------
+#
+# Two comparisons per layer test.  (1) The oracle that stores its tensors in fp16 wherever the
+# five kernels (and the reference's fp16 eager layer, src/benchmk_end2end.py:31-88) store them:
+# held to 2e-3 + 1e-2 |want|.  (2) The fp32-throughout oracle: the observed maximum error is
+# printed and held to the bound written at the call, which is what the fp16 stores between
+# the kernels cost (one fp16 ulp at |y| in [2, 4) is 1.95e-3).
 
-@pytest.mark.parametrize("fusion", ["fused", "split"])
-def test_encoder_layer_c3_reduced_batch(fusion):
-    """BERT-base layer (hidden 768, 12 heads, FFN 3072, eps 1e-12) at batch 4, per-sample
-    padding x sliding-window mask, against the fp32 oracle of the same layer."""
-    B, S, D, H, F = 4, 512, 768, 12, 3072
+def _max_err(got, want):
+    return float((got.float().cpu() - want.float().cpu()).abs().max())
+
+
+def _layer_checks(got, want16, want32, what, fp32_bound, valid=None):
+    got = got.cpu()
+    if valid is not None:
+        got, want16, want32 = got[valid], want16[valid], want32[valid]
+    e16, e32 = _max_err(got, want16), _max_err(got, want32)
+    print(f"{what}: max abs err vs fp16-storing oracle {e16:.2e}, vs fp32 oracle {e32:.2e}", flush=True)
+    _close(got, want16, what + " vs fp16-storing oracle")
+    assert e32 <= fp32_bound, f"{what}: max abs err vs the fp32 oracle {e32:.3e} above {fp32_bound}"
+
+
+@pytest.mark.timeout(300)
+@pytest.mark.parametrize("fusion", ["fused", "split", "auto"])
+@pytest.mark.parametrize("B", [4, 16])
+def test_encoder_layer_c3(fusion, B):
+    """BERT-base layer (hidden 768, 12 heads, FFN 3072, eps 1e-12), per-sample padding x
+    sliding-window mask, at a reduced batch and at the full batch of 16 (8192 tokens)."""
+    S, D, H, F = 512, 768, 12, 3072
     w = configs.layer_weights(D, F, seed=0)
     x = configs.layer_input(configs.LayerConfig("t", B, S, D, H, F, 1), seed=1)
     mask, L = configs.mask_c3(batch=B, s=S, window=256, seed=0)
     lut = pm.get_sparse_storage_batched(mask.float().cuda(), 64, 64)[1:]
     layer = EncoderLayer({k: v.cuda() for k, v in w.items()}, H, eps=1e-12, ln_fusion=fusion)
     got = layer(x.cuda(), lut)
-    want = oe.bert_layer(x, w, mask.float(), H, eps=1e-12)
+    runs_fused = layer._fuse(B * S)
+    want16 = oe.bert_layer(x, w, mask.float(), H, eps=1e-12, round_fp16=True if runs_fused else "split")
+    want32 = oe.bert_layer(x, w, mask.float(), H, eps=1e-12)
     valid = torch.arange(S)[None, :] < L[:, None]          # rows past the sample length are don't-care
-    _close(got.cpu()[valid], want[valid], f"layer {fusion}", atol=4e-3)
+    _layer_checks(got, want16, want32, f"C3 layer B{B} {fusion}", 4e-3, valid)
+
+
+@pytest.mark.parametrize("act", ["tanh", "relu"])
+def test_encoder_layer_gpt_and_t5_activations(act):
+    """tanh GELU (GPT, src/benchmk_end2end.py:25-26,144) and ReLU (T5, :206) in the FFN."""
+    B, S, D, H, F = 2, 256, 768, 12, 3072
+    w = configs.layer_weights(D, F, seed=7)
+    x = configs.layer_input(configs.LayerConfig("t", B, S, D, H, F, 1), seed=8)
+    mask = configs.mask_c5(S)[None].expand(B, -1, -1)
+    lut = pm.get_sparse_storage(mask[:1].float().cuda(), 64, 64)[1:]
+    layer = EncoderLayer({k: v.cuda() for k, v in w.items()}, H, eps=1e-12, gelu=act)
+    got = layer(x.cuda(), lut)
+    mode = True if layer._fuse(B * S) else "split"
+    _layer_checks(got, oe.bert_layer(x, w, mask.float(), H, eps=1e-12, gelu=act, round_fp16=mode),
+                  oe.bert_layer(x, w, mask.float(), H, eps=1e-12, gelu=act), f"layer {act}", 4e-3)
+    with pytest.raises(ValueError):
+        EncoderLayer({k: v.cuda() for k, v in w.items()}, H, gelu="swish")
 
 
 def test_encoder_stack_two_layers_c5_shape_reduced():
@@ -159,10 +202,44 @@ def test_encoder_stack_two_layers_c5_shape_reduced():
     lut = pm.get_sparse_storage(mask.float().cuda(), 64, 64)[1:]
     stack = EncoderStack([{k: v.cuda() for k, v in w.items()} for w in ws], H, eps=1e-12)
     got = stack(x.cuda(), lut)
-    want = x
+    mode = True if stack.layers[0]._fuse(B * S) else "split"
+    want16 = want32 = x
     for w in ws:
-        want = oe.bert_layer(want, w, mask.float(), H, eps=1e-12)
-    _close(got, want, "stack", atol=6e-3)
+        want16 = oe.bert_layer(want16, w, mask.float(), H, eps=1e-12, round_fp16=mode)
+        want32 = oe.bert_layer(want32, w, mask.float(), H, eps=1e-12)
+    # two chained layers: the second amplifies the first's last-place differences
+    _layer_checks(got, want16, want32, "two-layer stack", 6e-3)
+
+
+@pytest.mark.timeout(600)
+def test_encoder_stack_c5_full_size():
+    """C5 at its size: 24 layers, hidden 1024, 16 heads, FFN 4096, B4 S2048, causal window 256 +
+    one global block, run end to end on the GPU.  Layers 1, 2, 12 and 24 are each checked
+    against the oracle's layer evaluated on the GPU's own input to that layer (an fp32 layer
+    takes about 5 s on the host, so not all 24; chaining 24 oracle layers instead would
+    compare accumulated last-place differences, not the layer)."""
+    cfg = configs.C5
+    mask = configs.mask_c5(cfg.seq)
+    lut = pm.get_sparse_storage(mask.float()[None].cuda(), 64, 64)[1:]
+    assert int(lut[5][-1]) == 177
+    x = configs.layer_input(cfg, seed=1).cuda()
+    checked = {0, 1, 11, 23}
+    worst16 = worst32 = 0.0
+    for i in range(cfg.layers):
+        w = configs.layer_weights(cfg.hidden, cfg.ffn, seed=i)
+        layer = EncoderLayer({k: v.cuda() for k, v in w.items()}, cfg.heads, eps=cfg.eps)
+        y = layer(x, lut)
+        if i in checked:
+            print(f"C5 layer {i + 1}", flush=True)
+            mode = True if layer._fuse(cfg.batch * cfg.seq) else "split"
+            xin = x.cpu()
+            want16 = oe.bert_layer(xin, w, mask.float()[None], cfg.heads, eps=cfg.eps, round_fp16=mode)
+            want32 = oe.bert_layer(xin, w, mask.float()[None], cfg.heads, eps=cfg.eps)
+            _layer_checks(y, want16, want32, f"C5 layer {i + 1} of 24", 4e-3)
+            worst16 = max(worst16, _max_err(y, want16)); worst32 = max(worst32, _max_err(y, want32))
+        x = y
+    assert bool(torch.isfinite(x.float()).all())
+    print(f"C5 stack: worst layer error {worst16:.2e} (fp16-storing oracle), {worst32:.2e} (fp32 oracle)", flush=True)
 
 
 def test_captured_stack_replays_match_eager_launches():
@@ -182,6 +259,9 @@ def test_captured_stack_replays_match_eager_launches():
         got = run(x).clone()
         torch.cuda.synchronize()
         assert torch.equal(got, want), f"replay {i} differs from the eager result"
-    want0 = oe.bert_layer(oe.bert_layer(xs[0].cpu(), ws[0], mask.float(), H, eps=1e-12), ws[1], mask.float(), H, eps=1e-12)
-    _close(run(xs[0]), want0, "captured stack vs oracle", atol=6e-3)
+    mode = True if stack.layers[0]._fuse(B * S) else "split"
+    want0 = xs[0].cpu()
+    for w in ws:
+        want0 = oe.bert_layer(want0, w, mask.float(), H, eps=1e-12, round_fp16=mode)
+    _close(run(xs[0]), want0, "captured stack vs fp16-storing oracle")
 

@@ -70,3 +70,34 @@ def test_bert_layer_against_module_style_evaluation():
     # pre-made QKV activation variant (the reference's layer has no QKV GEMM)
     w2 = dict(w); w2["W_qkv"] = None; w2["qkv_act"] = x @ w["W_qkv"]
     assert torch.allclose(oe.bert_layer(x, w2, mask, H, eps=1e-12), want, atol=2e-5)
+
+
+def test_bert_layer_fp16_rounding_points_and_activations():
+    """round_fp16 is pinned by an independent evaluation with explicit .half() stores at the
+    five operator boundaries (and, for "split", after the two products that feed a
+    LayerNorm); relu / tanh against F.relu / F.gelu(approximate="tanh")."""
+    B, S, D, H, Fd = 2, 64, 64, 4, 128
+    w = configs.layer_weights(D, Fd, seed=5, dtype=torch.float16)
+    wf = {k: v.float() for k, v in w.items()}
+    x = _r(B, S, D, seed=17).half()
+    mask = torch.tril(torch.ones(S, S))[None].expand(B, -1, -1)
+    h16 = lambda t: t.half().float()
+    for mode in (True, "split"):
+        for act, fn in (("erf", F.gelu), ("tanh", lambda t: F.gelu(t, approximate="tanh")), ("relu", F.relu)):
+            got = oe.bert_layer(x, w, mask, H, eps=1e-12, gelu=act, round_fp16=mode)
+            qkv = h16(F.linear(x.float(), wf["W_qkv"].t(), wf["b_qkv"]))
+            q, k, v = (t.view(B, S, H, D // H).transpose(1, 2) for t in qkv.chunk(3, -1))
+            a = h16(F.scaled_dot_product_attention(q, k, v, is_causal=True).transpose(1, 2).reshape(B, S, D))
+            p1 = F.linear(a, wf["W_o"].t())
+            p1 = h16(p1) if mode == "split" else p1
+            h = h16(F.layer_norm(p1 + wf["b_o"] + x.float(), (D,), wf["g1"], wf["be1"], 1e-12))
+            f = h16(fn(F.linear(h, wf["W_1"].t(), wf["b_1"])))
+            p2 = F.linear(f, wf["W_2"].t())
+            p2 = h16(p2) if mode == "split" else p2
+            want = h16(F.layer_norm(p2 + wf["b_2"] + h, (D,), wf["g2"], wf["be2"], 1e-12))
+            # equal up to the last place of fp16 where the two evaluations' fp32 sums differ in order
+            assert float((got - want).abs().max()) <= 2e-3, (mode, act)
+            assert torch.equal(got, h16(got))                    # the result is an fp16 value
+    # and the rounding moves the layer's result by less than the comparison tolerance
+    ref = oe.bert_layer(x, w, mask, H, eps=1e-12)
+    assert 0 < float((oe.bert_layer(x, w, mask, H, eps=1e-12, round_fp16=True) - ref).abs().max()) < 4e-3

@@ -43,6 +43,29 @@ def test_dense_and_causal_masks_go_row_wise():
     assert selector.select_operator(gpu, _lut(band)[6], 1, 2048, 4, is_causal=True).operator == "block-wise"
 
 
+def test_row_wise_only_for_exactly_dense_or_causal_luts():
+    """With the PART row pointers the answer is exact: a nearly dense mask that still has
+    partial tiles must stay on the LUT (the dense row-wise operator would ignore them)."""
+    gpu = selector.GPUParams()
+    s = 512
+    dense = torch.ones(s, s)
+    lut = _lut(dense)
+    assert selector.select_operator(gpu, lut[6], 2, s, 12, lut=lut[1:]).operator == "row-wise"
+    holes = dense.clone(); holes[5, 70] = 0; holes[300, 301] = 0          # 62 full + 2 partial of 64 tiles: rho = 1.0
+    lut = _lut(holes)
+    assert selector.select_operator(gpu, lut[6], 2, s, 12).operator == "row-wise"                       # density estimate alone
+    assert selector.select_operator(gpu, lut[6], 2, s, 12, lut=lut[1:]).operator == "block-wise"
+    causal = torch.tril(torch.ones(s, s))
+    lut = _lut(causal)
+    assert selector.select_operator(gpu, lut[6], 2, s, 12, is_causal=True, lut=lut[1:]).operator == "row-wise"
+    assert selector.select_operator(gpu, lut[6], 2, s, 12, is_causal=False, lut=lut[1:]).operator == "block-wise"
+    shifted = torch.tril(torch.ones(s, s), diagonal=-1)                   # same tiles listed, different diagonal content
+    shifted[0, 0] = 1
+    lut = _lut(shifted)
+    assert selector.select_operator(gpu, lut[6], 2, s, 12, is_causal=True, lut=lut[1:]).operator == "block-wise"
+    assert selector.select_operator(gpu, lut[6], 2, s, 12, is_causal=True).operator == "row-wise"      # the density estimate alone cannot tell
+
+
 def test_per_sample_row_pointers_and_errors():
     mask, _ = configs.mask_c3(4, 512, 256, seed=0)
     lut = pm.get_sparse_storage_batched(mask.float(), 64, 64)
