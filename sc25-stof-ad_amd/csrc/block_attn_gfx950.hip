@@ -109,11 +109,12 @@ template <int ROWS> struct RowPtrs {
 // merged through LDS at the end).  The second form halves the work of a wave per key block,
 // so the chain of key blocks of a long LUT row finishes in half the time; it is used for
 // small grids, where that chain and not throughput sets the run time.
-template <int KIND, int ROWS, int KS>
+template <int KIND, int ROWS, int KS, bool PIPE = false>
 __device__ __forceinline__ void attn_group(const AttnParams& p, const int bh, const int pair, const RowPtrs<ROWS>& pre,
                                            unsigned char* k_lds0, unsigned char* k_lds1,
                                            unsigned char* v_lds0, unsigned char* v_lds1) {
   static_assert(KS == 1 || ROWS == 1, "the key split serves a single query block");
+  static_assert(!PIPE || KS == 1, "the software-pipelined loop keeps all 64 keys of a tile in one wave");
   constexpr int kDma = 4 / (ROWS * KS);   // direct-to-LDS instructions per wave and operand tile (8 per tile)
   constexpr int kMT = 2 / KS;             // 32-key sub-tiles of a key block handled by one wave
 
@@ -308,158 +309,396 @@ __device__ __forceinline__ void attn_group(const AttnParams& p, const int bh, co
     return s;
   };
 
-  // one key block: kt/vt hold the current tile, the next tile's loads go to kn/vn
-  auto step = [&](const Step cur, const Step nxt, const lds_byte* kt, const lds_byte* vt, lds_byte* kn, lds_byte* vn) {
-    // The row mask of a partial tile is fetched first so that its latency hides behind
-    // the wait below and no register-returning load is pending across the DMA issue.
-    // Longest remaining chain first.  Among waves of equal priority a SIMD issues from the
-    // oldest, which starves the youngest workgroup of a compute unit until the others are done
-    // and leaves it to finish a long chain alone (measured: the last of four equal chains had
-    // done 6 of 21 steps when the third finished).  Priority by remaining length makes the
-    // chains of a SIMD end together.
-    {
-      const int left = steps_left--;
-      if (left >= 3 * kPrioStep) __builtin_amdgcn_s_setprio(3);
-      else if (left >= 2 * kPrioStep) __builtin_amdgcn_s_setprio(2);
-      else if (left >= kPrioStep) __builtin_amdgcn_s_setprio(1);
-      else __builtin_amdgcn_s_setprio(0);
-    }
-    uint64_t bits = ~0ull;
-    if (KIND == kKindLut) {
-      if (cur.slot >= 0) bits = p.pbits[(int64_t)cur.slot * kBM + 32 * half + j32];
-    } else if (KIND == kKindBits) {
-      if (cur.mine) bits = p.row_bits[(qrow0 + j32) * p.words + cur.col];
-    }
-    // All DMA issued so far (the current tile) has landed for this wave; the barrier makes
-    // every wave's share visible and also orders last step's reads of the other buffers
-    // before the loads that overwrite them.
-    __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0)
-    __syncthreads();
-    if (nxt.valid) issue_tile(nxt.col, kn, vn);
-    if (!cur.mine) return;
-    // Row-wise front-ends: which elements of this tile may be used.  need_mask is wave-uniform.
-    bool need_mask = (KIND == kKindLut) ? (cur.slot >= 0) : false;
-    if (KIND != kKindLut) {
-      const int qmin = (int)qrow0, qmax = qmin + 31, kmin = cur.col * kBN, kmax = kmin + kBN - 1;
+  if constexpr (PIPE) {
+    // ---- software-pipelined main loop.
+    // Iteration i holds three tiles of the wave's chain at once: the scores of tile i+1 are
+    // produced (S = K Q^T, 8 MFMA), the probabilities of tile i are formed from the scores made
+    // one iteration ago (exp2, convert, row sum: vector ALU only) and the probabilities of tile
+    // i-1 go into O (O += V^T P^T, 8 MFMA).  The three are independent of one another, so inside
+    // ONE wave every MFMA is followed by vector-ALU work that does not wait for it: the matrix
+    // pipeline and the vector ALU run side by side.  (Across waves they overlap badly: an MFMA
+    // that waits for the pipeline holds the SIMD's issue slot.)
+    //
+    // Running max: the fast path takes the max as it stands and only verifies, from the row sums
+    // it needs anyway, that no probability left the fp16 range; if one did (or a lane has not
+    // seen a key yet, or a tile needs an element mask, or a neighbour tile is not this wave's),
+    // the iteration runs the general path below: exact online softmax with max search and
+    // rescale, one piece after the other.  O holds tile i-1 by then, so the rescale is the usual one.
+    //
+    // LDS: K is fetched two tiles ahead of V (iteration i issues K(i+2) and V(i), reads K(i+1) and
+    // V(i-1)); with two buffers each, an iteration reads one buffer pair and fills the other.
+    struct Tile { Step st; bool mask; };
+    auto dma_k = [&](int col, lds_byte* kdst) {
+      const char* kt = reinterpret_cast<const char*>(kb + (int64_t)col * kBN * p.ks[2]);
+      lds_byte* kd = kdst + (kDma * wave) * 1024;
+#pragma unroll
+      for (int i = 0; i < kDma; ++i)
+        __builtin_amdgcn_global_load_lds((gptr_t*)(kt + k_src[i]), (__attribute__((address_space(3))) void*)(kd + i * 1024), 16, 0, 0);
+    };
+    auto dma_v = [&](int col, lds_byte* vdst) {
+      const char* vt = reinterpret_cast<const char*>(vb + (int64_t)col * kBN * p.vs[2]);
+      lds_byte* vd = vdst + (kDma * wave) * 1024;
+#pragma unroll
+      for (int i = 0; i < kDma; ++i)
+        __builtin_amdgcn_global_load_lds((gptr_t*)(vt + v_src[i]), (__attribute__((address_space(3))) void*)(vd + i * 1024), 16, 0, 0);
+    };
+    // element-mask word of this lane's query for a tile (requested when the tile enters the queue)
+    auto request_bits = [&](const Step& st) -> uint64_t {
+      uint64_t bits = ~0ull;
+      if (KIND == kKindLut) {
+        if (st.valid && st.slot >= 0) bits = p.pbits[(int64_t)st.slot * kBM + 32 * half + j32];
+      } else if (KIND == kKindBits) {
+        if (st.valid && st.mine) bits = p.row_bits[(qrow0 + j32) * p.words + st.col];
+      }
+      return bits;
+    };
+    // whether the tile needs its element mask (wave-uniform); the index predicates of the
+    // row-wise front-ends are folded into the bit row; a tile that allows nothing is dropped
+    auto settle_mask = [&](Tile& t, uint64_t& bits) {
+      t.mask = false;
+      if (!t.st.valid || !t.st.mine) return;
+      if (KIND == kKindLut) { t.mask = t.st.slot >= 0; return; }
+      const int qmin = (int)qrow0, qmax = qmin + 31, kmin = t.st.col * kBN, kmax = kmin + kBN - 1;
       const bool range_full = (!p.causal || kmax <= qmin) && (!(KIND == kKindPred && p.band > 0) || kmin > qmax - p.band);
       if (KIND == kKindBits) {
-        if (!__any(bits != 0ull)) return;            // nothing allowed for these 32 queries
-        need_mask = !range_full || __any(bits != ~0ull);
+        if (!__any(bits != 0ull)) { t.st.mine = 0; return; }
+        t.mask = !range_full || __any(bits != ~0ull);
       } else {
-        need_mask = !range_full;
+        t.mask = !range_full;
       }
-      if (need_mask) {
-        // fold the index predicates into the bit row: bit t = key kmin + t allowed
+      if (t.mask) {
         const int qg = qmin + j32;
         if (p.causal) { const int nk = qg - kmin + 1; bits &= nk >= 64 ? ~0ull : (nk <= 0 ? 0ull : ((1ull << nk) - 1)); }
         if (KIND == kKindPred && p.band > 0) {
-          const int first = qg - p.band + 1 - kmin;   // keys below this offset are outside the window
+          const int first = qg - p.band + 1 - kmin;
           bits &= first <= 0 ? ~0ull : (first >= 64 ? 0ull : ~((1ull << first) - 1));
         }
       }
-    }
-
-    // ---- S^T = K . Q^T : sacc[mt][r] = S[query j32][key 32mt + 8(r/4) + 4g + r%4]
-    // A partial tile applies its element mask through the accumulator's INITIAL value: 0 where
-    // the key is allowed, -inf where it is not (-inf + finite = -inf), two instructions per
-    // element (sign-extended one-bit field of the inverted mask word, AND with the bit pattern
-    // of -inf) instead of test + compare + select after the product.  The two cases run their
-    // own copy of the product so that the unmasked one keeps the constant-zero accumulator input.
-    floatx16 sacc[kMT];
-    auto s_product = [&]() {
+    };
+    // S^T = K . Q^T into s (see the accumulator layout at the non-pipelined step)
+    auto qk_product = [&](const lds_byte* kt, floatx16 (&s)[2]) {
 #pragma unroll
       for (int ks = 0; ks < 4; ++ks)
 #pragma unroll
-        for (int mt = 0; mt < kMT; ++mt) {
-          const half8_t a = *reinterpret_cast<const __attribute__((address_space(3))) half8_t*>(kt + (mt0 + mt) * 4096 + k_rd[ks]);
-          sacc[mt] = mfma32(a, qf[ks], sacc[mt]);
+        for (int mt = 0; mt < 2; ++mt) {
+          const half8_t a = *reinterpret_cast<const __attribute__((address_space(3))) half8_t*>(kt + mt * 4096 + k_rd[ks]);
+          s[mt] = mfma32(a, qf[ks], s[mt]);
         }
     };
-    if (need_mask) {
+    auto init_scores = [&](floatx16 (&s)[2], bool masked, uint64_t bits) {
+      if (masked) {
 #pragma unroll
-      for (int mt = 0; mt < kMT; ++mt) {
-        const uint32_t nw = ~((uint32_t)(bits >> (32 * (mt0 + mt))) >> (4 * g));   // bit set = key masked
+        for (int mt = 0; mt < 2; ++mt) {
+          const uint32_t nw = ~((uint32_t)(bits >> (32 * mt)) >> (4 * g));   // bit set = key masked
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          // (asm: written with the builtin, the compiler turns the pair back into and + compare + select)
-          int all;   // -1 if masked, else 0
-          asm("v_bfe_i32 %0, %1, %2, 1" : "=v"(all) : "v"(nw), "n"(8 * (r >> 2) + (r & 3)));
-          sacc[mt][r] = __builtin_bit_cast(float, (uint32_t)all & 0xFF800000u);
+          for (int r = 0; r < 16; ++r) {
+            int all;   // -1 if masked, else 0
+            asm("v_bfe_i32 %0, %1, %2, 1" : "=v"(all) : "v"(nw), "n"(8 * (r >> 2) + (r & 3)));
+            s[mt][r] = __builtin_bit_cast(float, (uint32_t)all & 0xFF800000u);
+          }
         }
+      } else {
+#pragma unroll
+        for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) s[mt][r] = 0.f;
       }
-      s_product();
-    } else {
+    };
+    // O^T += V^T . P^T
+    auto pv_product = [&](const lds_byte* vt, const half8_t (&pf)[2][2]) {
 #pragma unroll
-      for (int i = 0; i < kMT; ++i)
+      for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) sacc[i][r] = 0.f;
-      s_product();
-    }
-
-    // ---- online softmax; one query per lane (shared with the partner lane ^ 32).
-    // The running max is only raised when the tile's max exceeds it by more than kLazy
-    // (in log2 units): probabilities then stay below 2^kLazy, well inside fp16 range, the
-    // normalisation by the running sum stays exact, and the O rescale becomes rare.
-    float mx = sacc[0][0];
+        for (int s2 = 0; s2 < 2; ++s2)
 #pragma unroll
-    for (int mt = 0; mt < kMT; ++mt)
+          for (int dt = 0; dt < 2; ++dt) {
+            const lds_byte* vp = vt + (32 * mt + 16 * s2) * 128;
+            const short4_t a0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4*)(vp + v_rd[dt][0]));
+            const short4_t a1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4*)(vp + v_rd[dt][1]));
+            const half8_t a = __builtin_bit_cast(half8_t, (short8_t)__builtin_shufflevector(a0, a1, 0, 1, 2, 3, 4, 5, 6, 7));
+            oacc[dt] = mfma32(a, pf[mt][s2], oacc[dt]);
+          }
+    };
+    bool warm = false;   // every lane of the wave has a finite running max
+    float mc = 0.f;      // running max * c, the constant the fast softmax subtracts
+    // exact online softmax of one tile (max search, lazy raise, rescale of O and of the sum)
+    auto softmax_exact = [&](const floatx16 (&s)[2], half8_t (&pf)[2][2]) {
+      float mx = s[0][0];
 #pragma unroll
-      for (int r = 0; r < 16; ++r) mx = fmaxf(mx, sacc[mt][r]);
-    mx = pair_max(mx);
-    const float m_new = (mx * p.c > m_run * p.c + kLazy || m_run == -INFINITY) ? mx : m_run;
-    // A row that has seen no allowed key yet has m_new == -inf: subtract 0 instead, so
-    // that its probabilities are exp2(-inf) = 0 and no inf - inf appears.
-    const float m_sub = (m_new == -INFINITY) ? 0.f : m_new;
-    const float alpha = __builtin_amdgcn_exp2f((m_run - m_sub) * p.c);
-    const float mc = m_sub * p.c;
-    half8_t pf[kMT][2];   // [key sub-tile][half]: B operand of O^T = V^T . P^T
-    float lsum = 0.f;
+      for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
-    for (int mt = 0; mt < kMT; ++mt)
+        for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s[mt][r]);
+      mx = pair_max(mx);
+      const float m_new = (mx * p.c > m_run * p.c + kLazy || m_run == -INFINITY) ? mx : m_run;
+      const float m_sub = (m_new == -INFINITY) ? 0.f : m_new;
+      const float alpha = __builtin_amdgcn_exp2f((m_run - m_sub) * p.c);
+      mc = m_sub * p.c;
+      float lsum = 0.f;
 #pragma unroll
-      for (int r = 0; r < 16; r += 2) {
-        const float e0 = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[mt][r], p.c, -mc));
-        const float e1 = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[mt][r + 1], p.c, -mc));
-        const half2_t e2 = {(half_t)e0, (half_t)e1};
-        pf[mt][r >> 3][r & 7] = e2[0];
-        pf[mt][r >> 3][(r & 7) + 1] = e2[1];
-        // Row sum with plain adds: v_dot2c_f32_f16 would halve the instruction count but runs
-        // on the matrix pipeline and stalls behind every MFMA in flight on the SIMD.
-        lsum += e0 + e1;
+      for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+        for (int r = 0; r < 16; r += 2) {
+          const float e0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[mt][r], p.c, -mc));
+          const float e1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[mt][r + 1], p.c, -mc));
+          const half2_t e2 = {(half_t)e0, (half_t)e1};
+          pf[mt][r >> 3][r & 7] = e2[0];
+          pf[mt][r >> 3][(r & 7) + 1] = e2[1];
+          lsum += e0 + e1;
+        }
+      l_run = l_run * alpha + lsum;
+      m_run = m_new;
+      if (__any(alpha != 1.0f)) {
+#pragma unroll
+        for (int dt = 0; dt < 2; ++dt)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) oacc[dt][r] *= alpha;
       }
-    l_run = l_run * alpha + lsum;   // per-lane partial sum; the two halves are added at the end
-    m_run = m_new;
-    if (__any(alpha != 1.0f)) {
+      warm = !__any(m_run == -INFINITY);
+    };
+    // Fast softmax: the max is taken as it stands.  The row sum is formed from the fp16
+    // probabilities themselves (the values the second product uses) by a tree of packed adds,
+    // folded to fp32 once; a probability beyond the fp16 range shows up in it as inf or as a
+    // large sum, which the caller tests before it commits the tile.
+    auto softmax_fast = [&](const floatx16 (&s)[2], half8_t (&pf)[2][2]) -> float {
+      half2_t acc[16];
 #pragma unroll
-      for (int dt = 0; dt < 2; ++dt)
+      for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) oacc[dt][r] *= alpha;
-    }
+        for (int r = 0; r < 16; r += 2) {
+          const float e0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[mt][r], p.c, -mc));
+          const float e1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[mt][r + 1], p.c, -mc));
+          const half2_t e2 = {(half_t)e0, (half_t)e1};
+          pf[mt][r >> 3][r & 7] = e2[0];
+          pf[mt][r >> 3][(r & 7) + 1] = e2[1];
+          acc[8 * mt + (r >> 1)] = e2;
+        }
+#pragma unroll
+      for (int w = 8; w > 0; w >>= 1)
+#pragma unroll
+        for (int i = 0; i < w; ++i) acc[i] = acc[i] + acc[i + w];
+      return (float)acc[0][0] + (float)acc[0][1];
+    };
+    constexpr float kSumLimit = 16384.f;   // 32 probabilities of at most 2^kLazy sum to 2^13
 
-    // ---- O^T += V^T . P^T
+    Tile t0, t1, t2, t3;   // tiles i-1 (PV), i (softmax), i+1 (QK^T), i+2 (loads)
+    t0.st.valid = t1.st.valid = t2.st.valid = false;
+    t0.st.mine = t1.st.mine = t2.st.mine = 0;
+    t0.st.col = t1.st.col = t2.st.col = 0; t0.st.slot = t1.st.slot = t2.st.slot = -1;
+    t0.mask = t1.mask = t2.mask = t3.mask = false;
+    t3.st = next_step();
+    uint64_t bits2 = ~0ull;          // mask word of tile t2
+    floatx16 sA[2], sB[2];
+    half8_t pA[2][2], pB[2][2];
 #pragma unroll
-    for (int mt = 0; mt < kMT; ++mt)
+    for (int mt = 0; mt < 2; ++mt) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) { sA[mt][r] = 0.f; sB[mt][r] = 0.f; }
 #pragma unroll
       for (int s2 = 0; s2 < 2; ++s2)
 #pragma unroll
-        for (int dt = 0; dt < 2; ++dt) {
-          const lds_byte* vp = vt + (32 * (mt0 + mt) + 16 * s2) * 128;
-          const short4_t a0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4*)(vp + v_rd[dt][0]));
-          const short4_t a1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4*)(vp + v_rd[dt][1]));
-          const half8_t a = __builtin_bit_cast(half8_t, (short8_t)__builtin_shufflevector(a0, a1, 0, 1, 2, 3, 4, 5, 6, 7));
-          oacc[dt] = mfma32(a, pf[mt][s2], oacc[dt]);
-        }
-  };
+        for (int e = 0; e < 8; ++e) { pA[mt][s2][e] = (half_t)0.f; pB[mt][s2][e] = (half_t)0.f; }
+    }
 
-  Step cur = next_step();
-  if (cur.valid) issue_tile(cur.col, (lds_byte*)k_lds0, (lds_byte*)v_lds0);
-  while (cur.valid) {   // single exit: an early exit between the two steps makes the compiler copy the accumulators
-    Step nxt = next_step();
-    step(cur, nxt, (const lds_byte*)k_lds0, (const lds_byte*)v_lds0, (lds_byte*)k_lds1, (lds_byte*)v_lds1);
-    cur = nxt;
-    if (nxt.valid) {
-      cur = next_step();
-      step(nxt, cur, (const lds_byte*)k_lds1, (const lds_byte*)v_lds1, (lds_byte*)k_lds0, (lds_byte*)v_lds0);
+    // One iteration: reads the buffer pair (kr, vr), fills (kw, vw); scores s_in -> probabilities
+    // p_out, scores of the next tile -> s_out, probabilities p_in -> O.
+    auto iteration = [&](const lds_byte* kr, const lds_byte* vr, lds_byte* kw, lds_byte* vw,
+                         floatx16 (&s_in)[2], floatx16 (&s_out)[2], half8_t (&p_in)[2][2], half8_t (&p_out)[2][2]) {
+      {
+        const int left = steps_left--;
+        if (left >= 3 * kPrioStep) __builtin_amdgcn_s_setprio(3);
+        else if (left >= 2 * kPrioStep) __builtin_amdgcn_s_setprio(2);
+        else if (left >= kPrioStep) __builtin_amdgcn_s_setprio(1);
+        else __builtin_amdgcn_s_setprio(0);
+      }
+      __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): K(i+1), V(i-1) and the mask word of tile i+1 have landed
+      __syncthreads();
+      if (t3.st.valid) dma_k(t3.st.col, kw);
+      if (t1.st.valid) dma_v(t1.st.col, vw);
+      const uint64_t bits3 = request_bits(t3.st);
+      settle_mask(t2, bits2);
+      const bool do_pv = t0.st.valid && t0.st.mine, do_sm = t1.st.valid && t1.st.mine, do_qk = t2.st.valid && t2.st.mine;
+      if (do_pv && do_sm && do_qk && !t2.mask && warm) {
+        init_scores(s_out, false, 0);
+        qk_product(kr, s_out);
+        const float lsum = softmax_fast(s_in, p_out);
+        pv_product(vr, p_in);
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // one MFMA
+          __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);   // LDS fragment reads of the MFMAs to come
+          __builtin_amdgcn_sched_group_barrier(0x400, 2, 0);   // two exp2
+          __builtin_amdgcn_sched_group_barrier(0x002, 5, 0);   // scale, convert, sum
+        }
+        if (__any(!(lsum < kSumLimit))) softmax_exact(s_in, p_out);
+        else l_run += lsum;
+      } else {
+        if (do_qk) { init_scores(s_out, t2.mask, bits2); qk_product(kr, s_out); }
+        if (do_pv) pv_product(vr, p_in);
+        if (do_sm) softmax_exact(s_in, p_out);
+      }
+      t0 = t1; t1 = t2; t2 = t3;
+      bits2 = bits3;
+      t3.st = next_step(); t3.mask = false;
+    };
+
+    while (t0.st.valid || t1.st.valid || t2.st.valid || t3.st.valid) {   // single exit
+      iteration((const lds_byte*)k_lds1, (const lds_byte*)v_lds1, (lds_byte*)k_lds0, (lds_byte*)v_lds0, sA, sB, pA, pB);
+      iteration((const lds_byte*)k_lds0, (const lds_byte*)v_lds0, (lds_byte*)k_lds1, (lds_byte*)v_lds1, sB, sA, pB, pA);
+    }
+  } else {
+    // one key block: kt/vt hold the current tile, the next tile's loads go to kn/vn
+    auto step = [&](const Step cur, const Step nxt, const lds_byte* kt, const lds_byte* vt, lds_byte* kn, lds_byte* vn) {
+      // The row mask of a partial tile is fetched first so that its latency hides behind
+      // the wait below and no register-returning load is pending across the DMA issue.
+      // Longest remaining chain first.  Among waves of equal priority a SIMD issues from the
+      // oldest, which starves the youngest workgroup of a compute unit until the others are done
+      // and leaves it to finish a long chain alone (measured: the last of four equal chains had
+      // done 6 of 21 steps when the third finished).  Priority by remaining length makes the
+      // chains of a SIMD end together.
+      {
+        const int left = steps_left--;
+        if (left >= 3 * kPrioStep) __builtin_amdgcn_s_setprio(3);
+        else if (left >= 2 * kPrioStep) __builtin_amdgcn_s_setprio(2);
+        else if (left >= kPrioStep) __builtin_amdgcn_s_setprio(1);
+        else __builtin_amdgcn_s_setprio(0);
+      }
+      uint64_t bits = ~0ull;
+      if (KIND == kKindLut) {
+        if (cur.slot >= 0) bits = p.pbits[(int64_t)cur.slot * kBM + 32 * half + j32];
+      } else if (KIND == kKindBits) {
+        if (cur.mine) bits = p.row_bits[(qrow0 + j32) * p.words + cur.col];
+      }
+      // All DMA issued so far (the current tile) has landed for this wave; the barrier makes
+      // every wave's share visible and also orders last step's reads of the other buffers
+      // before the loads that overwrite them.
+      __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0)
+      __syncthreads();
+      if (nxt.valid) issue_tile(nxt.col, kn, vn);
+      if (!cur.mine) return;
+      // Row-wise front-ends: which elements of this tile may be used.  need_mask is wave-uniform.
+      bool need_mask = (KIND == kKindLut) ? (cur.slot >= 0) : false;
+      if (KIND != kKindLut) {
+        const int qmin = (int)qrow0, qmax = qmin + 31, kmin = cur.col * kBN, kmax = kmin + kBN - 1;
+        const bool range_full = (!p.causal || kmax <= qmin) && (!(KIND == kKindPred && p.band > 0) || kmin > qmax - p.band);
+        if (KIND == kKindBits) {
+          if (!__any(bits != 0ull)) return;            // nothing allowed for these 32 queries
+          need_mask = !range_full || __any(bits != ~0ull);
+        } else {
+          need_mask = !range_full;
+        }
+        if (need_mask) {
+          // fold the index predicates into the bit row: bit t = key kmin + t allowed
+          const int qg = qmin + j32;
+          if (p.causal) { const int nk = qg - kmin + 1; bits &= nk >= 64 ? ~0ull : (nk <= 0 ? 0ull : ((1ull << nk) - 1)); }
+          if (KIND == kKindPred && p.band > 0) {
+            const int first = qg - p.band + 1 - kmin;   // keys below this offset are outside the window
+            bits &= first <= 0 ? ~0ull : (first >= 64 ? 0ull : ~((1ull << first) - 1));
+          }
+        }
+      }
+
+      // ---- S^T = K . Q^T : sacc[mt][r] = S[query j32][key 32mt + 8(r/4) + 4g + r%4]
+      // A partial tile applies its element mask through the accumulator's INITIAL value: 0 where
+      // the key is allowed, -inf where it is not (-inf + finite = -inf), two instructions per
+      // element (sign-extended one-bit field of the inverted mask word, AND with the bit pattern
+      // of -inf) instead of test + compare + select after the product.  The two cases run their
+      // own copy of the product so that the unmasked one keeps the constant-zero accumulator input.
+      floatx16 sacc[kMT];
+      auto s_product = [&]() {
+  #pragma unroll
+        for (int ks = 0; ks < 4; ++ks)
+  #pragma unroll
+          for (int mt = 0; mt < kMT; ++mt) {
+            const half8_t a = *reinterpret_cast<const __attribute__((address_space(3))) half8_t*>(kt + (mt0 + mt) * 4096 + k_rd[ks]);
+            sacc[mt] = mfma32(a, qf[ks], sacc[mt]);
+          }
+      };
+      if (need_mask) {
+  #pragma unroll
+        for (int mt = 0; mt < kMT; ++mt) {
+          const uint32_t nw = ~((uint32_t)(bits >> (32 * (mt0 + mt))) >> (4 * g));   // bit set = key masked
+  #pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            // (asm: written with the builtin, the compiler turns the pair back into and + compare + select)
+            int all;   // -1 if masked, else 0
+            asm("v_bfe_i32 %0, %1, %2, 1" : "=v"(all) : "v"(nw), "n"(8 * (r >> 2) + (r & 3)));
+            sacc[mt][r] = __builtin_bit_cast(float, (uint32_t)all & 0xFF800000u);
+          }
+        }
+        s_product();
+      } else {
+  #pragma unroll
+        for (int i = 0; i < kMT; ++i)
+  #pragma unroll
+          for (int r = 0; r < 16; ++r) sacc[i][r] = 0.f;
+        s_product();
+      }
+
+      // ---- online softmax; one query per lane (shared with the partner lane ^ 32).
+      // The running max is only raised when the tile's max exceeds it by more than kLazy
+      // (in log2 units): probabilities then stay below 2^kLazy, well inside fp16 range, the
+      // normalisation by the running sum stays exact, and the O rescale becomes rare.
+      float mx = sacc[0][0];
+  #pragma unroll
+      for (int mt = 0; mt < kMT; ++mt)
+  #pragma unroll
+        for (int r = 0; r < 16; ++r) mx = fmaxf(mx, sacc[mt][r]);
+      mx = pair_max(mx);
+      const float m_new = (mx * p.c > m_run * p.c + kLazy || m_run == -INFINITY) ? mx : m_run;
+      // A row that has seen no allowed key yet has m_new == -inf: subtract 0 instead, so
+      // that its probabilities are exp2(-inf) = 0 and no inf - inf appears.
+      const float m_sub = (m_new == -INFINITY) ? 0.f : m_new;
+      const float alpha = __builtin_amdgcn_exp2f((m_run - m_sub) * p.c);
+      const float mc = m_sub * p.c;
+      half8_t pf[kMT][2];   // [key sub-tile][half]: B operand of O^T = V^T . P^T
+      float lsum = 0.f;
+  #pragma unroll
+      for (int mt = 0; mt < kMT; ++mt)
+  #pragma unroll
+        for (int r = 0; r < 16; r += 2) {
+          const float e0 = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[mt][r], p.c, -mc));
+          const float e1 = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[mt][r + 1], p.c, -mc));
+          const half2_t e2 = {(half_t)e0, (half_t)e1};
+          pf[mt][r >> 3][r & 7] = e2[0];
+          pf[mt][r >> 3][(r & 7) + 1] = e2[1];
+          // Row sum with plain adds: v_dot2c_f32_f16 would halve the instruction count but runs
+          // on the matrix pipeline and stalls behind every MFMA in flight on the SIMD.
+          lsum += e0 + e1;
+        }
+      l_run = l_run * alpha + lsum;   // per-lane partial sum; the two halves are added at the end
+      m_run = m_new;
+      if (__any(alpha != 1.0f)) {
+  #pragma unroll
+        for (int dt = 0; dt < 2; ++dt)
+  #pragma unroll
+          for (int r = 0; r < 16; ++r) oacc[dt][r] *= alpha;
+      }
+
+      // ---- O^T += V^T . P^T
+  #pragma unroll
+      for (int mt = 0; mt < kMT; ++mt)
+  #pragma unroll
+        for (int s2 = 0; s2 < 2; ++s2)
+  #pragma unroll
+          for (int dt = 0; dt < 2; ++dt) {
+            const lds_byte* vp = vt + (32 * (mt0 + mt) + 16 * s2) * 128;
+            const short4_t a0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4*)(vp + v_rd[dt][0]));
+            const short4_t a1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4*)(vp + v_rd[dt][1]));
+            const half8_t a = __builtin_bit_cast(half8_t, (short8_t)__builtin_shufflevector(a0, a1, 0, 1, 2, 3, 4, 5, 6, 7));
+            oacc[dt] = mfma32(a, pf[mt][s2], oacc[dt]);
+          }
+    };
+
+    Step cur = next_step();
+    if (cur.valid) issue_tile(cur.col, (lds_byte*)k_lds0, (lds_byte*)v_lds0);
+    while (cur.valid) {   // single exit: an early exit between the two steps makes the compiler copy the accumulators
+      Step nxt = next_step();
+      step(cur, nxt, (const lds_byte*)k_lds0, (const lds_byte*)v_lds0, (lds_byte*)k_lds1, (lds_byte*)v_lds1);
+      cur = nxt;
+      if (nxt.valid) {
+        cur = next_step();
+        step(nxt, cur, (const lds_byte*)k_lds1, (const lds_byte*)v_lds1, (lds_byte*)k_lds0, (lds_byte*)v_lds0);
+      }
     }
   }
 

@@ -174,7 +174,7 @@ def test_encoder_layer_c3(fusion, B):
     want16 = oe.bert_layer(x, w, mask.float(), H, eps=1e-12, round_fp16=True if runs_fused else "split")
     want32 = oe.bert_layer(x, w, mask.float(), H, eps=1e-12)
     valid = torch.arange(S)[None, :] < L[:, None]          # rows past the sample length are don't-care
-    _layer_checks(got, want16, want32, f"C3 layer B{B} {fusion}", 4e-3, valid)
+    _layer_checks(got, want16, want32, f"C3 layer B{B} {fusion}", 5e-3, valid)   # observed 2.9e-3 (B4), 3.3e-3 (B16)
 
 
 @pytest.mark.parametrize("act", ["tanh", "relu"])
@@ -189,7 +189,7 @@ def test_encoder_layer_gpt_and_t5_activations(act):
     got = layer(x.cuda(), lut)
     mode = True if layer._fuse(B * S) else "split"
     _layer_checks(got, oe.bert_layer(x, w, mask.float(), H, eps=1e-12, gelu=act, round_fp16=mode),
-                  oe.bert_layer(x, w, mask.float(), H, eps=1e-12, gelu=act), f"layer {act}", 4e-3)
+                  oe.bert_layer(x, w, mask.float(), H, eps=1e-12, gelu=act), f"layer {act}", 5e-3)   # observed 3.5e-3
     with pytest.raises(ValueError):
         EncoderLayer({k: v.cuda() for k, v in w.items()}, H, gelu="swish")
 
@@ -235,7 +235,7 @@ def test_encoder_stack_c5_full_size():
             xin = x.cpu()
             want16 = oe.bert_layer(xin, w, mask.float()[None], cfg.heads, eps=cfg.eps, round_fp16=mode)
             want32 = oe.bert_layer(xin, w, mask.float()[None], cfg.heads, eps=cfg.eps)
-            _layer_checks(y, want16, want32, f"C5 layer {i + 1} of 24", 4e-3)
+            _layer_checks(y, want16, want32, f"C5 layer {i + 1} of 24", 5e-3)   # observed 3.1e-3 .. 3.8e-3
             worst16 = max(worst16, _max_err(y, want16)); worst32 = max(worst32, _max_err(y, want32))
         x = y
     assert bool(torch.isfinite(x.float()).all())
