@@ -56,7 +56,7 @@ enum {
 enum { STOF_ACT_NONE = 0, STOF_ACT_GELU_ERF = 1, STOF_ACT_GELU_TANH = 2, STOF_ACT_RELU = 3 };
 
 /* launch form of the attention entry points */
-enum { STOF_FORM_DEFAULT = -1, STOF_FORM_TWO_ROWS = 0, STOF_FORM_KEY_SPLIT = 1 };
+enum { STOF_FORM_DEFAULT = -1, STOF_FORM_TWO_ROWS = 0, STOF_FORM_KEY_SPLIT = 1, STOF_FORM_PIPELINED = 2 };
 
 /* rowwise front-end selector of stof_rowwise_attn_fwd */
 enum { STOF_ROW_FULL = 0, STOF_ROW_SLIDING = 1, STOF_ROW_MASK = 2 };

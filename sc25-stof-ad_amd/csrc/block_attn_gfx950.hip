@@ -112,7 +112,8 @@ template <int ROWS> struct RowPtrs {
 template <int KIND, int ROWS, int KS, bool PIPE = false>
 __device__ __forceinline__ void attn_group(const AttnParams& p, const int bh, const int pair, const RowPtrs<ROWS>& pre,
                                            unsigned char* k_lds0, unsigned char* k_lds1,
-                                           unsigned char* v_lds0, unsigned char* v_lds1) {
+                                           unsigned char* v_lds0, unsigned char* v_lds1,
+                                           unsigned char* k_lds2 = nullptr, unsigned char* v_lds2 = nullptr) {
   static_assert(KS == 1 || ROWS == 1, "the key split serves a single query block");
   static_assert(!PIPE || KS == 1, "the software-pipelined loop keeps all 64 keys of a tile in one wave");
   constexpr int kDma = 4 / (ROWS * KS);   // direct-to-LDS instructions per wave and operand tile (8 per tile)
@@ -244,6 +245,9 @@ __device__ __forceinline__ void attn_group(const AttnParams& p, const int bh, co
     for (int r = 0; r < 16; ++r) oacc[i][r] = 0.f;
   float m_run = -INFINITY;
   float l_run = 0.f;
+  float mc_run = 0.f;      // running max * c, what the exponent subtracts
+  bool warm = false;       // every lane of the wave has a finite running max
+  constexpr float kSumLimit = 16384.f;   // 32 probabilities of at most 2^kLazy sum to 2^13
 
   auto issue_tile = [&](int col, lds_byte* kdst, lds_byte* vdst) {
     const char* kt = reinterpret_cast<const char*>(kb + (int64_t)col * kBN * p.ks[2]);
@@ -310,63 +314,79 @@ __device__ __forceinline__ void attn_group(const AttnParams& p, const int bh, co
   };
 
   if constexpr (PIPE) {
-    // ---- software-pipelined main loop.
-    // Iteration i holds three tiles of the wave's chain at once: the scores of tile i+1 are
-    // produced (S = K Q^T, 8 MFMA), the probabilities of tile i are formed from the scores made
-    // one iteration ago (exp2, convert, row sum: vector ALU only) and the probabilities of tile
-    // i-1 go into O (O += V^T P^T, 8 MFMA).  The three are independent of one another, so inside
-    // ONE wave every MFMA is followed by vector-ALU work that does not wait for it: the matrix
-    // pipeline and the vector ALU run side by side.  (Across waves they overlap badly: an MFMA
-    // that waits for the pipeline holds the SIMD's issue slot.)
+    // ---- software-pipelined main loop, in units of HALF a tile (32 keys x this wave's 32 queries).
+    // For unit u the wave has three pieces of work: A(u) its scores S = K Q^T (4 MFMA), B(u) its
+    // probabilities exp2(S c - m c) with their row sum (vector ALU only) and C(u) its share of
+    // O += V^T P^T (4 MFMA).  A half-step runs A(u+1), B(u) and C(u-1) together: they are
+    // independent of one another, so inside ONE wave every MFMA is followed by vector-ALU work
+    // that does not wait for it, and the matrix pipeline and the vector ALU run side by side.
+    // (Across waves they overlap badly: an MFMA that waits for the pipeline holds the SIMD's
+    // issue slot.)  Per tile i, between two barriers, the wave runs two half-steps,
+    //     A(i, keys 32-63) | B(i, keys 0-31)  | C(i-1, keys 32-63)
+    //     A(i+1, keys 0-31) | B(i, keys 32-63) | C(i, keys 0-31)
+    // so one unit of scores (16 registers) and one unit of probabilities (8) cross an iteration.
     //
-    // Running max: the fast path takes the max as it stands and only verifies, from the row sums
-    // it needs anyway, that no probability left the fp16 range; if one did (or a lane has not
-    // seen a key yet, or a tile needs an element mask, or a neighbour tile is not this wave's),
-    // the iteration runs the general path below: exact online softmax with max search and
-    // rescale, one piece after the other.  O holds tile i-1 by then, so the rescale is the usual one.
+    // There is ONE code path for every unit (two paths that both update the accumulators cost
+    // some 90 registers at their merge points).  What differs is decided by small side blocks:
+    //  * a unit of a tile the wave's row does not list, or of a slot before the first / after
+    //    the last tile, is computed like any other but subtracts +inf in the exponent, so its
+    //    probabilities are exactly zero (the tile buffers are zero-filled once at the start, so
+    //    every operand is finite);
+    //  * a masked unit has -inf added to the scores of its masked elements, in place, before its
+    //    softmax;
+    //  * the running max: normally it is taken as it stands and the unit only verifies, from the
+    //    row sum it needs anyway, that no probability left the fp16 range (the max would have to
+    //    rise by more than 2^14 inside one unit).  While a lane has not seen a key yet the unit is
+    //    preceded by the exact update (max search, lazy raise, rescale of O, of the sum and of
+    //    the previous unit's probabilities, which go into O during this half-step).  A failed
+    //    verification raises a flag, and once the walk is over a workgroup with a raised flag
+    //    runs the whole walk a second time with the exact update before every unit.
     //
-    // LDS: K is fetched two tiles ahead of V (iteration i issues K(i+2) and V(i), reads K(i+1) and
-    // V(i-1)); with two buffers each, an iteration reads one buffer pair and fills the other.
-    struct Tile { Step st; bool mask; };
+    // LDS: rings of three K and three V tiles.  Iteration i reads K(i), K(i+1), V(i-1), V(i) and
+    // issues the loads of K(i+2) and V(i+1) into the buffers iteration i-1 read last.
+    enum { kValid = 1, kMine = 2, kMask = 4 };   // tile flags: listed by the walk, used by this wave's row, needs its element mask
+    struct Tile { int col, slot, f; };
+    const uint32_t k_tile_bytes = (uint32_t)(kBN * 2 * p.ks[2]), v_tile_bytes = (uint32_t)(kBN * 2 * p.vs[2]);   // < 2^28: strides_ok
     auto dma_k = [&](int col, lds_byte* kdst) {
-      const char* kt = reinterpret_cast<const char*>(kb + (int64_t)col * kBN * p.ks[2]);
+      const char* kt = reinterpret_cast<const char*>(kb) + (uint64_t)(uint32_t)col * k_tile_bytes;
       lds_byte* kd = kdst + (kDma * wave) * 1024;
 #pragma unroll
       for (int i = 0; i < kDma; ++i)
         __builtin_amdgcn_global_load_lds((gptr_t*)(kt + k_src[i]), (__attribute__((address_space(3))) void*)(kd + i * 1024), 16, 0, 0);
     };
     auto dma_v = [&](int col, lds_byte* vdst) {
-      const char* vt = reinterpret_cast<const char*>(vb + (int64_t)col * kBN * p.vs[2]);
+      const char* vt = reinterpret_cast<const char*>(vb) + (uint64_t)(uint32_t)col * v_tile_bytes;
       lds_byte* vd = vdst + (kDma * wave) * 1024;
 #pragma unroll
       for (int i = 0; i < kDma; ++i)
         __builtin_amdgcn_global_load_lds((gptr_t*)(vt + v_src[i]), (__attribute__((address_space(3))) void*)(vd + i * 1024), 16, 0, 0);
     };
     // element-mask word of this lane's query for a tile (requested when the tile enters the queue)
-    auto request_bits = [&](const Step& st) -> uint64_t {
+    auto request_bits = [&](const Tile& t) -> uint64_t {
       uint64_t bits = ~0ull;
       if (KIND == kKindLut) {
-        if (st.valid && st.slot >= 0) bits = p.pbits[(int64_t)st.slot * kBM + 32 * half + j32];
+        if (t.slot >= 0) bits = p.pbits[(int64_t)t.slot * kBM + 32 * half + j32];
       } else if (KIND == kKindBits) {
-        if (st.valid && st.mine) bits = p.row_bits[(qrow0 + j32) * p.words + st.col];
+        if (t.f & kMine) bits = p.row_bits[(qrow0 + j32) * p.words + t.col];
       }
       return bits;
     };
     // whether the tile needs its element mask (wave-uniform); the index predicates of the
     // row-wise front-ends are folded into the bit row; a tile that allows nothing is dropped
     auto settle_mask = [&](Tile& t, uint64_t& bits) {
-      t.mask = false;
-      if (!t.st.valid || !t.st.mine) return;
-      if (KIND == kKindLut) { t.mask = t.st.slot >= 0; return; }
-      const int qmin = (int)qrow0, qmax = qmin + 31, kmin = t.st.col * kBN, kmax = kmin + kBN - 1;
+      if (KIND == kKindLut) return;                  // decided by the walk: a PART slot
+      if (!(t.f & kMine)) return;
+      const int qmin = (int)qrow0, qmax = qmin + 31, kmin = t.col * kBN, kmax = kmin + kBN - 1;
       const bool range_full = (!p.causal || kmax <= qmin) && (!(KIND == kKindPred && p.band > 0) || kmin > qmax - p.band);
+      bool mask;
       if (KIND == kKindBits) {
-        if (!__any(bits != 0ull)) { t.st.mine = 0; return; }
-        t.mask = !range_full || __any(bits != ~0ull);
+        if (!__any(bits != 0ull)) { t.f &= ~kMine; return; }
+        mask = !range_full || __any(bits != ~0ull);
       } else {
-        t.mask = !range_full;
+        mask = !range_full;
       }
-      if (t.mask) {
+      if (mask) {
+        t.f |= kMask;
         const int qg = qmin + j32;
         if (p.causal) { const int nk = qg - kmin + 1; bits &= nk >= 64 ? ~0ull : (nk <= 0 ? 0ull : ((1ull << nk) - 1)); }
         if (KIND == kKindPred && p.band > 0) {
@@ -375,175 +395,239 @@ __device__ __forceinline__ void attn_group(const AttnParams& p, const int bh, co
         }
       }
     };
-    // S^T = K . Q^T into s (see the accumulator layout at the non-pipelined step)
-    auto qk_product = [&](const lds_byte* kt, floatx16 (&s)[2]) {
+    // Element mask of a unit, applied to its finished scores in place: -inf where the key is not
+    // allowed (added as a 0 / -inf bias: sign-extended one-bit field of the inverted mask word,
+    // AND with the bit pattern of -inf, add).
+    auto apply_mask = [&](floatx16& sc, uint32_t unit_bits) {
+      const uint32_t nw = ~(unit_bits >> (4 * g));   // bit set = key masked
 #pragma unroll
-      for (int ks = 0; ks < 4; ++ks)
-#pragma unroll
-        for (int mt = 0; mt < 2; ++mt) {
-          const half8_t a = *reinterpret_cast<const __attribute__((address_space(3))) half8_t*>(kt + mt * 4096 + k_rd[ks]);
-          s[mt] = mfma32(a, qf[ks], s[mt]);
-        }
-    };
-    auto init_scores = [&](floatx16 (&s)[2], bool masked, uint64_t bits) {
-      if (masked) {
-#pragma unroll
-        for (int mt = 0; mt < 2; ++mt) {
-          const uint32_t nw = ~((uint32_t)(bits >> (32 * mt)) >> (4 * g));   // bit set = key masked
-#pragma unroll
-          for (int r = 0; r < 16; ++r) {
-            int all;   // -1 if masked, else 0
-            asm("v_bfe_i32 %0, %1, %2, 1" : "=v"(all) : "v"(nw), "n"(8 * (r >> 2) + (r & 3)));
-            s[mt][r] = __builtin_bit_cast(float, (uint32_t)all & 0xFF800000u);
-          }
-        }
-      } else {
-#pragma unroll
-        for (int mt = 0; mt < 2; ++mt)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) s[mt][r] = 0.f;
+      for (int r = 0; r < 16; ++r) {
+        int all;   // -1 if masked, else 0
+        asm("v_bfe_i32 %0, %1, %2, 1" : "=v"(all) : "v"(nw), "n"(8 * (r >> 2) + (r & 3)));
+        sc[r] += __builtin_bit_cast(float, (uint32_t)all & 0xFF800000u);
       }
     };
-    // O^T += V^T . P^T
-    auto pv_product = [&](const lds_byte* vt, const half8_t (&pf)[2][2]) {
-#pragma unroll
-      for (int mt = 0; mt < 2; ++mt)
-#pragma unroll
-        for (int s2 = 0; s2 < 2; ++s2)
-#pragma unroll
-          for (int dt = 0; dt < 2; ++dt) {
-            const lds_byte* vp = vt + (32 * mt + 16 * s2) * 128;
-            const short4_t a0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4*)(vp + v_rd[dt][0]));
-            const short4_t a1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4*)(vp + v_rd[dt][1]));
-            const half8_t a = __builtin_bit_cast(half8_t, (short8_t)__builtin_shufflevector(a0, a1, 0, 1, 2, 3, 4, 5, 6, 7));
-            oacc[dt] = mfma32(a, pf[mt][s2], oacc[dt]);
-          }
+    // vh: the unit's half of a V tile buffer (key rows 32 mt .. 32 mt + 31)
+    auto v_frag = [&](const lds_byte* vh, int s2, int dt) -> half8_t {
+      const lds_byte* vp = vh + 16 * s2 * 128;
+      const short4_t a0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4*)(vp + v_rd[dt][0]));
+      const short4_t a1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4*)(vp + v_rd[dt][1]));
+      return __builtin_bit_cast(half8_t, (short8_t)__builtin_shufflevector(a0, a1, 0, 1, 2, 3, 4, 5, 6, 7));
     };
-    bool warm = false;   // every lane of the wave has a finite running max
-    float mc = 0.f;      // running max * c, the constant the fast softmax subtracts
-    // exact online softmax of one tile (max search, lazy raise, rescale of O and of the sum)
-    auto softmax_exact = [&](const floatx16 (&s)[2], half8_t (&pf)[2][2]) {
-      float mx = s[0][0];
+    // Exact update of the running max ahead of a unit's softmax: s = the unit's scores, p_prev =
+    // the previous unit's probabilities (they enter O during this half-step, so they are brought
+    // to the new max along with O and the running sum).
+    auto exact_update = [&](const floatx16& s, half8_t (&p_prev)[2]) {
+      float mx = s[0];
 #pragma unroll
-      for (int mt = 0; mt < 2; ++mt)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s[mt][r]);
+      for (int r = 1; r < 16; ++r) mx = fmaxf(mx, s[r]);
       mx = pair_max(mx);
       const float m_new = (mx * p.c > m_run * p.c + kLazy || m_run == -INFINITY) ? mx : m_run;
       const float m_sub = (m_new == -INFINITY) ? 0.f : m_new;
       const float alpha = __builtin_amdgcn_exp2f((m_run - m_sub) * p.c);
-      mc = m_sub * p.c;
-      float lsum = 0.f;
-#pragma unroll
-      for (int mt = 0; mt < 2; ++mt)
-#pragma unroll
-        for (int r = 0; r < 16; r += 2) {
-          const float e0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[mt][r], p.c, -mc));
-          const float e1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[mt][r + 1], p.c, -mc));
-          const half2_t e2 = {(half_t)e0, (half_t)e1};
-          pf[mt][r >> 3][r & 7] = e2[0];
-          pf[mt][r >> 3][(r & 7) + 1] = e2[1];
-          lsum += e0 + e1;
-        }
-      l_run = l_run * alpha + lsum;
+      mc_run = m_sub * p.c;
       m_run = m_new;
+      l_run *= alpha;
       if (__any(alpha != 1.0f)) {
 #pragma unroll
         for (int dt = 0; dt < 2; ++dt)
 #pragma unroll
           for (int r = 0; r < 16; ++r) oacc[dt][r] *= alpha;
+        const half_t ah = (half_t)alpha;
+#pragma unroll
+        for (int s2 = 0; s2 < 2; ++s2)
+#pragma unroll
+          for (int e = 0; e < 8; ++e) p_prev[s2][e] *= ah;
       }
       warm = !__any(m_run == -INFINITY);
     };
-    // Fast softmax: the max is taken as it stands.  The row sum is formed from the fp16
-    // probabilities themselves (the values the second product uses) by a tree of packed adds,
-    // folded to fp32 once; a probability beyond the fp16 range shows up in it as inf or as a
-    // large sum, which the caller tests before it commits the tile.
-    auto softmax_fast = [&](const floatx16 (&s)[2], half8_t (&pf)[2][2]) -> float {
-      half2_t acc[16];
-#pragma unroll
-      for (int mt = 0; mt < 2; ++mt)
-#pragma unroll
-        for (int r = 0; r < 16; r += 2) {
-          const float e0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[mt][r], p.c, -mc));
-          const float e1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[mt][r + 1], p.c, -mc));
-          const half2_t e2 = {(half_t)e0, (half_t)e1};
-          pf[mt][r >> 3][r & 7] = e2[0];
-          pf[mt][r >> 3][(r & 7) + 1] = e2[1];
-          acc[8 * mt + (r >> 1)] = e2;
-        }
-#pragma unroll
-      for (int w = 8; w > 0; w >>= 1)
-#pragma unroll
-        for (int i = 0; i < w; ++i) acc[i] = acc[i] + acc[i + w];
-      return (float)acc[0][0] + (float)acc[0][1];
-    };
-    constexpr float kSumLimit = 16384.f;   // 32 probabilities of at most 2^kLazy sum to 2^13
 
-    Tile t0, t1, t2, t3;   // tiles i-1 (PV), i (softmax), i+1 (QK^T), i+2 (loads)
-    t0.st.valid = t1.st.valid = t2.st.valid = false;
-    t0.st.mine = t1.st.mine = t2.st.mine = 0;
-    t0.st.col = t1.st.col = t2.st.col = 0; t0.st.slot = t1.st.slot = t2.st.slot = -1;
-    t0.mask = t1.mask = t2.mask = t3.mask = false;
-    t3.st = next_step();
-    uint64_t bits2 = ~0ull;          // mask word of tile t2
-    floatx16 sA[2], sB[2];
-    half8_t pA[2][2], pB[2][2];
+    // The walk as a table.  Finding the next key block in the bit sets costs some twenty scalar
+    // instructions per tile, which a wave issues one at a time between its vector work; with few
+    // waves per SIMD nothing hides them.  Per window of 64 key blocks the walk is therefore laid
+    // out once: the k-th block of the union goes to lane k of `table` (column inside the window,
+    // whether this wave's row lists it, whether it is partial there, and its rank in the row's
+    // PART list), by one forward lane permutation; a step is then one v_readlane.
+    int table = 0, tab_n = 0, tab_i = 0;
+    auto build_table = [&]() {
+      const uint64_t below = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
+      const int rank = __builtin_popcountll(set_union & below);
+      tab_n = __builtin_popcountll(set_union);
+      tab_i = 0;
+      const bool in_u = (set_union >> lane) & 1;
+      const int dst = in_u ? rank : tab_n + (lane - rank);          // a permutation of the 64 lanes
+      const int info = lane | ((int)((set_mine >> lane) & 1) << 6) | ((int)((set_part >> lane) & 1) << 7) |
+                       (__builtin_popcountll(set_part & below) << 8);
+      table = __builtin_amdgcn_ds_permute(dst << 2, info);
+      set_union = 0;   // the window is handed out through the table from here on
+    };
+    build_table();   // window 0 (consumed above)
+    auto next_tile = [&]() -> Tile {
+      Tile t; t.col = 0; t.slot = -1; t.f = 0;
+      while (tab_i >= tab_n) {
+        if (++win >= n_win) return t;
+        fetch_window();
+        consume_window(win);
+        build_table();
+      }
+      const int info = __builtin_amdgcn_readlane(table, tab_i++);
+      t.col = 64 * win + (info & 63);
+      t.f = kValid | ((info >> 5) & kMine);                        // bit 6 of the entry
+      if (KIND == kKindLut && (info & 0xC0) == 0xC0) { t.slot = part_base + (info >> 8); t.f |= kMask; }
+      return t;
+    };
+
+    Tile t0, t1, t2, t3;   // tiles i-1, i, i+1, i+2 of the walk
+    uint64_t bits1 = ~0ull, bits2 = ~0ull;   // mask words of tiles t1 and t2
+    int prio_in = 1;
+    floatx16 sU, sN;       // scores: of the unit whose softmax is next, of the unit after it
+    half8_t pU[2], pN[2];  // probabilities: of the unit whose PV product is next, of the unit after it
+    bool safe = false;       // second pass: exact path only
+    bool overflow = false;   // a fast unit failed its verification
+    const int chain_len = steps_left;
+
+    // One half-step: 8 slices, slice c = MFMA c (even: A, odd: C), the LDS fragment of a later
+    // MFMA and the softmax of one pair of scores (2 fma, 2 exp2, 1 convert, 1 packed add: about
+    // the issue time of the MFMA).  The slices are fenced so that the compiler keeps this order;
+    // inside a slice it is free.  Returns the unit's row sum.  frag[] holds the operands of this
+    // half-step's MFMAs (the first kAhead requested by the caller); fetch_next requests operands
+    // of the half-step that follows, so that its first MFMAs do not wait for LDS.
+    // sub: the exponent's subtrahend, mc_run or +inf (a unit that is not this wave's).
+    constexpr int kAhead = 2;
+    auto half_step = [&](auto&& fetch_this, auto&& fetch_next, half8_t (&frag)[8], half8_t (&frag_next)[8], bool has_next,
+                         const floatx16& s_in, floatx16& s_out, const half8_t (&p_in)[2], half8_t (&p_out)[2],
+                         float sub) -> float {
 #pragma unroll
-    for (int mt = 0; mt < 2; ++mt) {
+      for (int r = 0; r < 16; ++r) s_out[r] = 0.f;
+      half2_t part[4];
 #pragma unroll
-      for (int r = 0; r < 16; ++r) { sA[mt][r] = 0.f; sB[mt][r] = 0.f; }
+      for (int c = 0; c < 8; ++c) {
+        __builtin_amdgcn_sched_barrier(0);
+        const int j = c >> 1;
+        if (c & 1) oacc[j & 1] = mfma32(frag[c], p_in[j >> 1], oacc[j & 1]);
+        else s_out = mfma32(frag[c], qf[j], s_out);
+        if (c + kAhead < 8) frag[c + kAhead] = fetch_this(c + kAhead);
+        else if (has_next) frag_next[c + kAhead - 8] = fetch_next(c + kAhead - 8);
+        const int r = 2 * c;
+        const float e0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s_in[r], p.c, -sub));
+        const float e1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s_in[r + 1], p.c, -sub));
+        const half2_t e2 = {(half_t)e0, (half_t)e1};
+        p_out[r >> 3][r & 7] = e2[0];
+        p_out[r >> 3][(r & 7) + 1] = e2[1];
+        part[c & 3] = c < 4 ? e2 : part[c & 3] + e2;
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      // (Pin the probabilities here: being pure arithmetic that is only read by the next half-step,
+      // they would otherwise be sunk out of the slices, past the side blocks in between.)
+      asm volatile("" : "+v"(p_out[0]), "+v"(p_out[1]));
+      const half2_t tot = (part[0] + part[1]) + (part[2] + part[3]);
+      return (float)tot[0] + (float)tot[1];
+    };
+
+    // One iteration.  k_cur / k_nxt / v_prv / v_cur: the ring buffers of K(i), K(i+1), V(i-1), V(i);
+    // k_fill / v_fill: where K(i+2) and V(i+1) go.
+    auto iteration = [&](const lds_byte* k_cur, const lds_byte* k_nxt, const lds_byte* v_prv, const lds_byte* v_cur,
+                         lds_byte* k_fill, lds_byte* v_fill) {
+      if (--prio_in == 0) {   // issue priority by remaining chain length, looked at once per kPrioStep tiles
+        prio_in = kPrioStep;
+        steps_left -= kPrioStep;
+        if (steps_left >= 3 * kPrioStep) __builtin_amdgcn_s_setprio(3);
+        else if (steps_left >= 2 * kPrioStep) __builtin_amdgcn_s_setprio(2);
+        else if (steps_left >= kPrioStep) __builtin_amdgcn_s_setprio(1);
+        else __builtin_amdgcn_s_setprio(0);
+      }
+      __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): K(i+1), V(i) and the mask word of tile i+1 have landed
+      __syncthreads();
+      if (t3.f & kValid) dma_k(t3.col, k_fill);
+      if (t2.f & kValid) dma_v(t2.col, v_fill);
+      const uint64_t bits3 = request_bits(t3);
+      settle_mask(t2, bits2);
+      const lds_byte* ka = k_cur + 4096;   // A(i, keys 32-63)
+      const lds_byte* kb2 = k_nxt;         // A(i+1, keys 0-31)
+      const lds_byte* va = v_prv + 4096;   // C(i-1, keys 32-63)
+      const lds_byte* vb2 = v_cur;         // C(i, keys 0-31)
+      half8_t f1[8], f2[8];
+      auto fetch1 = [&](int m) -> half8_t {
+        if (m & 1) return v_frag(va, (m >> 1) >> 1, (m >> 1) & 1);
+        return *reinterpret_cast<const __attribute__((address_space(3))) half8_t*>(ka + k_rd[m >> 1]);
+      };
+      auto fetch2 = [&](int m) -> half8_t {
+        if (m & 1) return v_frag(vb2, (m >> 1) >> 1, (m >> 1) & 1);
+        return *reinterpret_cast<const __attribute__((address_space(3))) half8_t*>(kb2 + k_rd[m >> 1]);
+      };
+#pragma unroll
+      for (int m = 0; m < kAhead; ++m) f1[m] = fetch1(m);
+      const bool mine1 = (t1.f & kMine) != 0;
+      const bool exact = mine1 && (safe || !warm);
+      const bool mask1 = (t1.f & kMask) != 0;
+      // ---- half-step 1: A(i, keys 32-63) -> sN | B(i, keys 0-31): sU -> pN | C(i-1, keys 32-63): pU
+      if (mask1) apply_mask(sU, (uint32_t)bits1);
+      if (exact) exact_update(sU, pU);
+      const float sum1 = half_step(fetch1, fetch2, f1, f2, true, sU, sN, pU, pN, mine1 ? mc_run : INFINITY);
+      l_run += sum1;
+      // ---- half-step 2: A(i+1, keys 0-31) -> sU | B(i, keys 32-63): sN -> pU | C(i, keys 0-31): pN
+      if (mask1) apply_mask(sN, (uint32_t)(bits1 >> 32));
+      if (mine1 && (safe || !warm)) exact_update(sN, pN);
+      const float sum2 = half_step(fetch2, fetch2, f2, f1, false, sN, sU, pN, pU, mine1 ? mc_run : INFINITY);
+      l_run += sum2;
+      overflow |= __any(!(sum1 < kSumLimit) || !(sum2 < kSumLimit));
+      t0 = t1; t1 = t2; t2 = t3;
+      bits1 = bits2; bits2 = bits3;
+      t3 = next_tile();
+    };
+
+    // The tile buffers start as zeros: a slot before the first tile is then read as finite numbers.
+    {
+      const floatx4 z = {0.f, 0.f, 0.f, 0.f};
+      unsigned char* bufs[6] = {k_lds0, k_lds1, k_lds2, v_lds0, v_lds1, v_lds2};
+#pragma unroll
+      for (int bI = 0; bI < 6; ++bI)
+#pragma unroll
+        for (int i = 0; i < kTile / (256 * 16); ++i) *reinterpret_cast<floatx4*>(bufs[bI] + (i * 256 + threadIdx.x) * 16) = z;
+    }
+
+    for (;;) {
+      t0.col = t1.col = t2.col = 0; t0.slot = t1.slot = t2.slot = -1; t0.f = t1.f = t2.f = 0;
+      t3 = next_tile();
+      bits1 = bits2 = ~0ull;
+      prio_in = 1;                           // (the first iteration sets the priority)
+      steps_left = chain_len + kPrioStep;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) { sU[r] = 0.f; sN[r] = 0.f; }
 #pragma unroll
       for (int s2 = 0; s2 < 2; ++s2)
 #pragma unroll
-        for (int e = 0; e < 8; ++e) { pA[mt][s2][e] = (half_t)0.f; pB[mt][s2][e] = (half_t)0.f; }
-    }
-
-    // One iteration: reads the buffer pair (kr, vr), fills (kw, vw); scores s_in -> probabilities
-    // p_out, scores of the next tile -> s_out, probabilities p_in -> O.
-    auto iteration = [&](const lds_byte* kr, const lds_byte* vr, lds_byte* kw, lds_byte* vw,
-                         floatx16 (&s_in)[2], floatx16 (&s_out)[2], half8_t (&p_in)[2][2], half8_t (&p_out)[2][2]) {
-      {
-        const int left = steps_left--;
-        if (left >= 3 * kPrioStep) __builtin_amdgcn_s_setprio(3);
-        else if (left >= 2 * kPrioStep) __builtin_amdgcn_s_setprio(2);
-        else if (left >= kPrioStep) __builtin_amdgcn_s_setprio(1);
-        else __builtin_amdgcn_s_setprio(0);
+        for (int e = 0; e < 8; ++e) { pU[s2][e] = (half_t)0.f; pN[s2][e] = (half_t)0.f; }
+      while ((t0.f | t1.f | t2.f | t3.f) & kValid) {   // single exit; tile i uses ring slot (i + 2) mod 3
+        iteration((const lds_byte*)k_lds0, (const lds_byte*)k_lds1, (const lds_byte*)v_lds2, (const lds_byte*)v_lds0, (lds_byte*)k_lds2, (lds_byte*)v_lds1);
+        iteration((const lds_byte*)k_lds1, (const lds_byte*)k_lds2, (const lds_byte*)v_lds0, (const lds_byte*)v_lds1, (lds_byte*)k_lds0, (lds_byte*)v_lds2);
+        iteration((const lds_byte*)k_lds2, (const lds_byte*)k_lds0, (const lds_byte*)v_lds1, (const lds_byte*)v_lds2, (lds_byte*)k_lds1, (lds_byte*)v_lds0);
       }
-      __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): K(i+1), V(i-1) and the mask word of tile i+1 have landed
+      if (safe) break;
+      // Did a fast unit of any of the four waves fail its verification?  (They share the tile
+      // loads and the barriers, so the workgroup repeats the walk as a whole.)
+      int* flag = reinterpret_cast<int*>(k_lds0);
+      __syncthreads();                              // every wave is out of the loop: the tile buffers are free
+      if (threadIdx.x == 0) *flag = 0;
       __syncthreads();
-      if (t3.st.valid) dma_k(t3.st.col, kw);
-      if (t1.st.valid) dma_v(t1.st.col, vw);
-      const uint64_t bits3 = request_bits(t3.st);
-      settle_mask(t2, bits2);
-      const bool do_pv = t0.st.valid && t0.st.mine, do_sm = t1.st.valid && t1.st.mine, do_qk = t2.st.valid && t2.st.mine;
-      if (do_pv && do_sm && do_qk && !t2.mask && warm) {
-        init_scores(s_out, false, 0);
-        qk_product(kr, s_out);
-        const float lsum = softmax_fast(s_in, p_out);
-        pv_product(vr, p_in);
+      if (overflow && lane == 0) *flag = 1;
+      __syncthreads();
+      const int again = __builtin_amdgcn_readfirstlane(*reinterpret_cast<volatile int*>(flag));
+      __syncthreads();
+      if (!again) break;
+      // second pass from the start of the walk, exact path only
+      safe = true;
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
-          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // one MFMA
-          __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);   // LDS fragment reads of the MFMAs to come
-          __builtin_amdgcn_sched_group_barrier(0x400, 2, 0);   // two exp2
-          __builtin_amdgcn_sched_group_barrier(0x002, 5, 0);   // scale, convert, sum
-        }
-        if (__any(!(lsum < kSumLimit))) softmax_exact(s_in, p_out);
-        else l_run += lsum;
-      } else {
-        if (do_qk) { init_scores(s_out, t2.mask, bits2); qk_product(kr, s_out); }
-        if (do_pv) pv_product(vr, p_in);
-        if (do_sm) softmax_exact(s_in, p_out);
-      }
-      t0 = t1; t1 = t2; t2 = t3;
-      bits2 = bits3;
-      t3.st = next_step(); t3.mask = false;
-    };
-
-    while (t0.st.valid || t1.st.valid || t2.st.valid || t3.st.valid) {   // single exit
-      iteration((const lds_byte*)k_lds1, (const lds_byte*)v_lds1, (lds_byte*)k_lds0, (lds_byte*)v_lds0, sA, sB, pA, pB);
-      iteration((const lds_byte*)k_lds0, (const lds_byte*)v_lds0, (lds_byte*)k_lds1, (lds_byte*)v_lds1, sB, sA, pB, pA);
+      for (int dt = 0; dt < 2; ++dt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) oacc[dt][r] = 0.f;
+      m_run = -INFINITY; l_run = 0.f; mc_run = 0.f; warm = false;
+#pragma unroll
+      for (int r = 0; r < ROWS; ++r) { row[r].ptr = 0; row[r].pptr = 0; }
+      win = 0;
+      fetch_window();
+      consume_window(0);
+      build_table();
     }
   } else {
     // one key block: kt/vt hold the current tile, the next tile's loads go to kn/vn
@@ -638,41 +722,52 @@ __device__ __forceinline__ void attn_group(const AttnParams& p, const int bh, co
       // The running max is only raised when the tile's max exceeds it by more than kLazy
       // (in log2 units): probabilities then stay below 2^kLazy, well inside fp16 range, the
       // normalisation by the running sum stays exact, and the O rescale becomes rare.
-      float mx = sacc[0][0];
-  #pragma unroll
-      for (int mt = 0; mt < kMT; ++mt)
-  #pragma unroll
-        for (int r = 0; r < 16; ++r) mx = fmaxf(mx, sacc[mt][r]);
-      mx = pair_max(mx);
-      const float m_new = (mx * p.c > m_run * p.c + kLazy || m_run == -INFINITY) ? mx : m_run;
-      // A row that has seen no allowed key yet has m_new == -inf: subtract 0 instead, so
-      // that its probabilities are exp2(-inf) = 0 and no inf - inf appears.
-      const float m_sub = (m_new == -INFINITY) ? 0.f : m_new;
-      const float alpha = __builtin_amdgcn_exp2f((m_run - m_sub) * p.c);
-      const float mc = m_sub * p.c;
-      half8_t pf[kMT][2];   // [key sub-tile][half]: B operand of O^T = V^T . P^T
-      float lsum = 0.f;
-  #pragma unroll
-      for (int mt = 0; mt < kMT; ++mt)
-  #pragma unroll
-        for (int r = 0; r < 16; r += 2) {
-          const float e0 = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[mt][r], p.c, -mc));
-          const float e1 = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[mt][r + 1], p.c, -mc));
-          const half2_t e2 = {(half_t)e0, (half_t)e1};
-          pf[mt][r >> 3][r & 7] = e2[0];
-          pf[mt][r >> 3][(r & 7) + 1] = e2[1];
-          // Row sum with plain adds: v_dot2c_f32_f16 would halve the instruction count but runs
-          // on the matrix pipeline and stalls behind every MFMA in flight on the SIMD.
-          lsum += e0 + e1;
+      auto raise_max = [&]() {
+        float mx = sacc[0][0];
+#pragma unroll
+        for (int mt = 0; mt < kMT; ++mt)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) mx = fmaxf(mx, sacc[mt][r]);
+        mx = pair_max(mx);
+        const float m_new = (mx * p.c > m_run * p.c + kLazy || m_run == -INFINITY) ? mx : m_run;
+        // A row that has seen no allowed key yet has m_new == -inf: subtract 0 instead, so
+        // that its probabilities are exp2(-inf) = 0 and no inf - inf appears.
+        const float m_sub = (m_new == -INFINITY) ? 0.f : m_new;
+        const float alpha = __builtin_amdgcn_exp2f((m_run - m_sub) * p.c);
+        mc_run = m_sub * p.c;
+        l_run *= alpha;   // per-lane partial sum; the two halves are added at the end
+        m_run = m_new;
+        if (__any(alpha != 1.0f)) {
+#pragma unroll
+          for (int dt = 0; dt < 2; ++dt)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) oacc[dt][r] *= alpha;
         }
-      l_run = l_run * alpha + lsum;   // per-lane partial sum; the two halves are added at the end
-      m_run = m_new;
-      if (__any(alpha != 1.0f)) {
-  #pragma unroll
-        for (int dt = 0; dt < 2; ++dt)
-  #pragma unroll
-          for (int r = 0; r < 16; ++r) oacc[dt][r] *= alpha;
-      }
+        warm = !__any(m_run == -INFINITY);
+      };
+      half8_t pf[kMT][2];   // [key sub-tile][half]: B operand of O^T = V^T . P^T
+      auto probabilities = [&]() -> float {
+        half2_t part[4];   // four interleaved partial sums of at most 8 values each
+#pragma unroll
+        for (int mt = 0; mt < kMT; ++mt)
+#pragma unroll
+          for (int r = 0; r < 16; r += 2) {
+            const float e0 = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[mt][r], p.c, -mc_run));
+            const float e1 = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[mt][r + 1], p.c, -mc_run));
+            const half2_t e2 = {(half_t)e0, (half_t)e1};
+            pf[mt][r >> 3][r & 7] = e2[0];
+            pf[mt][r >> 3][(r & 7) + 1] = e2[1];
+            // Row sum with packed fp16 adds on the values the second product uses, folded to fp32
+            // once per tile (v_dot2c_f32_f16 would do it in one instruction per pair but runs on
+            // the matrix pipeline and stalls behind every MFMA in flight on the SIMD).
+            const int i = (r >> 1) & 3;
+            part[i] = (mt == 0 && r < 8) ? e2 : part[i] + e2;
+          }
+        const half2_t tot = (part[0] + part[1]) + (part[2] + part[3]);
+        return (float)tot[0] + (float)tot[1];
+      };
+      raise_max();
+      l_run += probabilities();
 
       // ---- O^T += V^T . P^T
   #pragma unroll
@@ -858,6 +953,27 @@ __global__ __launch_bounds__(128 * ROWS * KS, 4) void block_attn_fwd_kernel(cons
   attn_group<KIND, ROWS, KS>(p, bh, pair, pre, k_lds0, k_lds1, v_lds0, v_lds1);
 }
 
+// Two query blocks per workgroup with the software-pipelined main loop (rings of three K and
+// three V tiles: 48 KB of LDS).
+template <int KIND>
+__global__ __launch_bounds__(256, 3) void block_attn_pipe_kernel(const AttnParams p) {
+  STOF_ATTN_LDS_TILES;
+  __shared__ __attribute__((aligned(1024))) unsigned char k_lds2[kTile];
+  __shared__ __attribute__((aligned(1024))) unsigned char v_lds2[kTile];
+  int bh, pair;
+  RowPtrs<2> pre;
+  pre.valid = false;
+  if (p.balance) {
+    balanced_group<KIND, 2>(p, bh, pair, pre);
+  } else {
+    const int vid = xcd_contiguous_id(p);
+    if (vid >= p.total) return;
+    bh = vid / p.nP;
+    pair = zigzag(vid - bh * p.nP, bh, p.nP);
+  }
+  attn_group<KIND, 2, 1, true>(p, bh, pair, pre, k_lds0, k_lds1, v_lds0, v_lds1, k_lds2, v_lds2);
+}
+
 // dst[r*(cols/64)+w] bit t = pred(src[r*ld + 64w + t]).
 // Vector form: a lane loads 8 elements (16 B) and forms one byte of the word; the 8 lanes of a
 // word merge their bytes with three lane exchanges and the first of them stores 8 B.  A
@@ -920,7 +1036,7 @@ __global__ __launch_bounds__(256) void pack_mask_bits_kernel(const half_t* __res
 // of each tile split over two wave pairs is the form for small grids, which are bound by the
 // longest chain of key blocks: the chain runs twice as fast.
 constexpr int kRowsPerGroup = 2;
-enum { kFormAuto = -1, kFormTwoRows = 0, kFormKeySplit = 1 };
+enum { kFormAuto = -1, kFormTwoRows = 0, kFormKeySplit = 1, kFormPipelined = 2 };
 int g_attn_form = kFormAuto;
 
 // Automatic choice: key split when the sequence has at least kKeySplitMinQueryBlocks query
@@ -983,7 +1099,10 @@ void launch_attn(AttnParams& p, int nQ, int64_t bh, int requested_form, hipStrea
     p.total = (int)two_row_groups;
     p.chunk = (p.total + 7) / 8;
     set_balance(p, kBalanceMaxGroupsTwoRows);
-    hipLaunchKernelGGL((block_attn_fwd_kernel<KIND, kRowsPerGroup, 1>), dim3(p.chunk * 8), dim3(128 * kRowsPerGroup), 0, stream, p);
+    if (form == kFormPipelined)
+      hipLaunchKernelGGL((block_attn_pipe_kernel<KIND>), dim3(p.chunk * 8), dim3(256), 0, stream, p);
+    else
+      hipLaunchKernelGGL((block_attn_fwd_kernel<KIND, kRowsPerGroup, 1>), dim3(p.chunk * 8), dim3(128 * kRowsPerGroup), 0, stream, p);
   }
 }
 
@@ -994,7 +1113,7 @@ bool strides_ok(const int64_t s[3]) {
 }  // namespace
 
 extern "C" int stof_attn_set_launch_form(int form) {
-  if (form != kFormAuto && form != kFormTwoRows && form != kFormKeySplit) return STOF_ERR_UNSUPPORTED;
+  if (form < kFormAuto || form > kFormPipelined) return STOF_ERR_UNSUPPORTED;
   g_attn_form = form;
   return STOF_OK;
 }
@@ -1009,7 +1128,7 @@ extern "C" int stof_block_attn_fwd(
     const int64_t v_strides[3], const int64_t out_strides[3],
     int batch_size, int seq_len, int head_num, int head_size,
     int64_t lut_batch_stride, int launch_form, void* stream) {
-  if (launch_form != kFormAuto && launch_form != kFormTwoRows && launch_form != kFormKeySplit) return STOF_ERR_UNSUPPORTED;
+  if (launch_form < kFormAuto || launch_form > kFormPipelined) return STOF_ERR_UNSUPPORTED;
   if (!q || !k || !v || !out || !full_row_ptr || !part_row_ptr || !load_row_ptr ||
       !q_strides || !k_strides || !v_strides || !out_strides)
     return STOF_ERR_NULL_POINTER;
@@ -1043,7 +1162,7 @@ extern "C" int stof_rowwise_attn_fwd(
     const void* q, const void* k, const void* v, void* out,
     int kind, int is_causal, int bandwidth, const uint64_t* mask_bits,
     int batch_size, int seq_len, int head_num, int head_size, int launch_form, void* stream) {
-  if (launch_form != kFormAuto && launch_form != kFormTwoRows && launch_form != kFormKeySplit) return STOF_ERR_UNSUPPORTED;
+  if (launch_form < kFormAuto || launch_form > kFormPipelined) return STOF_ERR_UNSUPPORTED;
   if (!q || !k || !v || !out) return STOF_ERR_NULL_POINTER;
   if (kind != STOF_ROW_FULL && kind != STOF_ROW_SLIDING && kind != STOF_ROW_MASK) return STOF_ERR_UNSUPPORTED;
   if (kind == STOF_ROW_MASK && !mask_bits) return STOF_ERR_NULL_POINTER;

@@ -44,12 +44,12 @@ def _require(cond, msg):
         raise StofError(msg)
 
 
-_LAUNCH_FORMS = {None: -1, "default": -1, "auto": -1, "two_rows": 0, "key_split": 1}
+_LAUNCH_FORMS = {None: -1, "default": -1, "auto": -1, "two_rows": 0, "key_split": 1, "pipelined": 2}
 
 
 def _form(launch_form):
     _require(launch_form in _LAUNCH_FORMS,
-             f"launch form must be one of 'default', 'two_rows', 'key_split', got {launch_form!r}")
+             f"launch form must be one of 'default', 'two_rows', 'key_split', 'pipelined', got {launch_form!r}")
     return _LAUNCH_FORMS[launch_form]
 
 
@@ -61,7 +61,8 @@ def set_attention_launch_form(form="auto"):
     call with ``num_warps`` (src/ops/src/block_attn_mask_cuda.cu:6064-6322); the per-call
     counterpart here is the ``launch_form`` argument of ``block_attn`` and of the row-wise
     operators' functional form.  Results agree within rounding in every form."""
-    _require(form in ("auto", "two_rows", "key_split"), f"launch form must be 'auto', 'two_rows' or 'key_split', got {form!r}")
+    _require(form in ("auto", "two_rows", "key_split", "pipelined"),
+             f"launch form must be 'auto', 'two_rows', 'key_split' or 'pipelined', got {form!r}")
     check(_lib.lib().stof_attn_set_launch_form(_LAUNCH_FORMS[form]), "stof_attn_set_launch_form")
 
 

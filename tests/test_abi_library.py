@@ -60,7 +60,7 @@ def test_block_attn_argument_checks(lib):
     assert call(q=P + 2) == -4           # misaligned pointer
     assert call(qs=_s3(12 * 128 * 64, 128 * 64, 65)) == -4   # stride not a multiple of 8
     assert call(lbs=2) == -6             # per-sample LUT stride too small
-    assert call(form=2) == -3            # launch form
+    assert call(form=3) == -3            # launch form
 
 
 def test_other_entry_points_argument_checks(lib):

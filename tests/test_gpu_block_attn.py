@@ -18,7 +18,7 @@ pytestmark = pytest.mark.gpu
 ATOL, RTOL = 2e-3, 1e-2
 
 
-@pytest.fixture(autouse=True, params=["two_rows", "key_split"])
+@pytest.fixture(autouse=True, params=["two_rows", "key_split", "pipelined"])
 def launch_form(request):
     """Every test of this module runs once per launch form of the kernel."""
     from stof.ops import set_attention_launch_form
@@ -246,6 +246,26 @@ def test_large_logits_no_overflow():
     got = _run(q, k, v, mask)
     assert bool(torch.isfinite(got).all())
     _close(got, _oracle(q, k, v, mask), "large logits")
+
+
+@pytest.mark.parametrize("S", [512, 1024])
+def test_rising_logits_along_the_keys(S):
+    """Scores that grow by far more than the fp16 range of the probabilities from one key block
+    to the next: every tile raises the running max.  (The software-pipelined launch form takes
+    the max as it stands on its fast path and verifies the row sums; here the verification
+    fails and the workgroup repeats its walk on the exact path.)"""
+    B, H = 2, 4
+    g = torch.Generator().manual_seed(11)
+    q = (torch.ones(B, H, S, 64) * 0.5 + 0.05 * torch.randn(B, H, S, 64, generator=g)).half().cuda()
+    ramp = torch.arange(S).float()[None, None, :, None] / S * 12.0           # q.k rises by about 24 per 64 keys
+    k = (ramp * torch.ones(B, H, S, 64) + 0.05 * torch.randn(B, H, S, 64, generator=g)).half().cuda()
+    v = torch.randn(B, H, S, 64, generator=g).half().cuda()
+    mask = torch.ones(S, S, dtype=torch.bool)
+    mask[:, S // 2:S // 2 + 64] = False                                        # one empty key block
+    mask[70:90, :] &= torch.rand(20, S, generator=g) < 0.5                      # and some partial tiles
+    got = _run(q, k, v, mask)
+    assert bool(torch.isfinite(got).all())
+    _close(got, _oracle(q, k, v, mask), "rising logits")
 
 
 def test_error_paths_raise():

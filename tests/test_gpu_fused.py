@@ -104,7 +104,7 @@ def test_fused_op_errors():
 
 # ---- row-wise attention front-ends ---------------------------------------------------------------
 
-@pytest.fixture(params=["two_rows", "key_split"])
+@pytest.fixture(params=["two_rows", "key_split", "pipelined"])
 def launch_form(request):
     from stof.ops import set_attention_launch_form
     set_attention_launch_form(request.param)
