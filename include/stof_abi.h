@@ -22,6 +22,8 @@
  *   stof_rowwise_attn_fwd      launcher_rowwise_attn_{full,sliding,mask}
  *                                                           src/ops/src/rowwise_attn_full.cpp:8-12,
  *                                                           rowwise_attn_sliding.cpp:8-12, rowwise_attn_mask.cpp:8-12
+ *   stof_build_lut,
+ *   stof_lut_additive_blocks   get_sparse_storage            src/util/masks.py:125-184 (the host loop :145-170)
  *   stof_bias_res_ln           batched_bias_layer_norm_fused_kernel
  *                                                           src/triton_template/add_layernorm.py:19-107
  *   stof_gemm_bias_act         the first product + bias + GELU of triton_matmul_batch_kernel
@@ -145,6 +147,43 @@ int stof_rowwise_attn_fwd(
     const void* q, const void* k, const void* v, void* out,
     int kind, int is_causal, int bandwidth, const uint64_t* mask_bits,
     int batch_size, int seq_len, int head_num, int head_size, int launch_form, void* stream);
+
+/*
+ * Block LUT of a dense 0/1 mask, built on the GPU: the classification loop of get_sparse_storage
+ * (src/util/masks.py:145-170) as two launches (classify every tile in one pass over the mask,
+ * then compact).  mask: seq_len x seq_len elements of elem_bytes (2: fp16, 4: fp32) at a row
+ * pitch of ld elements - batch 0 of the reference's [B,S,S] tensor (:147).  A block_m x block_n
+ * tile whose elements are all 1 is FULL, all 0 is absent, anything else PARTIAL (:149-166).
+ * Outputs, all int32 device arrays owned by the caller:
+ *   full/part/load_row_ptr [seq_len/block_m + 1]; full/part/load_col_idx with room for cap_full /
+ *   cap_part / cap_load entries (seq_len/block_m * seq_len/block_n always suffices), ascending
+ *   key-block indices per row, LOAD = FULL and PARTIAL merged;
+ *   part_bitmask [cap_part][64] (optional, 64 x 64 blocks only): bit j of row i of PART slot s =
+ *   key j allowed, the form stof_block_attn_fwd reads;
+ *   counts[4] (optional): {entries in FULL, PART, LOAD; 1 if a capacity was too small (the lists are
+ *   then truncated, the row pointers still exact)}.
+ * workspace: stof_build_lut_workspace_bytes() bytes of device memory, 8-byte aligned, used as
+ * scratch for the duration of the call (one class byte per tile, 512 B of bit rows per tile).
+ * block_m, block_n in {16, 32, 64, 128} dividing seq_len; mask 16-byte aligned, ld * elem_bytes
+ * a multiple of 16.  HBM-bound: seq_len^2 * elem_bytes bytes read once.
+ */
+int64_t stof_build_lut_workspace_bytes(int seq_len, int block_m, int block_n);
+int stof_build_lut(const void* mask, int elem_bytes, int64_t ld, int seq_len, int block_m, int block_n,
+                   int32_t* full_row_ptr, int32_t* full_col_idx,
+                   int32_t* part_row_ptr, int32_t* part_col_idx,
+                   int32_t* load_row_ptr, int32_t* load_col_idx,
+                   uint64_t* part_bitmask, int32_t* counts,
+                   int64_t cap_full, int64_t cap_part, int64_t cap_load,
+                   void* workspace, int64_t workspace_bytes, void* stream);
+
+/*
+ * The reference's additive fp16 blocks for the PART list of a LUT:
+ * part_block_mask[s] = -10000 * (1 - block.half()) (src/util/masks.py:159-166), fp16
+ * [n_part, block_m, block_n], for PART slots 0 .. n_part-1 as stof_build_lut wrote them.
+ */
+int stof_lut_additive_blocks(const void* mask, int elem_bytes, int64_t ld, int seq_len, int block_m, int block_n,
+                             const int32_t* part_row_ptr, const int32_t* part_col_idx, int64_t n_part,
+                             void* part_block_mask, void* stream);
 
 /*
  * y[m,:] = LayerNorm(x[m,:] + bias[:] + residual[m,:]) * gamma + beta     (fp32 statistics)

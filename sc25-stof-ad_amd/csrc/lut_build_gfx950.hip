@@ -1,0 +1,283 @@
+// Dense 0/1 mask -> block LUT on the GPU, for gfx950.
+//
+// Replaces the host loop of get_sparse_storage (src/util/masks.py:145-170: one torch.all per
+// (query block, key block) pair, list appends, host -> device copies) with two launches:
+//
+//  1. classify: one wavefront per block_m x block_n tile reads the tile once with 16-byte loads
+//     and decides with two wave-wide votes whether every element is 1 (FULL), every element is 0
+//     (absent) or neither (PARTIAL); for 64 x 64 tiles it forms, in the same pass, the tile's 64
+//     bit rows (bit j of row i = key j allowed) from the lanes' 16-byte chunks by lane exchanges.
+//     One byte per tile (and 512 B of bit rows per partial tile) go to a scratch buffer.  This
+//     pass moves the whole mask once and is bound by HBM bandwidth.
+//  2. compact: one workgroup per row of tiles counts the FULL / PARTIAL tiles of the rows above
+//     it (the class bytes: a few KB, L2-resident), ranks its own tiles with wave votes, and
+//     writes its slice of the three CSR lists (row pointers, ascending key-block indices) and
+//     the bit rows of its partial tiles into their PART slots.
+//
+// A third kernel writes, on request, the reference's additive fp16 blocks
+// -10000 * (1 - block.half()) (src/util/masks.py:159-166) for the PART list.
+//
+// The scratch buffer is passed in by the caller.
+#include "stof_common.h"
+
+namespace {
+
+enum { kClsEmpty = 0, kClsFull = 1, kClsPart = 2 };
+
+struct LutParams {
+  const void* mask; int64_t ld;           // row pitch in elements
+  int S, bm, bn, nQ, nK;
+  unsigned char* cls; uint64_t* ws_bits;  // scratch: class byte per tile; 64 bit rows per tile (64 x 64 only, else null)
+  int32_t* frp; int32_t* fci; int32_t* prp; int32_t* pci; int32_t* lrp; int32_t* lci;
+  uint64_t* pbits;                        // [cap_part][64] or null
+  int32_t* counts;                        // {n_full, n_part, n_load, overflow} or null
+  int64_t cap_full, cap_part, cap_load;
+};
+
+__device__ __forceinline__ half_t additive_of(half_t x) {
+  // -10000 * (1 - x) in fp16 arithmetic, as the reference forms it (src/util/masks.py:160)
+  return (half_t)-10000.0f * ((half_t)1.0f - x);
+}
+
+// One 16-byte chunk of a tile row: updates the two "every element is ..." votes and returns the
+// chunk's keep bits (bit e = element e allowed, by the rule the bit rows are packed with
+// elsewhere: additive value above -5000).
+template <typename T>
+__device__ __forceinline__ uint32_t chunk_bits(const T* src, bool& not_one, bool& not_zero) {
+  constexpr int E = 16 / (int)sizeof(T);
+  typedef T vec_t __attribute__((ext_vector_type(E)));
+  const vec_t x = *reinterpret_cast<const vec_t*>(src);
+  uint32_t cb = 0;
+#pragma unroll
+  for (int e = 0; e < E; ++e) {
+    const float f = (float)x[e];
+    not_one |= f != 1.0f;
+    not_zero |= f != 0.0f;
+    cb |= (uint32_t)((float)additive_of((half_t)x[e]) > -5000.0f) << e;
+  }
+  return cb;
+}
+
+// T = half_t or float; E elements per 16-byte chunk.  One wavefront per tile.
+template <typename T>
+__global__ __launch_bounds__(256) void lut_classify_kernel(const LutParams p) {
+  constexpr int E = 16 / (int)sizeof(T);
+  const int lane = threadIdx.x & 63;
+  const int64_t tile = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (tile >= (int64_t)p.nQ * p.nK) return;
+  const int r = (int)(tile / p.nK), c = (int)(tile - (int64_t)r * p.nK);
+  const T* base = reinterpret_cast<const T*>(p.mask) + (int64_t)r * p.bm * p.ld + (int64_t)c * p.bn;
+  bool not_one = false, not_zero = false;
+  if (p.ws_bits) {
+    // 64 x 64 tile: CPR lanes hold one row of 64 keys, a pass covers 64 / CPR rows, 64 / E passes
+    constexpr int CPR = 64 / E, PASSES = 64 / E, ROWS = 64 / CPR;
+    const int ch = lane & (CPR - 1), row_in_pass = lane / CPR;
+    uint64_t words[PASSES];   // lanes with chunk 0: the bit row of (pass, row_in_pass)
+#pragma unroll
+    for (int ps = 0; ps < PASSES; ++ps) {
+      const uint32_t cb = chunk_bits<T>(base + (int64_t)(ps * ROWS + row_in_pass) * p.ld + ch * E, not_one, not_zero);
+      const int sh = ch * E;
+      uint32_t lo = sh < 32 ? cb << sh : 0u, hi = sh >= 32 ? cb << (sh - 32) : 0u;
+#pragma unroll
+      for (int m = 1; m < CPR; m <<= 1) {
+        lo |= (uint32_t)__shfl_xor((int)lo, m, 64);
+        hi |= (uint32_t)__shfl_xor((int)hi, m, 64);
+      }
+      words[ps] = ((uint64_t)hi << 32) | lo;
+    }
+    const bool full = __ballot(not_one) == 0ull, empty = __ballot(not_zero) == 0ull;
+    if (lane == 0) p.cls[tile] = (unsigned char)(empty ? kClsEmpty : (full ? kClsFull : kClsPart));
+    if (!full && !empty && ch == 0) {
+#pragma unroll
+      for (int ps = 0; ps < PASSES; ++ps) p.ws_bits[tile * 64 + ps * ROWS + row_in_pass] = words[ps];
+    }
+  } else {
+    const int cpr = p.bn / E;                 // 16-byte chunks per tile row
+    const int total = p.bm * cpr;
+    for (int idx = lane; idx < total; idx += 64) {
+      const int row = idx / cpr, ch = idx - row * cpr;
+      chunk_bits<T>(base + (int64_t)row * p.ld + ch * E, not_one, not_zero);
+    }
+    const bool full = __ballot(not_one) == 0ull, empty = __ballot(not_zero) == 0ull;
+    if (lane == 0) p.cls[tile] = (unsigned char)(empty ? kClsEmpty : (full ? kClsFull : kClsPart));
+  }
+}
+
+__device__ __forceinline__ int block_sum(int v, int* lds) {
+  // sum over the 256 threads of the workgroup; lds: 4 ints
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) lds[threadIdx.x >> 6] = v;
+  __syncthreads();
+  return lds[0] + lds[1] + lds[2] + lds[3];
+}
+
+__global__ __launch_bounds__(256) void lut_compact_kernel(const LutParams p) {
+  __shared__ int red[4];
+  __shared__ int wave_cnt[2][4];
+  __shared__ int part_col[256], part_slot[256];
+  const int r = blockIdx.x;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  // tiles of the rows above: FULL and PARTIAL counts
+  int nf = 0, np = 0;
+  const int64_t above = (int64_t)r * p.nK;
+  for (int64_t i = tid; i < above; i += 256) {
+    const int c = p.cls[i];
+    nf += c == kClsFull; np += c == kClsPart;
+  }
+  int fbase = block_sum(nf, red);
+  int pbase = block_sum(np, red);
+  const unsigned char* row_cls = p.cls + above;
+  for (int c0 = 0; c0 < p.nK; c0 += 256) {
+    const int c = c0 + tid;
+    const int cl = c < p.nK ? row_cls[c] : kClsEmpty;
+    const uint64_t bf = __ballot(cl == kClsFull), bp = __ballot(cl == kClsPart);
+    const uint64_t below = lane == 0 ? 0ull : (~0ull >> (64 - lane));
+    if (lane == 0) { wave_cnt[0][wave] = __builtin_popcountll(bf); wave_cnt[1][wave] = __builtin_popcountll(bp); }
+    __syncthreads();
+    int f_before = 0, p_before = 0, f_all = 0, p_all = 0;
+    for (int w = 0; w < 4; ++w) {
+      if (w < wave) { f_before += wave_cnt[0][w]; p_before += wave_cnt[1][w]; }
+      f_all += wave_cnt[0][w]; p_all += wave_cnt[1][w];
+    }
+    const int rf = fbase + f_before + __builtin_popcountll(bf & below);
+    const int rp = pbase + p_before + __builtin_popcountll(bp & below);
+    part_slot[tid] = -1;
+    if (cl == kClsFull) {
+      if (rf < p.cap_full) p.fci[rf] = c;
+      if (rf + rp < p.cap_load) p.lci[rf + rp] = c;
+    } else if (cl == kClsPart) {
+      if (rp < p.cap_part) { p.pci[rp] = c; part_col[tid] = c; part_slot[tid] = rp; }
+      if (rf + rp < p.cap_load) p.lci[rf + rp] = c;
+    }
+    __syncthreads();
+    // bit rows of this chunk's partial tiles into their PART slots (a wavefront per tile)
+    if (p.pbits && p.ws_bits) {
+      for (int t = wave; t < 256; t += 4) {
+        const int slot = part_slot[t];
+        if (slot >= 0) p.pbits[(int64_t)slot * 64 + lane] = p.ws_bits[(above + part_col[t]) * 64 + lane];
+      }
+    }
+    fbase += f_all; pbase += p_all;
+    __syncthreads();
+  }
+  if (tid == 0) {
+    if (r == 0) { p.frp[0] = 0; p.prp[0] = 0; p.lrp[0] = 0; }
+    p.frp[r + 1] = fbase; p.prp[r + 1] = pbase; p.lrp[r + 1] = fbase + pbase;
+    if (r == p.nQ - 1 && p.counts) {
+      p.counts[0] = fbase; p.counts[1] = pbase; p.counts[2] = fbase + pbase;
+      p.counts[3] = (fbase > p.cap_full || pbase > p.cap_part || fbase + pbase > p.cap_load) ? 1 : 0;
+    }
+  }
+}
+
+// out[s] = -10000 * (1 - block.half()) for PART slot s: (row from the PART row pointers, column pci[s]).
+template <typename T>
+__global__ __launch_bounds__(256) void lut_additive_blocks_kernel(const void* mask, int64_t ld, int bm, int bn, int nQ,
+                                                                  const int32_t* __restrict__ prp, const int32_t* __restrict__ pci,
+                                                                  half_t* __restrict__ out) {
+  __shared__ int s_row;
+  const int s = blockIdx.x;
+  if (threadIdx.x == 0) {
+    int lo = 0, hi = nQ;           // last r with prp[r] <= s
+    while (hi - lo > 1) { const int mid = (lo + hi) >> 1; if (prp[mid] <= s) lo = mid; else hi = mid; }
+    s_row = lo;
+  }
+  __syncthreads();
+  const int r = s_row, c = pci[s];
+  const T* base = reinterpret_cast<const T*>(mask) + (int64_t)r * bm * ld + (int64_t)c * bn;
+  half_t* o = out + (int64_t)s * bm * bn;
+  for (int i = threadIdx.x; i < bm * bn; i += 256) {
+    const int row = i / bn, col = i - row * bn;
+    o[i] = additive_of((half_t)base[(int64_t)row * ld + col]);
+  }
+}
+
+bool block_ok(int b) { return b == 16 || b == 32 || b == 64 || b == 128; }
+
+int check_common(const void* mask, int elem_bytes, int64_t ld, int seq_len, int block_m, int block_n) {
+  if (!mask) return STOF_ERR_NULL_POINTER;
+  if (elem_bytes != 2 && elem_bytes != 4) return STOF_ERR_UNSUPPORTED;
+  if (!block_ok(block_m) || !block_ok(block_n)) return STOF_ERR_UNSUPPORTED;
+  if (seq_len <= 0 || seq_len % block_m != 0 || seq_len % block_n != 0 || ld < seq_len) return STOF_ERR_BAD_SHAPE;
+  if (!stof_aligned16(mask) || (ld * elem_bytes) % 16 != 0) return STOF_ERR_MISALIGNED;
+  return STOF_OK;
+}
+
+int build(const void* mask, int elem_bytes, int64_t ld, int seq_len, int block_m, int block_n,
+          int32_t* frp, int32_t* fci, int32_t* prp, int32_t* pci, int32_t* lrp, int32_t* lci,
+          uint64_t* part_bitmask, int32_t* counts, int64_t cap_full, int64_t cap_part, int64_t cap_load,
+          unsigned char* cls, uint64_t* ws_bits, hipStream_t stream) {
+  LutParams p;
+  p.mask = mask; p.ld = ld; p.S = seq_len; p.bm = block_m; p.bn = block_n;
+  p.nQ = seq_len / block_m; p.nK = seq_len / block_n;
+  p.cls = cls; p.ws_bits = (block_m == 64 && block_n == 64 && part_bitmask) ? ws_bits : nullptr;
+  p.frp = frp; p.fci = fci; p.prp = prp; p.pci = pci; p.lrp = lrp; p.lci = lci;
+  p.pbits = p.ws_bits ? part_bitmask : nullptr; p.counts = counts;
+  p.cap_full = cap_full; p.cap_part = cap_part; p.cap_load = cap_load;
+  const int64_t tiles = (int64_t)p.nQ * p.nK;
+  const dim3 grid1((unsigned)((tiles + 3) / 4)), block(256);
+  if (elem_bytes == 2) hipLaunchKernelGGL(lut_classify_kernel<half_t>, grid1, block, 0, stream, p);
+  else hipLaunchKernelGGL(lut_classify_kernel<float>, grid1, block, 0, stream, p);
+  hipLaunchKernelGGL(lut_compact_kernel, dim3((unsigned)p.nQ), block, 0, stream, p);
+  return stof_check_launch();
+}
+
+int check_outputs(const int32_t* frp, const int32_t* fci, const int32_t* prp, const int32_t* pci,
+                  const int32_t* lrp, const int32_t* lci, const uint64_t* part_bitmask, int block_m, int block_n,
+                  int64_t cap_full, int64_t cap_part, int64_t cap_load) {
+  if (!frp || !prp || !lrp) return STOF_ERR_NULL_POINTER;
+  if (cap_full < 0 || cap_part < 0 || cap_load < 0) return STOF_ERR_BAD_SHAPE;
+  if ((cap_full > 0 && !fci) || (cap_part > 0 && !pci) || (cap_load > 0 && !lci)) return STOF_ERR_NULL_POINTER;
+  if (part_bitmask && (block_m != 64 || block_n != 64)) return STOF_ERR_UNSUPPORTED;
+  return STOF_OK;
+}
+
+}  // namespace
+
+extern "C" int64_t stof_build_lut_workspace_bytes(int seq_len, int block_m, int block_n) {
+  if (seq_len <= 0 || !block_ok(block_m) || !block_ok(block_n) || seq_len % block_m || seq_len % block_n) return STOF_ERR_BAD_SHAPE;
+  const int64_t tiles = (int64_t)(seq_len / block_m) * (seq_len / block_n);
+  const int64_t cls = (tiles + 255) / 256 * 256;
+  return cls + ((block_m == 64 && block_n == 64) ? tiles * 64 * 8 : 0);
+}
+
+extern "C" int stof_build_lut(const void* mask, int elem_bytes, int64_t ld, int seq_len, int block_m, int block_n,
+                              int32_t* full_row_ptr, int32_t* full_col_idx,
+                              int32_t* part_row_ptr, int32_t* part_col_idx,
+                              int32_t* load_row_ptr, int32_t* load_col_idx,
+                              uint64_t* part_bitmask, int32_t* counts,
+                              int64_t cap_full, int64_t cap_part, int64_t cap_load,
+                              void* workspace, int64_t workspace_bytes, void* stream) {
+  int rc = check_common(mask, elem_bytes, ld, seq_len, block_m, block_n);
+  if (rc != STOF_OK) return rc;
+  rc = check_outputs(full_row_ptr, full_col_idx, part_row_ptr, part_col_idx, load_row_ptr, load_col_idx,
+                     part_bitmask, block_m, block_n, cap_full, cap_part, cap_load);
+  if (rc != STOF_OK) return rc;
+  if (!workspace) return STOF_ERR_NULL_POINTER;
+  if (workspace_bytes < stof_build_lut_workspace_bytes(seq_len, block_m, block_n)) return STOF_ERR_BAD_SHAPE;
+  if ((reinterpret_cast<uintptr_t>(workspace) & 7) != 0) return STOF_ERR_MISALIGNED;
+  const int64_t tiles = (int64_t)(seq_len / block_m) * (seq_len / block_n);
+  unsigned char* cls = static_cast<unsigned char*>(workspace);
+  uint64_t* bits = reinterpret_cast<uint64_t*>(cls + (tiles + 255) / 256 * 256);
+  return build(mask, elem_bytes, ld, seq_len, block_m, block_n, full_row_ptr, full_col_idx, part_row_ptr, part_col_idx,
+               load_row_ptr, load_col_idx, part_bitmask, counts, cap_full, cap_part, cap_load, cls, bits, (hipStream_t)stream);
+}
+
+extern "C" int stof_lut_additive_blocks(const void* mask, int elem_bytes, int64_t ld, int seq_len, int block_m, int block_n,
+                                        const int32_t* part_row_ptr, const int32_t* part_col_idx, int64_t n_part,
+                                        void* part_block_mask, void* stream) {
+  int rc = check_common(mask, elem_bytes, ld, seq_len, block_m, block_n);
+  if (rc != STOF_OK) return rc;
+  if (n_part < 0 || n_part > ((int64_t)1 << 30)) return STOF_ERR_BAD_SHAPE;
+  if (n_part == 0) return STOF_OK;
+  if (!part_row_ptr || !part_col_idx || !part_block_mask) return STOF_ERR_NULL_POINTER;
+  const int nQ = seq_len / block_m;
+  if (elem_bytes == 2)
+    hipLaunchKernelGGL(lut_additive_blocks_kernel<half_t>, dim3((unsigned)n_part), dim3(256), 0, (hipStream_t)stream,
+                       mask, ld, block_m, block_n, nQ, part_row_ptr, part_col_idx, (half_t*)part_block_mask);
+  else
+    hipLaunchKernelGGL(lut_additive_blocks_kernel<float>, dim3((unsigned)n_part), dim3(256), 0, (hipStream_t)stream,
+                       mask, ld, block_m, block_n, nQ, part_row_ptr, part_col_idx, (half_t*)part_block_mask);
+  return stof_check_launch();
+}

@@ -131,6 +131,64 @@ def _csr(flag):
     return row_ptr.to(torch.int32), col_idx.to(torch.int32)
 
 
+_DEVICE_BLOCKS = (16, 32, 64, 128)
+
+
+def _device_path(Mask, bm, bn):
+    """The GPU kernels take fp16 / fp32 masks with 16-byte aligned rows and block sizes of 16..128."""
+    n = Mask.shape[-1]
+    return (Mask.is_cuda and Mask.dtype in (torch.float16, torch.float32) and bm in _DEVICE_BLOCKS and bn in _DEVICE_BLOCKS
+            and Mask.dim() == 3 and Mask.shape[-2] == n and n % bm == 0 and n % bn == 0 and (n * Mask.element_size()) % 16 == 0)
+
+
+def _build_on_device(m2d, bm, bn, want_bits):
+    """One sample's mask [S,S] on the GPU -> (row pointers x3, column lists x3 at full capacity,
+    bit rows or None, counts tensor).  No synchronisation: everything stays on the device."""
+    from . import _lib
+    from .ops import _stream
+    if m2d.stride(1) != 1 or (m2d.stride(0) * m2d.element_size()) % 16 or m2d.data_ptr() % 16:
+        m2d = m2d.contiguous()
+    n = m2d.shape[-1]
+    nq, nk = n // bm, n // bn
+    tiles = nq * nk
+    dev = m2d.device
+    i32 = lambda k: torch.empty(k, dtype=torch.int32, device=dev)
+    frp, prp, lrp = i32(nq + 1), i32(nq + 1), i32(nq + 1)
+    fci, pci, lci = i32(tiles), i32(tiles), i32(tiles)
+    counts = i32(4)
+    bits = torch.empty((tiles, 64), dtype=torch.int64, device=dev) if (want_bits and bm == 64 and bn == 64) else None
+    lib = _lib.lib()
+    ws = torch.empty(lib.stof_build_lut_workspace_bytes(n, bm, bn), dtype=torch.uint8, device=dev)
+    _lib.check(lib.stof_build_lut(m2d.data_ptr(), m2d.element_size(), m2d.stride(0), n, bm, bn,
+                                  frp.data_ptr(), fci.data_ptr(), prp.data_ptr(), pci.data_ptr(), lrp.data_ptr(), lci.data_ptr(),
+                                  bits.data_ptr() if bits is not None else None, counts.data_ptr(),
+                                  tiles, tiles, tiles, ws.data_ptr(), ws.numel(), _stream(dev)), "stof_build_lut")
+    return m2d, frp, fci, prp, pci, lrp, lci, bits, counts
+
+
+def _get_sparse_storage_device(m2d, bm, bn):
+    """The seven LUT tensors of one sample, exactly shaped, built by the GPU kernels (one
+    device -> host read of the three list lengths)."""
+    from . import _lib
+    from ._cache import BITS_ATTR, content_key
+    from .ops import _stream
+    m2d, frp, fci, prp, pci, lrp, lci, bits, counts = _build_on_device(m2d, bm, bn, want_bits=True)
+    n_full, n_part, n_load, overflow = counts.tolist()
+    assert not overflow
+    n = m2d.shape[-1]
+    fci, pci, lci = fci[:n_full], pci[:n_part], lci[:n_load]
+    if n_part == 0:
+        pbm = torch.ones(1, bm, bn, dtype=torch.float16, device=m2d.device)
+    else:
+        pbm = torch.empty(n_part, bm, bn, dtype=torch.float16, device=m2d.device)
+        _lib.check(_lib.lib().stof_lut_additive_blocks(m2d.data_ptr(), m2d.element_size(), m2d.stride(0), n, bm, bn,
+                                                       prp.data_ptr(), pci.data_ptr(), n_part, pbm.data_ptr(),
+                                                       _stream(m2d.device)), "stof_lut_additive_blocks")
+        if bits is not None:   # the attention operator finds the bit rows of these blocks already packed
+            setattr(pbm, BITS_ATTR, (content_key(pbm), bits[:n_part]))
+    return frp, fci, prp, pci, pbm, lrp, lci
+
+
 def get_sparse_storage(Mask, block_size_m, block_size_n):
     """src/util/masks.py:125-184.  Mask [B,S,S] of 0/1 (any float dtype, any device).
 
@@ -139,9 +197,15 @@ def get_sparse_storage(Mask, block_size_m, block_size_n):
     percentage of non-zeros of the WHOLE tensor over S*S (:137), the LUT describes
     batch 0 only (:147), partial tiles carry ``-10000 * (1 - block.half())`` (:160)
     and an LUT without partial tiles carries one dummy block of ones (:179-180).
+
+    An fp16 / fp32 mask on the GPU is compiled by the library's kernels (one pass over the
+    mask, stof_build_lut); anything else by the tensor operations below on the mask's device.
+    Both give the same tensors bit for bit.
     """
     n = Mask.shape[-1]
     nnz = torch.count_nonzero(Mask) / (n * n) * 100
+    if _device_path(Mask, block_size_m, block_size_n):
+        return (nnz,) + _get_sparse_storage_device(Mask[0], block_size_m, block_size_n)
     blocks, full, part = _classify(Mask[0], block_size_m, block_size_n)
     full_row_ptr, full_col_idx = _csr(full)
     part_row_ptr, part_col_idx = _csr(part)
@@ -152,6 +216,23 @@ def get_sparse_storage(Mask, block_size_m, block_size_n):
         part_block_mask = (NEG_MASK * (1.0 - blocks[part].to(torch.float16))).contiguous()
     return (nnz, full_row_ptr, full_col_idx, part_row_ptr, part_col_idx,
             part_block_mask, load_row_ptr, load_col_idx)
+
+
+def build_lut_device(Mask, block_size_m=64, block_size_n=64):
+    """Mask [B,S,S] (fp16 / fp32, on the GPU) -> LUT of batch 0 without any device -> host
+    synchronisation, for use with ``stof.ops.block_attn``: the same seven tensors as
+    ``get_sparse_storage`` (without ``nnz``), except that the three column lists keep their
+    full capacity (entries beyond the last row pointer are unused) and ``part_block_mask`` is a
+    one-block placeholder that carries the partial tiles' packed bit rows, which is what the
+    attention kernel reads.  64 x 64 blocks only."""
+    from ._cache import BITS_ATTR, LUT_OK_ATTR, content_key
+    if not _device_path(Mask, block_size_m, block_size_n) or (block_size_m, block_size_n) != (64, 64):
+        raise ValueError("build_lut_device needs an fp16 / fp32 [B,S,S] mask on the GPU and 64 x 64 blocks")
+    _, frp, fci, prp, pci, lrp, lci, bits, _ = _build_on_device(Mask[0], 64, 64, want_bits=True)
+    pbm = torch.ones(1, 64, 64, dtype=torch.float16, device=Mask.device)
+    setattr(pbm, BITS_ATTR, (content_key(pbm), bits))
+    setattr(lci, LUT_OK_ATTR, tuple(content_key(t) for t in (lci, pci, lrp, prp)))   # in order by construction
+    return frp, fci, prp, pci, pbm, lrp, lci
 
 
 def get_sparse_storage_batched(Mask, block_size_m, block_size_n):
@@ -165,14 +246,19 @@ def get_sparse_storage_batched(Mask, block_size_m, block_size_n):
     nnz = torch.count_nonzero(Mask) / (n * n) * 100
     outs = {k: [] for k in ("frp", "fci", "prp", "pci", "pbm", "lrp", "lci")}
     fo = po = lo = 0
+    on_device = _device_path(Mask, block_size_m, block_size_n)
     for b in range(B):
-        blocks, full, part = _classify(Mask[b], block_size_m, block_size_n)
-        frp, fci = _csr(full); prp, pci = _csr(part); lrp, lci = _csr(full | part)
+        if on_device:
+            frp, fci, prp, pci, pbm_b, lrp, lci = _get_sparse_storage_device(Mask[b], block_size_m, block_size_n)
+        else:
+            blocks, full, part = _classify(Mask[b], block_size_m, block_size_n)
+            frp, fci = _csr(full); prp, pci = _csr(part); lrp, lci = _csr(full | part)
+            pbm_b = (NEG_MASK * (1.0 - blocks[part].to(torch.float16))) if pci.numel() else None
         outs["frp"].append(frp + fo); outs["fci"].append(fci)
         outs["prp"].append(prp + po); outs["pci"].append(pci)
         outs["lrp"].append(lrp + lo); outs["lci"].append(lci)
         if pci.numel():
-            outs["pbm"].append((NEG_MASK * (1.0 - blocks[part].to(torch.float16))))
+            outs["pbm"].append(pbm_b)
         fo += fci.numel(); po += pci.numel(); lo += lci.numel()
     if po == 0:
         pbm = torch.ones(1, block_size_m, block_size_n, dtype=torch.float16, device=Mask.device)

@@ -17,12 +17,11 @@ import torch
 from torch.autograd import Function
 
 from . import _lib
+from ._cache import BITS_ATTR as _BITS_ATTR, LUT_OK_ATTR as _LUT_OK_ATTR, content_key as _content_key
 from ._lib import StofError, check, strides3
 
 __all__ = ["block_attn", "rowwise_attn", "block_attn_mask_op", "rowwise_attn_full_op", "rowwise_attn_sliding_op",
            "rowwise_attn_mask_op", "pack_mask_bits", "set_attention_launch_form", "StofError"]
-
-_BITS_ATTR = "_stof_packed_bits"
 
 
 _raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
@@ -81,13 +80,6 @@ def pack_mask_bits(src, additive):
     return dst
 
 
-def _content_key(t):
-    """What the per-tensor caches are keyed on: the storage address and PyTorch's in-place
-    version counter.  A write that goes around PyTorch (another library through ``data_ptr``,
-    DLPack, numpy-shared memory) changes neither: such callers pass ``revalidate=True``."""
-    return (t.data_ptr(), t._version)
-
-
 def _drop_caches(lut):
     for t in lut:
         for attr in (_BITS_ATTR, _LUT_OK_ATTR, _LUT64_ATTR, _LUT_READY_ATTR):
@@ -117,9 +109,6 @@ def _packed_partial_bits(part_block_mask):
     except AttributeError:
         pass
     return bits
-
-
-_LUT_OK_ATTR = "_stof_lut_checked"
 
 
 def _check_lut_order(lrp, lci, prp, pci, n_cols):

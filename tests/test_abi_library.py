@@ -89,3 +89,22 @@ def test_missing_library_fails_loudly(monkeypatch, tmp_path):
     monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "nope.so"))
     with pytest.raises(_lib.StofError):
         _lib.lib()
+
+
+def test_lut_build_argument_checks(lib):
+    P = 4096
+    i = lambda **kw: lib.stof_build_lut(kw.get("mask", P), kw.get("eb", 2), kw.get("ld", 256), kw.get("S", 256), kw.get("bm", 64), kw.get("bn", 64),
+                                        P, P, P, P, P, P, kw.get("bits", None), None, 16, 16, 16, kw.get("ws", P), kw.get("wsb", 1 << 20), None)
+    assert i(mask=None) == -1
+    assert i(eb=1) == -3                       # element size
+    assert i(bm=48) == -3                      # block size
+    assert i(S=200) == -2                      # not divisible
+    assert i(ld=128) == -2                     # pitch below S
+    assert i(ld=257) == -4                     # rows not 16-byte aligned
+    assert i(bits=P, bm=32, bn=32) == -3       # bit rows exist for 64 x 64 only
+    assert i(ws=None) == -1
+    assert i(wsb=100) == -2                    # workspace too small
+    assert lib.stof_build_lut_workspace_bytes(4096, 64, 64) == 4096 + 4096 * 512
+    assert lib.stof_build_lut_workspace_bytes(256, 16, 16) == 256
+    assert lib.stof_lut_additive_blocks(P, 2, 256, 256, 64, 64, None, None, 0, None, None) == 0
+    assert lib.stof_lut_additive_blocks(P, 2, 256, 256, 64, 64, None, None, 3, None, None) == -1

@@ -1,0 +1,123 @@
+"""The mask -> block LUT kernels (stof_build_lut, stof_lut_additive_blocks) on the GPU, bit for
+bit against the CPU oracle's restatement of get_sparse_storage (src/util/masks.py:125-184)."""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import attention as oa
+from oracle import masks as om
+from stof import _lib, configs, masks as pm
+from stof._cache import BITS_ATTR
+from stof.ops import block_attn
+
+pytestmark = pytest.mark.gpu
+
+
+def _same_lut(got, want, bm, bn, what):
+    """got: the product's 8-tuple (device tensors); want: the oracle's (numpy)."""
+    names = ["nnz", "full_row_ptr", "full_col_idx", "part_row_ptr", "part_col_idx", "part_block_mask", "load_row_ptr", "load_col_idx"]
+    assert abs(float(got[0]) - float(want[0])) < 1e-3, f"{what}: nnz"
+    for i in (1, 2, 3, 4, 6, 7):
+        g = got[i].cpu().numpy()
+        assert g.dtype == np.int32 and g.shape == want[i].shape and np.array_equal(g, want[i]), f"{what}: {names[i]} differs"
+    g = got[5].cpu().numpy()
+    assert g.dtype == np.float16 and g.shape == want[5].shape, f"{what}: part_block_mask shape {g.shape} vs {want[5].shape}"
+    assert np.array_equal(g.view(np.uint16), want[5].view(np.uint16)), f"{what}: part_block_mask bits differ"
+
+
+def _bit_rows(additive):
+    """[n,64,64] additive fp16 blocks -> uint64 [n,64] bit rows (bit j = key j allowed)."""
+    keep = (additive.astype(np.float32) > -5000).astype(np.uint64)
+    return (keep << np.arange(64, dtype=np.uint64)[None, None, :]).sum(-1)
+
+
+@pytest.mark.parametrize("name", ["C1", "C2", "C4", "C5"])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
+def test_baseline_masks_bit_identical_on_device(name, dtype):
+    s = {"C1": 512, "C2": 1024, "C4": 4096, "C5": 2048}[name]
+    mask = configs.ATTN_MASKS[name](s)
+    dev_mask = mask.to(dtype)[None].cuda()
+    got = pm.get_sparse_storage(dev_mask, 64, 64)
+    want = om.get_sparse_storage(mask.float()[None].numpy(), 64, 64)
+    _same_lut(got, want, 64, 64, f"{name} {dtype}")
+    full, part = configs.BLOCK_COUNTS[name]
+    assert int(got[1][-1]) == full and int(got[3][-1]) == part
+    bits = getattr(got[5], BITS_ATTR, None)
+    if part:
+        assert bits is not None, "the kernel's bit rows were not handed to the attention operator"
+        assert np.array_equal(bits[1].cpu().numpy().view(np.uint64), _bit_rows(want[5])), f"{name}: bit rows differ"
+
+
+@pytest.mark.parametrize("bm,bn", [(64, 64), (32, 32), (16, 64), (128, 64), (64, 128), (16, 16), (128, 128)])
+@pytest.mark.parametrize("seed", [0, 1])
+def test_random_masks_and_block_sizes(bm, bn, seed):
+    """Random tile classes (empty / full / sparse partial / dense partial / a single 0 or 1 in a
+    corner), rows of one class only, for every supported block shape."""
+    g = torch.Generator().manual_seed(100 + seed)
+    S = 768 if max(bm, bn) > 64 else 384
+    nq, nk = S // bm, S // bn
+    kind = torch.randint(0, 5, (nq, nk), generator=g)
+    kind[0, :] = 0; kind[1 % nq, :] = 1                     # an empty row of tiles, a full one
+    mask = torch.zeros(S, S)
+    for r in range(nq):
+        for c in range(nk):
+            t = mask[r * bm:(r + 1) * bm, c * bn:(c + 1) * bn]
+            k = int(kind[r, c])
+            if k == 1: t.fill_(1)
+            elif k == 2: t.copy_((torch.rand(bm, bn, generator=g) < 0.1).float())
+            elif k == 3: t.fill_(1); t[bm - 1, bn - 1] = 0
+            elif k == 4: t[0, 0] = 1
+    for dtype in (torch.float16, torch.float32):
+        got = pm.get_sparse_storage(mask.to(dtype)[None].cuda(), bm, bn)
+        want = om.get_sparse_storage(mask[None].numpy(), bm, bn)
+        _same_lut(got, want, bm, bn, f"random {bm}x{bn} seed {seed} {dtype}")
+
+
+def test_batch_zero_only_strided_rows_and_batched():
+    """The LUT describes batch 0 (src/util/masks.py:147); rows at a pitch above S; per-sample LUTs."""
+    g = torch.Generator().manual_seed(7)
+    B, S = 3, 256
+    mask = (torch.rand(B, S, S, generator=g) < 0.5).float()
+    mask[:, :64, :128] = 1; mask[:, 64:128, :64] = 0
+    got = pm.get_sparse_storage(mask.half().cuda(), 64, 64)
+    _same_lut(got, om.get_sparse_storage(mask.numpy(), 64, 64), 64, 64, "batch 0")
+    wide = torch.zeros(B, S, S + 64).half().cuda()
+    wide[:, :, :S] = mask.half().cuda()
+    got = pm.get_sparse_storage(wide[:, :, :S], 64, 64)               # a view: row pitch S + 64
+    _same_lut(got, om.get_sparse_storage(mask.numpy(), 64, 64), 64, 64, "strided rows")
+    gb = pm.get_sparse_storage_batched(mask.half().cuda(), 64, 64)
+    cb = pm.get_sparse_storage_batched(mask, 64, 64)                  # the tensor-op path on the CPU
+    for a, b in zip(gb[1:], cb[1:]):
+        assert torch.equal(a.cpu(), b), "batched LUT differs between the GPU kernels and the tensor-op path"
+
+
+def test_device_lut_feeds_attention_without_a_host_round_trip():
+    cfg = configs.AttnConfig("t", 2, 4, 2048)
+    mask = configs.mask_c5(cfg.seq)
+    q, k, v = configs.qkv(cfg, seed=3, device="cuda")
+    lut = pm.build_lut_device(mask.half()[None].cuda())
+    got = block_attn(q, k, v, lut)
+    want = oa.dense_masked_attention(q.cpu().float(), k.cpu().float(), v.cpu().float(), mask)
+    err = (got.float().cpu() - want).abs()
+    assert bool((err <= 2e-3 + 1e-2 * want.abs()).all()), f"max abs err {float(err.max()):.3e}"
+    assert torch.equal(got, block_attn(q, k, v, pm.get_sparse_storage(mask.half()[None].cuda(), 64, 64)[1:]))
+
+
+def test_capacity_too_small_is_reported_not_overrun():
+    lib = _lib.lib()
+    S = 256
+    mask = torch.ones(S, S, dtype=torch.float16, device="cuda")
+    mask[0, 0] = 0                                                     # 15 full tiles + 1 partial
+    i32 = lambda n: torch.full((n,), -7, dtype=torch.int32, device="cuda")
+    frp, prp, lrp = i32(5), i32(5), i32(5)
+    fci, pci, lci = i32(16), i32(16), i32(16)
+    counts = i32(4)
+    ws = torch.empty(lib.stof_build_lut_workspace_bytes(S, 64, 64), dtype=torch.uint8, device="cuda")
+    rc = lib.stof_build_lut(mask.data_ptr(), 2, S, S, 64, 64, frp.data_ptr(), fci.data_ptr(), prp.data_ptr(), pci.data_ptr(),
+                            lrp.data_ptr(), lci.data_ptr(), None, counts.data_ptr(), 4, 16, 16, ws.data_ptr(), ws.numel(), None)
+    assert rc == 0
+    torch.cuda.synchronize()
+    assert counts.tolist() == [15, 1, 16, 1]                           # full list truncated: flagged
+    assert fci[4:].eq(-7).all() and lrp.tolist() == [0, 4, 8, 12, 16]  # nothing written past the capacity
