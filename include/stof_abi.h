@@ -51,7 +51,8 @@ enum {
   STOF_ERR_UNSUPPORTED = -3,    /* head size / block size / activation not implemented */
   STOF_ERR_MISALIGNED = -4,     /* pointer or stride breaks the 16-byte vector-access rule */
   STOF_ERR_LAUNCH = -5,         /* hipGetLastError() reported a failure after the launch */
-  STOF_ERR_BAD_LUT = -6         /* inconsistent LUT description (host-visible part) */
+  STOF_ERR_BAD_LUT = -6,        /* inconsistent LUT description (host-visible part) */
+  STOF_ERR_TOO_LARGE = -7       /* the problem exceeds the fixed scratch of an entry point that allocates nothing */
 };
 
 /* activation selector of stof_gemm_bias_act */
@@ -175,6 +176,26 @@ int stof_build_lut(const void* mask, int elem_bytes, int64_t ld, int seq_len, in
                    uint64_t* part_bitmask, int32_t* counts,
                    int64_t cap_full, int64_t cap_part, int64_t cap_load,
                    void* workspace, int64_t workspace_bytes, void* stream);
+
+/*
+ * stof_build_lut without the workspace argument, for callers that cannot allocate device memory
+ * (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has
+ * no counterpart in the reference.  The scratch is a fixed array in device memory that the
+ * library holds per GPU until the process ends (8.02 MB: class bytes and bit rows for up to
+ * stof_build_lut_static_max_tiles() = 16384 tiles, i.e. seq_len 8192 at 64 x 64 blocks); a
+ * larger problem returns STOF_ERR_TOO_LARGE.  No hipMalloc / hipFree or allocating routine is
+ * called.  Every call on a GPU uses that GPU's one array: calls that overlap on one GPU (two
+ * streams, two host threads) race - serialise them, or give the overlapping ones a workspace
+ * through stof_build_lut.  Nothing in the array has to start at zero (every byte a call reads it
+ * has written itself).  Arguments and results are those of stof_build_lut.
+ */
+int64_t stof_build_lut_static_max_tiles(void);
+int stof_build_lut_static(const void* mask, int elem_bytes, int64_t ld, int seq_len, int block_m, int block_n,
+                          int32_t* full_row_ptr, int32_t* full_col_idx,
+                          int32_t* part_row_ptr, int32_t* part_col_idx,
+                          int32_t* load_row_ptr, int32_t* load_col_idx,
+                          uint64_t* part_bitmask, int32_t* counts,
+                          int64_t cap_full, int64_t cap_part, int64_t cap_load, void* stream);
 
 /*
  * The reference's additive fp16 blocks for the PART list of a LUT:

@@ -12,6 +12,7 @@ extern "C" const char* stof_status_string(int status) {
     case STOF_ERR_MISALIGNED: return "pointer or stride is not aligned for 16-byte vector access";
     case STOF_ERR_LAUNCH: return "kernel launch failed";
     case STOF_ERR_BAD_LUT: return "inconsistent block LUT description";
+    case STOF_ERR_TOO_LARGE: return "the problem exceeds the fixed scratch memory of this entry point (use the variant that takes a workspace)";
     default: return "unknown status";
   }
 }

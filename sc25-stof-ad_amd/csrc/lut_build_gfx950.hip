@@ -17,8 +17,18 @@
 // A third kernel writes, on request, the reference's additive fp16 blocks
 // -10000 * (1 - block.half()) (src/util/masks.py:159-166) for the PART list.
 //
-// The scratch buffer is passed in by the caller.
+// The scratch buffer is either passed in by the caller (stof_build_lut) or a fixed array in
+// device memory (stof_build_lut_static), for callers that cannot allocate.
 #include "stof_common.h"
+
+// Scratch of stof_build_lut_static, the entry point that allocates nothing: class bytes and bit
+// rows for at most kStaticMaxTiles tiles (8.02 MB per GPU, held until the process ends).  In
+// host code the array's name is a stand-in, not a device address: the address of each device's
+// copy is taken once per device with hipGetSymbolAddress and only that pointer is used.
+constexpr int64_t kStaticMaxTiles = 16384;   // S = 8192 at 64 x 64 blocks
+constexpr int64_t kClsBytesStatic = kStaticMaxTiles;
+constexpr int64_t kBitsBytesStatic = kStaticMaxTiles * 64 * 8;
+static __device__ __align__(256) unsigned char scratch[kClsBytesStatic + kBitsBytesStatic];
 
 namespace {
 
@@ -193,6 +203,21 @@ __global__ __launch_bounds__(256) void lut_additive_blocks_kernel(const void* ma
   }
 }
 
+constexpr int kMaxDevices = 64;
+unsigned char* g_scratch_ptr[kMaxDevices] = {nullptr};
+
+int static_scratch(unsigned char** out) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return STOF_ERR_LAUNCH;
+  if (!g_scratch_ptr[dev]) {
+    void* ptr = nullptr;
+    if (hipGetSymbolAddress((void**)&ptr, HIP_SYMBOL(scratch)) != hipSuccess || !ptr) return STOF_ERR_LAUNCH;
+    g_scratch_ptr[dev] = static_cast<unsigned char*>(ptr);
+  }
+  *out = g_scratch_ptr[dev];
+  return STOF_OK;
+}
+
 bool block_ok(int b) { return b == 16 || b == 32 || b == 64 || b == 128; }
 
 int check_common(const void* mask, int elem_bytes, int64_t ld, int seq_len, int block_m, int block_n) {
@@ -262,6 +287,29 @@ extern "C" int stof_build_lut(const void* mask, int elem_bytes, int64_t ld, int 
   uint64_t* bits = reinterpret_cast<uint64_t*>(cls + (tiles + 255) / 256 * 256);
   return build(mask, elem_bytes, ld, seq_len, block_m, block_n, full_row_ptr, full_col_idx, part_row_ptr, part_col_idx,
                load_row_ptr, load_col_idx, part_bitmask, counts, cap_full, cap_part, cap_load, cls, bits, (hipStream_t)stream);
+}
+
+extern "C" int64_t stof_build_lut_static_max_tiles(void) { return kStaticMaxTiles; }
+
+extern "C" int stof_build_lut_static(const void* mask, int elem_bytes, int64_t ld, int seq_len, int block_m, int block_n,
+                                     int32_t* full_row_ptr, int32_t* full_col_idx,
+                                     int32_t* part_row_ptr, int32_t* part_col_idx,
+                                     int32_t* load_row_ptr, int32_t* load_col_idx,
+                                     uint64_t* part_bitmask, int32_t* counts,
+                                     int64_t cap_full, int64_t cap_part, int64_t cap_load, void* stream) {
+  int rc = check_common(mask, elem_bytes, ld, seq_len, block_m, block_n);
+  if (rc != STOF_OK) return rc;
+  rc = check_outputs(full_row_ptr, full_col_idx, part_row_ptr, part_col_idx, load_row_ptr, load_col_idx,
+                     part_bitmask, block_m, block_n, cap_full, cap_part, cap_load);
+  if (rc != STOF_OK) return rc;
+  const int64_t tiles = (int64_t)(seq_len / block_m) * (seq_len / block_n);
+  if (tiles > kStaticMaxTiles) return STOF_ERR_TOO_LARGE;   // beyond the fixed scratch: use stof_build_lut with a workspace
+  unsigned char* ptr = nullptr;   // this device's copy of the scratch array
+  rc = static_scratch(&ptr);
+  if (rc != STOF_OK) return rc;
+  return build(mask, elem_bytes, ld, seq_len, block_m, block_n, full_row_ptr, full_col_idx, part_row_ptr, part_col_idx,
+               load_row_ptr, load_col_idx, part_bitmask, counts, cap_full, cap_part, cap_load,
+               ptr, reinterpret_cast<uint64_t*>(ptr + kClsBytesStatic), (hipStream_t)stream);
 }
 
 extern "C" int stof_lut_additive_blocks(const void* mask, int elem_bytes, int64_t ld, int seq_len, int block_m, int block_n,

@@ -29,6 +29,9 @@ _SIGNATURES = {
     "stof_build_lut_workspace_bytes": (c_int64, [c_int, c_int, c_int]),
     "stof_build_lut": (c_int, [_P, c_int, c_int64, c_int, c_int, c_int, _P, _P, _P, _P, _P, _P, _P, _P,
                                c_int64, c_int64, c_int64, _P, c_int64, _P]),
+    "stof_build_lut_static_max_tiles": (c_int64, []),
+    "stof_build_lut_static": (c_int, [_P, c_int, c_int64, c_int, c_int, c_int, _P, _P, _P, _P, _P, _P, _P, _P,
+                                      c_int64, c_int64, c_int64, _P]),
     "stof_lut_additive_blocks": (c_int, [_P, c_int, c_int64, c_int, c_int, c_int, _P, _P, c_int64, _P, _P]),
     "stof_bias_res_ln": (c_int, [_P, _P, _P, _P, _P, _P, _P, _P, c_int64, c_int64, c_float, _P]),
     "stof_gemm_bias_act": (c_int, [_P, _P, _P, _P, c_int64, c_int64, c_int64, c_int64, c_int64, c_int, _P]),
