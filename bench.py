@@ -306,18 +306,42 @@ def bench_hbm_kernels(steps, warmup):
     return out
 
 
-def bench_lut_build(with_cpu):
-    """Block LUT of the C4 mask (S 4096, 64 x 64 blocks) built on the GPU, and the reference's
-    Python double loop (restated in oracle/) on the host for the same mask at S 2048."""
+def bench_lut_build(with_cpu, steps=200):
+    """Block LUT of the C4 mask (S 4096, 64 x 64 blocks) built by the GPU kernels: the whole
+    get_sparse_storage call (exactly shaped tensors: one device -> host read of the list lengths,
+    plus the reference's nnz figure and additive fp16 blocks), and the two kernels alone
+    (build_lut_device: no synchronisation; HBM-bound, S^2 x element bytes read once); next to
+    the reference's Python double loop (restated in oracle/) on the host at S 2048."""
     from stof import configs, masks as pm
-    mask = configs.mask_c4(4096).float()[None].cuda()
-    pm.get_sparse_storage(mask, 64, 64)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(5):
+    out = {}
+    for tag, dtype in (("fp16", torch.float16), ("fp32", torch.float32)):
+        mask = configs.mask_c4(4096).to(dtype)[None].cuda()
         pm.get_sparse_storage(mask, 64, 64)
-    torch.cuda.synchronize()
-    out = {"gpu_ms_S4096": (time.perf_counter() - t0) / 5 * 1e3}
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(20):
+            pm.get_sparse_storage(mask, 64, 64)
+        torch.cuda.synchronize()
+        out[f"get_sparse_storage_ms_S4096_{tag}"] = (time.perf_counter() - t0) / 20 * 1e3
+        # the two kernels with every buffer allocated beforehand (what a serving loop would do)
+        from stof import _lib
+        lib = _lib.lib()
+        S, tiles = 4096, 64 * 64
+        i32 = lambda n: torch.empty(n, dtype=torch.int32, device="cuda")
+        frp, prp, lrp, fci, pci, lci, counts = i32(65), i32(65), i32(65), i32(tiles), i32(tiles), i32(tiles), i32(4)
+        bits = torch.empty(tiles * 64, dtype=torch.int64, device="cuda")
+        ws = torch.empty(lib.stof_build_lut_workspace_bytes(S, 64, 64), dtype=torch.uint8, device="cuda")
+        m2d = mask[0]
+        stream = torch.cuda.current_stream().cuda_stream
+        args = (m2d.data_ptr(), m2d.element_size(), S, S, 64, 64, frp.data_ptr(), fci.data_ptr(), prp.data_ptr(), pci.data_ptr(),
+                lrp.data_ptr(), lci.data_ptr(), bits.data_ptr(), counts.data_ptr(), tiles, tiles, tiles, ws.data_ptr(), ws.numel(), stream)
+        _, ev = time_region(lambda: lib.stof_build_lut(*args), steps, 20)
+        assert counts.tolist() == [840, 106, 946, 0]
+        nbytes = 4096 * 4096 * mask.element_size()
+        out[f"kernels_ms_S4096_{tag}"] = ev
+        out[f"kernels_GBs_{tag}"] = nbytes / ev / 1e6
+        out[f"kernels_frac_hbm_{tag}"] = nbytes / ev / 1e6 / PEAK_HBM_GBS
+    out["gpu_ms_S4096"] = out["kernels_ms_S4096_fp16"]
     if with_cpu:
         from oracle import masks as om
         m2 = configs.mask_c4(2048).float()[None].numpy()

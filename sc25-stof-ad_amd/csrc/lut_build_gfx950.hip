@@ -125,14 +125,19 @@ __device__ __forceinline__ int block_sum(int v, int* lds) {
 __global__ __launch_bounds__(256) void lut_compact_kernel(const LutParams p) {
   __shared__ int red[4];
   __shared__ int wave_cnt[2][4];
-  __shared__ int part_col[256], part_slot[256];
+  __shared__ int part_col[256], part_slot[256];   // this chunk's partial tiles, in column order
   const int r = blockIdx.x;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  // tiles of the rows above: FULL and PARTIAL counts
+  // FULL and PARTIAL tiles of the rows above: the class bytes (0, 1, 2) four at a time
   int nf = 0, np = 0;
   const int64_t above = (int64_t)r * p.nK;
-  for (int64_t i = tid; i < above; i += 256) {
-    const int c = p.cls[i];
+  const uint32_t* cls4 = reinterpret_cast<const uint32_t*>(p.cls);   // (the class array is 4-byte aligned)
+  for (int64_t i = tid; i < (above >> 2); i += 256) {
+    const uint32_t x = cls4[i];
+    nf += __builtin_popcount(x & 0x01010101u); np += __builtin_popcount(x & 0x02020202u);
+  }
+  if (tid < (int)(above & 3)) {
+    const int c = p.cls[(above & ~(int64_t)3) + tid];
     nf += c == kClsFull; np += c == kClsPart;
   }
   int fbase = block_sum(nf, red);
@@ -150,20 +155,22 @@ __global__ __launch_bounds__(256) void lut_compact_kernel(const LutParams p) {
       if (w < wave) { f_before += wave_cnt[0][w]; p_before += wave_cnt[1][w]; }
       f_all += wave_cnt[0][w]; p_all += wave_cnt[1][w];
     }
+    const int pl = p_before + __builtin_popcountll(bp & below);   // rank among this chunk's partial tiles
     const int rf = fbase + f_before + __builtin_popcountll(bf & below);
-    const int rp = pbase + p_before + __builtin_popcountll(bp & below);
-    part_slot[tid] = -1;
+    const int rp = pbase + pl;
     if (cl == kClsFull) {
       if (rf < p.cap_full) p.fci[rf] = c;
       if (rf + rp < p.cap_load) p.lci[rf + rp] = c;
     } else if (cl == kClsPart) {
-      if (rp < p.cap_part) { p.pci[rp] = c; part_col[tid] = c; part_slot[tid] = rp; }
+      part_col[pl] = c;
+      part_slot[pl] = rp < p.cap_part ? rp : -1;
+      if (rp < p.cap_part) p.pci[rp] = c;
       if (rf + rp < p.cap_load) p.lci[rf + rp] = c;
     }
     __syncthreads();
     // bit rows of this chunk's partial tiles into their PART slots (a wavefront per tile)
     if (p.pbits && p.ws_bits) {
-      for (int t = wave; t < 256; t += 4) {
+      for (int t = wave; t < p_all; t += 4) {
         const int slot = part_slot[t];
         if (slot >= 0) p.pbits[(int64_t)slot * 64 + lane] = p.ws_bits[(above + part_col[t]) * 64 + lane];
       }
