@@ -22,6 +22,10 @@ __device__ __forceinline__ void load8(const half_t* p, float (&v)[8]) {
 }
 
 // CH = 16-byte chunks per lane; the row has at most 64*CH chunks (N <= 512*CH).
+// Every load of the row (x, residual, bias for all of the lane's chunks) is issued before the
+// first value is converted, so a wave has 2-3 x CH 16-byte loads in flight instead of one: with
+// one wave per row of 1.5 KB that is what it takes to keep HBM busy.  A chunk past the end of
+// the row reads chunk 0 instead (a valid address) and is zeroed afterwards.
 template <int CH>
 __global__ __launch_bounds__(256) void bias_res_ln_kernel(const LnParams p) {
   const int lane = threadIdx.x & 63;
@@ -31,31 +35,35 @@ __global__ __launch_bounds__(256) void bias_res_ln_kernel(const LnParams p) {
   const half_t* xr = p.x + row * p.N;
   const half_t* rr = p.res ? p.res + row * p.N : nullptr;
 
+  half8_t hx[CH], hr[CH], hb[CH];
+  bool valid[CH];
+#pragma unroll
+  for (int c = 0; c < CH; ++c) {
+    const int ch = lane + 64 * c;
+    valid[c] = ch < nchunk;
+    const int chs = valid[c] ? ch : 0;
+    hx[c] = *reinterpret_cast<const half8_t*>(xr + 8 * chs);
+    if (rr) hr[c] = *reinterpret_cast<const half8_t*>(rr + 8 * chs);
+    if (p.bias) hb[c] = *reinterpret_cast<const half8_t*>(p.bias + 8 * chs);
+  }
   float v[CH][8];
   float s = 0.f;
 #pragma unroll
   for (int c = 0; c < CH; ++c) {
-    const int ch = lane + 64 * c;
-    if (ch < nchunk) {
-      load8(xr + 8 * ch, v[c]);
-      if (p.bias) { float t[8]; load8(p.bias + 8 * ch, t);
 #pragma unroll
-        for (int i = 0; i < 8; ++i) v[c][i] += t[i]; }
-      if (rr) { float t[8]; load8(rr + 8 * ch, t);
-#pragma unroll
-        for (int i = 0; i < 8; ++i) v[c][i] += t[i]; }
-#pragma unroll
-      for (int i = 0; i < 8; ++i) s += v[c][i];
-    } else {
-#pragma unroll
-      for (int i = 0; i < 8; ++i) v[c][i] = 0.f;
+    for (int i = 0; i < 8; ++i) {
+      float t = (float)hx[c][i];
+      if (p.bias) t += (float)hb[c][i];
+      if (rr) t += (float)hr[c][i];
+      v[c][i] = valid[c] ? t : 0.f;
+      s += v[c][i];
     }
   }
   const float mean = wave_sum(s) * p.inv_n;
   float q = 0.f;
 #pragma unroll
   for (int c = 0; c < CH; ++c)
-    if (lane + 64 * c < nchunk) {
+    if (valid[c]) {
 #pragma unroll
       for (int i = 0; i < 8; ++i) { const float d = v[c][i] - mean; q += d * d; }
     }
@@ -69,7 +77,7 @@ __global__ __launch_bounds__(256) void bias_res_ln_kernel(const LnParams p) {
 #pragma unroll
   for (int c = 0; c < CH; ++c) {
     const int ch = lane + 64 * c;
-    if (ch < nchunk) {
+    if (valid[c]) {
       float gm[8], bt[8];
       if (p.gamma) load8(p.gamma + 8 * ch, gm);
       if (p.beta) load8(p.beta + 8 * ch, bt);
