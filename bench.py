@@ -94,12 +94,13 @@ def time_region(fn, steps, warmup, settle_ms=SETTLE_MS):
     return (t1 - t0) * 1e3 / steps, e0.elapsed_time(e1) / steps
 
 
-def bench_attn(cfg, mask_fn, steps, warmup, settle_ms=SETTLE_MS):
+def bench_attn(cfg, mask_fn, steps, warmup, settle_ms=SETTLE_MS, launch_form=None, dtype=torch.float16):
     from stof.ops import block_attn
     q, k, v, lut, n_active, _ = attn_setup(cfg, mask_fn, "cuda")
+    q, k, v = (t.to(dtype) for t in (q, k, v))
     out = torch.empty_like(q)
-    block_attn(q, k, v, lut, out=out)          # packs the partial-block bit masks once
-    wall_ms, ev_ms = time_region(lambda: block_attn(q, k, v, lut, out=out), steps, warmup, settle_ms)
+    block_attn(q, k, v, lut, out=out, launch_form=launch_form)          # packs the partial-block bit masks once
+    wall_ms, ev_ms = time_region(lambda: block_attn(q, k, v, lut, out=out, launch_form=launch_form), steps, warmup, settle_ms)
     flop = FLOP_PER_BLOCK * cfg.batch * cfg.heads * n_active
     return {"wall_ms": wall_ms, "kernel_ms": ev_ms, "flop": flop, "active_blocks": n_active,
             "tflops_wall": flop / wall_ms / 1e9, "tflops_kernel": flop / ev_ms / 1e9}
@@ -358,7 +359,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=2000,
                     help="untimed steps before the timed ones; the default (about 70 ms of load) lets the clocks settle")
     ap.add_argument("--no-extras", action="store_true", help="skip everything but the C4 attention step")
-    ap.add_argument("--extras", default="c1,c2,c4big,dense,c3,c3small,c5,hbm,lut",
+    ap.add_argument("--extras", default="c1,c2,c4big,forms,dense,c3,c3small,c5,hbm,lut",
                     help="comma-separated subset of the extra workloads to run (for profiling one kind of kernel)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--copy-probe", action="store_true",
@@ -410,6 +411,14 @@ def main():
             c4b = bench_attn(big, configs.mask_c4, max(args.steps // 4, 10), 5)
             also["C4_mask_B16_H16"] = {"tflops": c4b["tflops_kernel"], "frac_mfma_peak": c4b["tflops_kernel"] / PEAK_FP16_TFLOPS,
                                        "kernel_ms": c4b["kernel_ms"]}
+        if "forms" in want:
+            # the three launch forms on the headline workload (the default picks by grid size)
+            also["C4_launch_forms_kernel_ms"] = {
+                form: bench_attn(configs.C4, configs.mask_c4, max(args.steps // 4, 50), 50, launch_form=form)["kernel_ms"]
+                for form in ("two_rows", "key_split", "pipelined")}
+            # the same workload on bfloat16 tensors (not the headline: the reference computes in fp16)
+            also["C4_bf16_kernel_ms"] = bench_attn(configs.C4, configs.mask_c4, max(args.steps // 4, 50), 50,
+                                                   dtype=torch.bfloat16)["kernel_ms"]
         if "dense" in want:
             also["dense_S4096_B16_H16_vs_torch_sdpa"] = bench_dense_vs_sdpa(max(args.steps // 10, 10), 3)
         if "c1" in want:

@@ -7,7 +7,8 @@
  * Conventions
  *   - every pointer is a DEVICE pointer unless stated otherwise; the library never
  *     allocates, frees or retains caller memory;
- *   - all activations are IEEE fp16 (two bytes); accumulation and statistics are fp32;
+ *   - all activations are IEEE fp16 (two bytes; the attention entry points also take bfloat16);
+ *     accumulation and statistics are fp32;
  *   - `stream` is a hipStream_t passed as void* (NULL = the null stream); launches
  *     are asynchronous, nothing synchronises;
  *   - every function returns 0 on success or a negative STOF_ERR_* code; no launch
@@ -58,6 +59,9 @@ enum {
 /* activation selector of stof_gemm_bias_act */
 enum { STOF_ACT_NONE = 0, STOF_ACT_GELU_ERF = 1, STOF_ACT_GELU_TANH = 2, STOF_ACT_RELU = 3 };
 
+/* element format of q, k, v and out at the attention entry points */
+enum { STOF_DTYPE_F16 = 0, STOF_DTYPE_BF16 = 1 };
+
 /* launch form of the attention entry points */
 enum { STOF_FORM_DEFAULT = -1, STOF_FORM_TWO_ROWS = 0, STOF_FORM_KEY_SPLIT = 1, STOF_FORM_PIPELINED = 2 };
 
@@ -92,7 +96,9 @@ const char* stof_status_string(int status);
  * may be NULL when every row range over it is empty (no partial blocks; nothing allowed at all).
  *
  * Supported: D == 64, block_m == block_n == 64, S % 64 == 0 (the Python operator re-tiles LUTs
- * built with other block sizes to 64 x 64 before it calls this).
+ * built with other block sizes to 64 x 64 before it calls this).  dtype: STOF_DTYPE_F16 (the
+ * reference's only format) or STOF_DTYPE_BF16 for q, k, v and out alike; scores, softmax
+ * statistics and the output accumulator are fp32 either way.
  *
  * launch_form is the per-call counterpart of the reference launcher's num_warps (its kernel
  * selection by (num_warps, BLOCK_M, BLOCK_N), block_attn_mask_cuda.cu:6064-6322):
@@ -113,7 +119,7 @@ int stof_block_attn_fwd(
     int block_m, int block_n, float softmax_scale,
     const int64_t q_strides[3], const int64_t k_strides[3],
     const int64_t v_strides[3], const int64_t out_strides[3],
-    int batch_size, int seq_len, int head_num, int head_size,
+    int batch_size, int seq_len, int head_num, int head_size, int dtype,
     int64_t lut_batch_stride, int launch_form, void* stream);
 
 /*
@@ -142,12 +148,12 @@ int stof_pack_mask_bits(const void* src, uint64_t* dst, int64_t rows, int64_t co
  *   kind STOF_ROW_MASK:    additionally bit j of mask_bits[i*(S/64) + j/64] set
  * Unlike the reference kernels the softmax is max-subtracted (no overflow) and rows
  * without an allowed key produce zeros.  q, k, v contiguous [B,H,S,D], D == 64, S % 64 == 0.
- * launch_form as for stof_block_attn_fwd.
+ * dtype and launch_form as for stof_block_attn_fwd.
  */
 int stof_rowwise_attn_fwd(
     const void* q, const void* k, const void* v, void* out,
     int kind, int is_causal, int bandwidth, const uint64_t* mask_bits,
-    int batch_size, int seq_len, int head_num, int head_size, int launch_form, void* stream);
+    int batch_size, int seq_len, int head_num, int head_size, int dtype, int launch_form, void* stream);
 
 /*
  * Block LUT of a dense 0/1 mask, built on the GPU: the classification loop of get_sparse_storage

@@ -66,8 +66,23 @@ struct AttnParams {
 
 enum { kKindLut = 0, kKindPred = 1, kKindBits = 2 };
 
+// BF: the tensors are bfloat16 instead of fp16.  Operand fragments are carried as 16-bit
+// patterns in half8_t either way (loads, LDS and the transposing read do not look at the
+// format); only the MFMA opcode, the conversion of the probabilities and the final store differ.
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef unsigned short ushort8_t __attribute__((ext_vector_type(8)));
+template <bool BF>
 __device__ __forceinline__ floatx16 mfma32(half8_t a, half8_t b, floatx16 c) {
-  return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+  if constexpr (BF)
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
+  else
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+}
+// fp32 -> the tensors' 16-bit format (round to nearest even), as a 16-bit pattern in half_t
+template <bool BF>
+__device__ __forceinline__ half_t to_elem(float x) {
+  if constexpr (BF) return __builtin_bit_cast(half_t, (__bf16)x);
+  else return (half_t)x;
 }
 
 // max / sum of a value with its partner lane (lane ^ 32).  v_permlane32_swap(x, x) leaves
@@ -109,7 +124,7 @@ template <int ROWS> struct RowPtrs {
 // merged through LDS at the end).  The second form halves the work of a wave per key block,
 // so the chain of key blocks of a long LUT row finishes in half the time; it is used for
 // small grids, where that chain and not throughput sets the run time.
-template <int KIND, int ROWS, int KS, bool PIPE = false>
+template <int KIND, int ROWS, int KS, bool PIPE, bool BF>
 __device__ __forceinline__ void attn_group(const AttnParams& p, const int bh, const int pair, const RowPtrs<ROWS>& pre,
                                            unsigned char* k_lds0, unsigned char* k_lds1,
                                            unsigned char* v_lds0, unsigned char* v_lds1,
@@ -433,11 +448,17 @@ __device__ __forceinline__ void attn_group(const AttnParams& p, const int bh, co
         for (int dt = 0; dt < 2; ++dt)
 #pragma unroll
           for (int r = 0; r < 16; ++r) oacc[dt][r] *= alpha;
-        const half_t ah = (half_t)alpha;
 #pragma unroll
-        for (int s2 = 0; s2 < 2; ++s2)
+        for (int s2 = 0; s2 < 2; ++s2) {
+          // (bf16 -> fp32 as a shift of the whole vector's bit patterns: casting single elements
+          // of the half-typed container to __bf16 is miscompiled by this toolchain)
+          const ushort8_t bits16 = __builtin_bit_cast(ushort8_t, p_prev[s2]);
 #pragma unroll
-          for (int e = 0; e < 8; ++e) p_prev[s2][e] *= ah;
+          for (int e = 0; e < 8; ++e) {
+            if constexpr (BF) p_prev[s2][e] = to_elem<BF>(__builtin_bit_cast(float, (uint32_t)bits16[e] << 16) * alpha);
+            else p_prev[s2][e] *= (half_t)alpha;
+          }
+        }
       }
       warm = !__any(m_run == -INFINITY);
     };
@@ -500,26 +521,29 @@ __device__ __forceinline__ void attn_group(const AttnParams& p, const int bh, co
 #pragma unroll
       for (int r = 0; r < 16; ++r) s_out[r] = 0.f;
       half2_t part[4];
+      float fsum = 0.f;
 #pragma unroll
       for (int c = 0; c < 8; ++c) {
         __builtin_amdgcn_sched_barrier(0);
         const int j = c >> 1;
-        if (c & 1) oacc[j & 1] = mfma32(frag[c], p_in[j >> 1], oacc[j & 1]);
-        else s_out = mfma32(frag[c], qf[j], s_out);
+        if (c & 1) oacc[j & 1] = mfma32<BF>(frag[c], p_in[j >> 1], oacc[j & 1]);
+        else s_out = mfma32<BF>(frag[c], qf[j], s_out);
         if (c + kAhead < 8) frag[c + kAhead] = fetch_this(c + kAhead);
         else if (has_next) frag_next[c + kAhead - 8] = fetch_next(c + kAhead - 8);
         const int r = 2 * c;
         const float e0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s_in[r], p.c, -sub));
         const float e1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s_in[r + 1], p.c, -sub));
-        const half2_t e2 = {(half_t)e0, (half_t)e1};
+        const half2_t e2 = {to_elem<BF>(e0), to_elem<BF>(e1)};
         p_out[r >> 3][r & 7] = e2[0];
         p_out[r >> 3][(r & 7) + 1] = e2[1];
-        part[c & 3] = c < 4 ? e2 : part[c & 3] + e2;
+        if constexpr (BF) fsum = c == 0 ? e0 + e1 : fsum + (e0 + e1);   // (bf16 keeps 8 bits: sum in fp32)
+        else part[c & 3] = c < 4 ? e2 : part[c & 3] + e2;
       }
       __builtin_amdgcn_sched_barrier(0);
       // (Pin the probabilities here: being pure arithmetic that is only read by the next half-step,
       // they would otherwise be sunk out of the slices, past the side blocks in between.)
       asm volatile("" : "+v"(p_out[0]), "+v"(p_out[1]));
+      if constexpr (BF) return fsum;
       const half2_t tot = (part[0] + part[1]) + (part[2] + part[3]);
       return (float)tot[0] + (float)tot[1];
     };
@@ -694,7 +718,7 @@ __device__ __forceinline__ void attn_group(const AttnParams& p, const int bh, co
   #pragma unroll
           for (int mt = 0; mt < kMT; ++mt) {
             const half8_t a = *reinterpret_cast<const __attribute__((address_space(3))) half8_t*>(kt + (mt0 + mt) * 4096 + k_rd[ks]);
-            sacc[mt] = mfma32(a, qf[ks], sacc[mt]);
+            sacc[mt] = mfma32<BF>(a, qf[ks], sacc[mt]);
           }
       };
       if (need_mask) {
@@ -748,21 +772,24 @@ __device__ __forceinline__ void attn_group(const AttnParams& p, const int bh, co
       half8_t pf[kMT][2];   // [key sub-tile][half]: B operand of O^T = V^T . P^T
       auto probabilities = [&]() -> float {
         half2_t part[4];   // four interleaved partial sums of at most 8 values each
+        float fsum = 0.f;
 #pragma unroll
         for (int mt = 0; mt < kMT; ++mt)
 #pragma unroll
           for (int r = 0; r < 16; r += 2) {
             const float e0 = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[mt][r], p.c, -mc_run));
             const float e1 = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[mt][r + 1], p.c, -mc_run));
-            const half2_t e2 = {(half_t)e0, (half_t)e1};
+            const half2_t e2 = {to_elem<BF>(e0), to_elem<BF>(e1)};
             pf[mt][r >> 3][r & 7] = e2[0];
             pf[mt][r >> 3][(r & 7) + 1] = e2[1];
+            if constexpr (BF) { fsum += e0 + e1; continue; }   // (bf16 keeps 8 bits: sum in fp32)
             // Row sum with packed fp16 adds on the values the second product uses, folded to fp32
             // once per tile (v_dot2c_f32_f16 would do it in one instruction per pair but runs on
             // the matrix pipeline and stalls behind every MFMA in flight on the SIMD).
             const int i = (r >> 1) & 3;
             part[i] = (mt == 0 && r < 8) ? e2 : part[i] + e2;
           }
+        if constexpr (BF) return fsum;
         const half2_t tot = (part[0] + part[1]) + (part[2] + part[3]);
         return (float)tot[0] + (float)tot[1];
       };
@@ -780,7 +807,7 @@ __device__ __forceinline__ void attn_group(const AttnParams& p, const int bh, co
             const short4_t a0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4*)(vp + v_rd[dt][0]));
             const short4_t a1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4*)(vp + v_rd[dt][1]));
             const half8_t a = __builtin_bit_cast(half8_t, (short8_t)__builtin_shufflevector(a0, a1, 0, 1, 2, 3, 4, 5, 6, 7));
-            oacc[dt] = mfma32(a, pf[mt][s2], oacc[dt]);
+            oacc[dt] = mfma32<BF>(a, pf[mt][s2], oacc[dt]);
           }
     };
 
@@ -837,7 +864,7 @@ __device__ __forceinline__ void attn_group(const AttnParams& p, const int bh, co
     for (int q4 = 0; q4 < 4; ++q4) {
       half4_t o4;
 #pragma unroll
-      for (int e = 0; e < 4; ++e) o4[e] = (half_t)(oacc[dt][4 * q4 + e] * inv);
+      for (int e = 0; e < 4; ++e) o4[e] = to_elem<BF>(oacc[dt][4 * q4 + e] * inv);
       *reinterpret_cast<half4_t*>(orow + 32 * dt + 8 * q4 + 4 * g) = o4;
     }
 }
@@ -936,7 +963,7 @@ __device__ __forceinline__ void balanced_group(const AttnParams& p, int& bh, int
   }
 }
 
-template <int KIND, int ROWS, int KS>
+template <int KIND, int ROWS, int KS, bool BF>
 __global__ __launch_bounds__(128 * ROWS * KS, 4) void block_attn_fwd_kernel(const AttnParams p) {
   STOF_ATTN_LDS_TILES;
   int bh, pair;
@@ -950,12 +977,12 @@ __global__ __launch_bounds__(128 * ROWS * KS, 4) void block_attn_fwd_kernel(cons
     bh = vid / p.nP;
     pair = zigzag(vid - bh * p.nP, bh, p.nP);
   }
-  attn_group<KIND, ROWS, KS>(p, bh, pair, pre, k_lds0, k_lds1, v_lds0, v_lds1);
+  attn_group<KIND, ROWS, KS, false, BF>(p, bh, pair, pre, k_lds0, k_lds1, v_lds0, v_lds1);
 }
 
 // Two query blocks per workgroup with the software-pipelined main loop (rings of three K and
 // three V tiles: 48 KB of LDS).
-template <int KIND>
+template <int KIND, bool BF>
 __global__ __launch_bounds__(256, 3) void block_attn_pipe_kernel(const AttnParams p) {
   STOF_ATTN_LDS_TILES;
   __shared__ __attribute__((aligned(1024))) unsigned char k_lds2[kTile];
@@ -971,7 +998,7 @@ __global__ __launch_bounds__(256, 3) void block_attn_pipe_kernel(const AttnParam
     bh = vid / p.nP;
     pair = zigzag(vid - bh * p.nP, bh, p.nP);
   }
-  attn_group<KIND, 2, 1, true>(p, bh, pair, pre, k_lds0, k_lds1, v_lds0, v_lds1, k_lds2, v_lds2);
+  attn_group<KIND, 2, 1, true, BF>(p, bh, pair, pre, k_lds0, k_lds1, v_lds0, v_lds1, k_lds2, v_lds2);
 }
 
 // dst[r*(cols/64)+w] bit t = pred(src[r*ld + 64w + t]).
@@ -1084,8 +1111,8 @@ void set_balance(AttnParams& p, int max_groups) {
   p.balance = (p.total % 8 == 0 && p.chunk % p.nP == 0 && p.nP <= max_groups && p.nP > 1 && cus % 8 == 0 && cus >= 8) ? 1 : 0;
 }
 
-template <int KIND>
-void launch_attn(AttnParams& p, int nQ, int64_t bh, int requested_form, hipStream_t stream) {
+template <int KIND, bool BF>
+void launch_attn_as(AttnParams& p, int nQ, int64_t bh, int requested_form, hipStream_t stream) {
   const int64_t two_row_groups = (int64_t)((nQ + kRowsPerGroup - 1) / kRowsPerGroup) * bh;
   const int form = pick_form(requested_form, two_row_groups, nQ);
   if (form == kFormKeySplit) {
@@ -1093,17 +1120,23 @@ void launch_attn(AttnParams& p, int nQ, int64_t bh, int requested_form, hipStrea
     p.total = (int)(nQ * bh);
     p.chunk = (p.total + 7) / 8;
     set_balance(p, kBalanceMaxGroupsKeySplit);
-    hipLaunchKernelGGL((block_attn_fwd_kernel<KIND, 1, 2>), dim3(p.chunk * 8), dim3(256), 0, stream, p);
+    hipLaunchKernelGGL((block_attn_fwd_kernel<KIND, 1, 2, BF>), dim3(p.chunk * 8), dim3(256), 0, stream, p);
   } else {
     p.nP = (nQ + kRowsPerGroup - 1) / kRowsPerGroup;
     p.total = (int)two_row_groups;
     p.chunk = (p.total + 7) / 8;
     set_balance(p, kBalanceMaxGroupsTwoRows);
     if (form == kFormPipelined)
-      hipLaunchKernelGGL((block_attn_pipe_kernel<KIND>), dim3(p.chunk * 8), dim3(256), 0, stream, p);
+      hipLaunchKernelGGL((block_attn_pipe_kernel<KIND, BF>), dim3(p.chunk * 8), dim3(256), 0, stream, p);
     else
-      hipLaunchKernelGGL((block_attn_fwd_kernel<KIND, kRowsPerGroup, 1>), dim3(p.chunk * 8), dim3(128 * kRowsPerGroup), 0, stream, p);
+      hipLaunchKernelGGL((block_attn_fwd_kernel<KIND, kRowsPerGroup, 1, BF>), dim3(p.chunk * 8), dim3(128 * kRowsPerGroup), 0, stream, p);
   }
+}
+
+template <int KIND>
+void launch_attn(AttnParams& p, int nQ, int64_t bh, int requested_form, int dtype, hipStream_t stream) {
+  if (dtype == STOF_DTYPE_BF16) launch_attn_as<KIND, true>(p, nQ, bh, requested_form, stream);
+  else launch_attn_as<KIND, false>(p, nQ, bh, requested_form, stream);
 }
 
 bool strides_ok(const int64_t s[3]) {
@@ -1126,9 +1159,10 @@ extern "C" int stof_block_attn_fwd(
     int block_m, int block_n, float softmax_scale,
     const int64_t q_strides[3], const int64_t k_strides[3],
     const int64_t v_strides[3], const int64_t out_strides[3],
-    int batch_size, int seq_len, int head_num, int head_size,
+    int batch_size, int seq_len, int head_num, int head_size, int dtype,
     int64_t lut_batch_stride, int launch_form, void* stream) {
   if (launch_form < kFormAuto || launch_form > kFormPipelined) return STOF_ERR_UNSUPPORTED;
+  if (dtype != STOF_DTYPE_F16 && dtype != STOF_DTYPE_BF16) return STOF_ERR_UNSUPPORTED;
   if (!q || !k || !v || !out || !full_row_ptr || !part_row_ptr || !load_row_ptr ||
       !q_strides || !k_strides || !v_strides || !out_strides)
     return STOF_ERR_NULL_POINTER;
@@ -1154,15 +1188,16 @@ extern "C" int stof_block_attn_fwd(
   p.B = batch_size; p.S = seq_len; p.H = head_num; p.nQ = nQ;
   p.c = softmax_scale * 1.4426950408889634f;
   p.row_bits = nullptr; p.words = 0; p.causal = 0; p.band = 0;
-  launch_attn<kKindLut>(p, nQ, (int64_t)batch_size * head_num, launch_form, (hipStream_t)stream);
+  launch_attn<kKindLut>(p, nQ, (int64_t)batch_size * head_num, launch_form, dtype, (hipStream_t)stream);
   return stof_check_launch();
 }
 
 extern "C" int stof_rowwise_attn_fwd(
     const void* q, const void* k, const void* v, void* out,
     int kind, int is_causal, int bandwidth, const uint64_t* mask_bits,
-    int batch_size, int seq_len, int head_num, int head_size, int launch_form, void* stream) {
+    int batch_size, int seq_len, int head_num, int head_size, int dtype, int launch_form, void* stream) {
   if (launch_form < kFormAuto || launch_form > kFormPipelined) return STOF_ERR_UNSUPPORTED;
+  if (dtype != STOF_DTYPE_F16 && dtype != STOF_DTYPE_BF16) return STOF_ERR_UNSUPPORTED;
   if (!q || !k || !v || !out) return STOF_ERR_NULL_POINTER;
   if (kind != STOF_ROW_FULL && kind != STOF_ROW_SLIDING && kind != STOF_ROW_MASK) return STOF_ERR_UNSUPPORTED;
   if (kind == STOF_ROW_MASK && !mask_bits) return STOF_ERR_NULL_POINTER;
@@ -1184,8 +1219,8 @@ extern "C" int stof_rowwise_attn_fwd(
   p.c = (1.0f / sqrtf((float)head_size)) * 1.4426950408889634f;
   p.row_bits = mask_bits; p.words = seq_len / 64; p.causal = is_causal ? 1 : 0;
   p.band = kind == STOF_ROW_SLIDING ? bandwidth : 0;
-  if (kind == STOF_ROW_MASK) launch_attn<kKindBits>(p, nQ, (int64_t)batch_size * head_num, launch_form, (hipStream_t)stream);
-  else launch_attn<kKindPred>(p, nQ, (int64_t)batch_size * head_num, launch_form, (hipStream_t)stream);
+  if (kind == STOF_ROW_MASK) launch_attn<kKindBits>(p, nQ, (int64_t)batch_size * head_num, launch_form, dtype, (hipStream_t)stream);
+  else launch_attn<kKindPred>(p, nQ, (int64_t)batch_size * head_num, launch_form, dtype, (hipStream_t)stream);
   return stof_check_launch();
 }
 

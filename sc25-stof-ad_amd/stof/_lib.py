@@ -21,11 +21,11 @@ _SIGNATURES = {
     "stof_block_attn_fwd": (c_int, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P,
                                     c_int, c_int, c_float,
                                     POINTER(c_int64), POINTER(c_int64), POINTER(c_int64), POINTER(c_int64),
-                                    c_int, c_int, c_int, c_int, c_int64, c_int, _P]),
+                                    c_int, c_int, c_int, c_int, c_int, c_int64, c_int, _P]),
     "stof_attn_set_launch_form": (c_int, [c_int]),
     "stof_pack_mask_bits": (c_int, [_P, _P, c_int64, c_int64, c_int64, c_int, _P]),
     "stof_rowwise_attn_fwd": (c_int, [_P, _P, _P, _P, c_int, c_int, c_int, _P,
-                                      c_int, c_int, c_int, c_int, c_int, _P]),
+                                      c_int, c_int, c_int, c_int, c_int, c_int, _P]),
     "stof_build_lut_workspace_bytes": (c_int64, [c_int, c_int, c_int]),
     "stof_build_lut": (c_int, [_P, c_int, c_int64, c_int, c_int, c_int, _P, _P, _P, _P, _P, _P, _P, _P,
                                c_int64, c_int64, c_int64, _P, c_int64, _P]),

@@ -43,6 +43,7 @@ def _require(cond, msg):
         raise StofError(msg)
 
 
+_DTYPES = {torch.float16: 0, torch.bfloat16: 1}   # STOF_DTYPE_*
 _LAUNCH_FORMS = {None: -1, "default": -1, "auto": -1, "two_rows": 0, "key_split": 1, "pipelined": 2}
 
 
@@ -218,8 +219,8 @@ def _check_i32(name, t, device):
 
 def block_attn(q, k, v, lut, block_m=64, block_n=64, out=None, out_layout="bhsd", softmax_scale=None,
                launch_form=None, revalidate=False):
-    """Block-masked attention.  q, k, v: fp16 views ``[B,H,S,D]`` with unit stride in D (any
-    other strides).  ``lut`` = (full_row_ptr, full_col_idx, part_row_ptr, part_col_idx,
+    """Block-masked attention.  q, k, v: fp16 (or, all three, bfloat16) views ``[B,H,S,D]`` with
+    unit stride in D (any other strides).  ``lut`` = (full_row_ptr, full_col_idx, part_row_ptr, part_col_idx,
     part_block_mask, load_row_ptr, load_col_idx) as returned by ``get_sparse_storage`` (the
     leading ``nnz`` dropped) or by ``get_sparse_storage_batched`` (2-D row pointers: one LUT
     per sample).  Returns ``out``: ``[B,H,S,D]`` (``out_layout='bhsd'``) or ``[B,S,H*D]``
@@ -233,8 +234,9 @@ def block_attn(q, k, v, lut, block_m=64, block_n=64, out=None, out_layout="bhsd"
     """
     _require(q.is_cuda, "q must be a CUDA tensor (this path has no CPU implementation)")
     dev = q.device
+    _require(q.dtype in _DTYPES, f"q must be float16 or bfloat16, got {q.dtype}")
     for name, t in (("q", q), ("k", k), ("v", v)):
-        _require(t.dtype == torch.float16, f"{name} must be float16, got {t.dtype}")
+        _require(t.dtype == q.dtype, f"{name} must be {q.dtype} like q, got {t.dtype}")
         _require(t.dim() == 4 and t.stride(3) == 1, f"{name} must be [B,H,S,D] with contiguous D")
         _require(t is q or t.device == dev, f"{name} is on a different device than q")
     _require(k.shape == q.shape and v.shape == q.shape, "q, k, v must have the same shape")
@@ -245,9 +247,9 @@ def block_attn(q, k, v, lut, block_m=64, block_n=64, out=None, out_layout="bhsd"
     lut_ptrs, lut_bs = _prepared_lut(lut, B, S, block_m, block_n, dev)
     if out is None:
         if out_layout == "bhsd":
-            out = torch.empty((B, H, S, D), dtype=torch.float16, device=dev)
+            out = torch.empty((B, H, S, D), dtype=q.dtype, device=dev)
         else:
-            out = torch.empty((B, S, H * D), dtype=torch.float16, device=dev)
+            out = torch.empty((B, S, H * D), dtype=q.dtype, device=dev)
     if out_layout == "bhsd":
         _require(out.shape == (B, H, S, D) and out.stride(3) == 1, "out must be [B,H,S,D] with contiguous D")
         ostr = strides3(out)
@@ -256,13 +258,13 @@ def block_attn(q, k, v, lut, block_m=64, block_n=64, out=None, out_layout="bhsd"
         ostr = (_lib.c_int64 * 3)(out.stride(0), D, out.stride(1))
     else:
         raise StofError(f"unknown out_layout {out_layout!r}")
-    _require(out.dtype == torch.float16 and out.device == dev, "out must be fp16 on q's device")
+    _require(out.dtype == q.dtype and out.device == dev, "out must have q's dtype and device")
     scale = softmax_scale if softmax_scale is not None else 1.0 / math.sqrt(D)
     check(_lib.lib().stof_block_attn_fwd(
         q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(),
         *lut_ptrs, 64, 64, scale,
         strides3(q), strides3(k), strides3(v), ostr,
-        B, S, H, D, lut_bs, form, _stream(dev)), "stof_block_attn_fwd")
+        B, S, H, D, _DTYPES[q.dtype], lut_bs, form, _stream(dev)), "stof_block_attn_fwd")
     return out
 
 
@@ -293,8 +295,9 @@ class Block_Attn_Mask(Function):
 
 def _rowwise(kind, q, k, v, is_causal, bandwidth, row_mask, launch_form=None):
     _require(q.is_cuda, "q must be a CUDA tensor (this path has no CPU implementation)")
-    for name, t in (("q", q), ("k", k), ("v", v)):
-        _require(t.dtype == torch.float16, f"{name} must be float16, got {t.dtype}")
+    _require(q.dtype in _DTYPES, f"q must be float16 or bfloat16, got {q.dtype}")
+    for name, t in (("k", k), ("v", v)):
+        _require(t.dtype == q.dtype, f"{name} must be {q.dtype} like q, got {t.dtype}")
     q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
     B, H, S, D = q.shape
     result = torch.zeros((B, S, H * D), device=q.device, dtype=q.dtype)
@@ -313,7 +316,7 @@ def _rowwise(kind, q, k, v, is_causal, bandwidth, row_mask, launch_form=None):
     check(_lib.lib().stof_rowwise_attn_fwd(
         q.data_ptr(), k.data_ptr(), v.data_ptr(), result.data_ptr(),
         kind, 1 if is_causal else 0, int(bandwidth), _ptr(bits),
-        B, S, H, D, _form(launch_form), _stream(q.device)), "stof_rowwise_attn_fwd")
+        B, S, H, D, _DTYPES[q.dtype], _form(launch_form), _stream(q.device)), "stof_rowwise_attn_fwd")
     return result
 
 

@@ -51,7 +51,7 @@ def test_block_attn_argument_checks(lib):
     P = 4096   # fake, 16-byte aligned, never dereferenced: validation fails first
     call = lambda **kw: lib.stof_block_attn_fwd(
         kw.get("q", P), P, P, P, P, P, P, P, P, P, P, kw.get("bm", 64), kw.get("bn", 64), 0.125,
-        kw.get("qs", st), st, st, st, 1, kw.get("S", 128), 12, kw.get("D", 64), kw.get("lbs", 0), kw.get("form", -1), None)
+        kw.get("qs", st), st, st, st, 1, kw.get("S", 128), 12, kw.get("D", 64), kw.get("dtype", 0), kw.get("lbs", 0), kw.get("form", -1), None)
     assert call(q=None) == -1            # NULL pointer
     assert call(S=100) == -2             # seq_len not a multiple of 64
     assert call(S=0) == -2
@@ -61,6 +61,7 @@ def test_block_attn_argument_checks(lib):
     assert call(qs=_s3(12 * 128 * 64, 128 * 64, 65)) == -4   # stride not a multiple of 8
     assert call(lbs=2) == -6             # per-sample LUT stride too small
     assert call(form=3) == -3            # launch form
+    assert call(dtype=2) == -3           # element format
 
 
 def test_other_entry_points_argument_checks(lib):
@@ -77,11 +78,11 @@ def test_other_entry_points_argument_checks(lib):
     assert lib.stof_gemm_bias_act(P, P + 8, None, P, 64, 64, 64, 64, 64, 0, None) == -4
     assert lib.stof_gemm_bias_res_ln(P, P, None, None, None, None, P, 64, 384, 64, 1e-5, None) == -3   # N
     assert lib.stof_gemm_bias_res_ln(P, P, None, None, None, None, P, 64, 768, 48, 1e-5, None) == -2   # K % 32
-    assert lib.stof_rowwise_attn_fwd(P, P, P, P, 7, 0, 0, None, 1, 128, 12, 64, -1, None) == -3
-    assert lib.stof_rowwise_attn_fwd(P, P, P, P, 2, 0, 0, None, 1, 128, 12, 64, -1, None) == -1            # mask kind, no bits
-    assert lib.stof_rowwise_attn_fwd(P, P, P, P, 1, 1, 0, None, 1, 128, 12, 64, -1, None) == -2            # band <= 0
-    assert lib.stof_rowwise_attn_fwd(P, P, P, P, 0, 0, 0, None, 1, 130, 12, 64, -1, None) == -2
-    assert lib.stof_rowwise_attn_fwd(P, P, P, P, 0, 0, 0, None, 1, 128, 12, 64, 5, None) == -3           # launch form
+    assert lib.stof_rowwise_attn_fwd(P, P, P, P, 7, 0, 0, None, 1, 128, 12, 64, 0, -1, None) == -3
+    assert lib.stof_rowwise_attn_fwd(P, P, P, P, 2, 0, 0, None, 1, 128, 12, 64, 0, -1, None) == -1            # mask kind, no bits
+    assert lib.stof_rowwise_attn_fwd(P, P, P, P, 1, 1, 0, None, 1, 128, 12, 64, 0, -1, None) == -2            # band <= 0
+    assert lib.stof_rowwise_attn_fwd(P, P, P, P, 0, 0, 0, None, 1, 130, 12, 64, 0, -1, None) == -2
+    assert lib.stof_rowwise_attn_fwd(P, P, P, P, 0, 0, 0, None, 1, 128, 12, 64, 0, 5, None) == -3           # launch form
 
 
 def test_missing_library_fails_loudly(monkeypatch, tmp_path):
