@@ -226,7 +226,7 @@ int stof_bias_res_ln(const void* x, const void* bias, const void* residual,
 /*
  * C[M,N] = act( A[M,K] @ W^T + bias[N] ) with W given as Wt[N,K] (K contiguous, the
  * nn.Linear orientation).  A rows at pitch lda, C rows at pitch ldc (elements).
- * K % 64 == 0, N % 8 == 0, lda % 8 == 0, ldc % 4 == 0; M arbitrary.  bias may be NULL.
+ * K % 64 == 0, N % 8 == 0, lda % 8 == 0, ldc % 8 == 0; M arbitrary.  bias may be NULL.
  */
 int stof_gemm_bias_act(const void* A, const void* Wt, const void* bias, void* C,
                        int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldc,
