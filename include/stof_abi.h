@@ -233,6 +233,24 @@ int stof_gemm_bias_act(const void* A, const void* Wt, const void* bias, void* C,
                        int act, void* stream);
 
 /*
+ * Y[M,H] = act( X[M,K] @ W1^T + b1[F] ) @ W2^T (+ b2[H]) in ONE launch, W1 given as W1t[F,K] and W2
+ * as W2t[H,F] (nn.Linear orientation); the [M,F] intermediate is rounded to fp16 and stays on
+ * chip.  Replaces triton_matmul_batch (src/triton_template/gemm_gemm.py:99-174; b2 is an
+ * addition for the encoder's second FFN bias, NULL gives the reference's result).  Meant for
+ * small M (<= ~1024 rows), where two separate GEMM launches are latency-bound.
+ * K % 64 == 0, F % 128 == 0, H % 128 == 0, ldx % 8 == 0, ldy % 4 == 0; b1, b2 may be NULL.
+ * workspace: stof_gemm_act_gemm_workspace_bytes(M, H) bytes of device memory (16-byte aligned)
+ * that hold ZEROS at the first call; every call leaves them zero again, so one buffer serves
+ * any number of calls that do not overlap in time (calls sharing a workspace on different
+ * streams race).  The contributions of the F / 128 chunks are added in fp32 with atomic adds,
+ * so the last bits of the fp32 sums depend on arrival order.
+ */
+int64_t stof_gemm_act_gemm_workspace_bytes(int64_t M, int64_t H);
+int stof_gemm_act_gemm(const void* X, const void* W1t, const void* b1, const void* W2t, const void* b2,
+                       void* Y, int64_t M, int64_t K, int64_t F, int64_t H, int64_t ldx, int64_t ldy,
+                       int act, void* workspace, int64_t workspace_bytes, void* stream);
+
+/*
  * C[M,N] = LayerNorm( A[M,K] @ W^T + bias[N] + residual[M,N] ) * gamma + beta, the whole
  * row of N owned by one workgroup so the pre-normalisation values never reach HBM.
  * N in {256, 512, 768, 1024}; K % 32 == 0.  bias / residual / gamma / beta may be NULL.

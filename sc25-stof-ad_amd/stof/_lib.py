@@ -35,6 +35,9 @@ _SIGNATURES = {
     "stof_lut_additive_blocks": (c_int, [_P, c_int, c_int64, c_int, c_int, c_int, _P, _P, c_int64, _P, _P]),
     "stof_bias_res_ln": (c_int, [_P, _P, _P, _P, _P, _P, _P, _P, c_int64, c_int64, c_float, _P]),
     "stof_gemm_bias_act": (c_int, [_P, _P, _P, _P, c_int64, c_int64, c_int64, c_int64, c_int64, c_int, _P]),
+    "stof_gemm_act_gemm_workspace_bytes": (c_int64, [c_int64, c_int64]),
+    "stof_gemm_act_gemm": (c_int, [_P, _P, _P, _P, _P, _P, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64,
+                                   c_int, _P, c_int64, _P]),
     "stof_gemm_bias_res_ln": (c_int, [_P, _P, _P, _P, _P, _P, _P, c_int64, c_int64, c_int64, c_float, _P]),
 }
 

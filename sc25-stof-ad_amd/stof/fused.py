@@ -9,6 +9,7 @@ Reference-named entry points (same signatures as ``src/triton_template``):
 and the explicit forms the encoder layer uses:
 
 * ``gemm_bias_act(x, Wt, bias, act)``                          act(x @ Wt^T + bias)
+* ``gemm_act_gemm(x, W1t, b1, W2t, b2, act)``                  act(x @ W1t^T + b1) @ W2t^T + b2, one launch
 * ``gemm_bias_residual_layernorm(x, Wt, bias, residual, gamma, beta, eps)``
 * ``bias_residual_layernorm(x, bias, residual, gamma, beta, eps)``
 
@@ -153,10 +154,74 @@ def triton_matmul_bias_layernorm(A, B, bias, eps=1e-5):
     return gemm_bias_residual_layernorm(A, Wt, None, bias, None, None, eps)
 
 
-def triton_matmul_batch(a, b, d, bias):
+# Rows up to which "auto" callers take the single-launch chained form.  0: never - measured on
+# MI355X it loses to two GEMM launches at every row count tried (M 256 / 512 / 1024 at K 768,
+# F 3072: 57 / 79 / 123 us against 30 / 31 / 35 us), see csrc/ffn_chain_gfx950.hip.
+CHAIN_MAX_ROWS = 0
+_chain_ws = {}            # (device index, stream handle) -> zeroed workspace tensor, grown on demand
+
+
+def chain_supported(M, K, F, H):
+    """Shapes the single-launch chained kernel takes (stof_gemm_act_gemm)."""
+    return K % 64 == 0 and F % 128 == 0 and H % 128 == 0
+
+
+def _chain_workspace(dev, stream, nbytes):
+    """A zeroed workspace for stof_gemm_act_gemm, one per (device, stream): every call leaves
+    its workspace zero again, and calls on one stream do not overlap."""
+    key = (dev.index, stream)
+    ws = _chain_ws.get(key)
+    if ws is None or ws.numel() < nbytes:
+        ws = torch.zeros(max(nbytes, 1 << 22), dtype=torch.uint8, device=dev)
+        _chain_ws[key] = ws
+    return ws
+
+
+def gemm_act_gemm(x, W1t, b1, W2t, b2=None, act="gelu", out=None):
+    """act(x @ W1t^T + b1) @ W2t^T (+ b2) in one launch (stof_gemm_act_gemm): x [..., K],
+    W1t [F, K], W2t [H, F]; the [.., F] intermediate is fp16 and stays on chip.  For small row
+    counts; K % 64 == 0, F % 128 == 0, H % 128 == 0."""
+    _require(act in ACT, f"unknown activation {act!r}")
+    _require(x.is_cuda and x.dtype == torch.float16, "x must be a CUDA float16 tensor")
+    W1t = _f16c("W1t", W1t); W2t = _f16c("W2t", W2t)
+    b1 = _f16c("b1", b1, True); b2 = _f16c("b2", b2, True)
+    K = x.shape[-1]
+    F, H = W1t.shape[0], W2t.shape[0]
+    _require(W1t.dim() == 2 and W1t.shape[1] == K, f"W1t must be [F, {K}]")
+    _require(W2t.dim() == 2 and W2t.shape[1] == F, f"W2t must be [H, {F}]")
+    _require(b1 is None or b1.numel() == F, f"b1 must have {F} elements")
+    _require(b2 is None or b2.numel() == H, f"b2 must have {H} elements")
+    x2 = x.reshape(-1, K)
+    if x2.stride(1) != 1:
+        x2 = x2.contiguous()
+    M = x2.shape[0]
+    _require(chain_supported(M, K, F, H), f"unsupported shape for the chained kernel: K {K}, F {F}, H {H}")
+    if out is None:
+        out = torch.empty(x.shape[:-1] + (H,), dtype=torch.float16, device=x.device)
+    o2 = out.view(-1, H)
+    _require(o2.shape[0] == M and o2.stride(1) == 1, "out must be [..., H] with contiguous rows")
+    lib = _lib.lib()
+    st = _stream(o2)
+    nbytes = lib.stof_gemm_act_gemm_workspace_bytes(M, H)
+    ws = _chain_workspace(x.device, st, nbytes)
+    check(lib.stof_gemm_act_gemm(x2.data_ptr(), W1t.data_ptr(), _p(b1), W2t.data_ptr(), _p(b2), o2.data_ptr(),
+                                 M, K, F, H, x2.stride(0), o2.stride(0), ACT[act], ws.data_ptr(), ws.numel(), st),
+          "stof_gemm_act_gemm")
+    return out
+
+
+def triton_matmul_batch(a, b, d, bias, single_launch=None):
     """src/triton_template/gemm_gemm.py:158-174: gelu_tanh(a @ b + bias) @ d, a [B,M,K],
-    b [K,N], d [N,H]; the intermediate is fp16 (gemm_gemm.py:152).  Two launches of the GEMM
-    kernel; the intermediate stays in fp16 as in the reference."""
+    b [K,N], d [N,H]; the intermediate is fp16 (gemm_gemm.py:152).  ``single_launch=True`` (or a
+    row count up to CHAIN_MAX_ROWS) takes the chained kernel that keeps the intermediate on chip;
+    the default is two launches of the GEMM kernel with the fp16 intermediate in HBM, which is
+    the faster form on MI355X at every size measured."""
     _require(a.dim() == 3 and b.dim() == 2 and d.dim() == 2, "a [B,M,K], b [K,N], d [N,H] expected")
-    t = gemm_bias_act(a, pack_weight(b), bias.reshape(-1)[: b.shape[1]], "gelu_tanh")
+    b1 = bias.reshape(-1)[: b.shape[1]]
+    rows = a.shape[0] * a.shape[1]
+    fits = chain_supported(rows, a.shape[2], b.shape[1], d.shape[1])
+    _require(fits or not single_launch, "shape not supported by the single-launch form (K % 64, F % 128, H % 128)")
+    if fits and (single_launch or (single_launch is None and rows <= CHAIN_MAX_ROWS)):
+        return gemm_act_gemm(a, pack_weight(b), b1, pack_weight(d), None, "gelu_tanh")
+    t = gemm_bias_act(a, pack_weight(b), b1, "gelu_tanh")
     return gemm_bias_act(t, pack_weight(d), None, "none")

@@ -23,10 +23,14 @@ from .ops import block_attn
 
 
 class EncoderLayer:
-    def __init__(self, weights, n_heads, eps=1e-12, gelu="erf", ln_fusion="auto"):
+    def __init__(self, weights, n_heads, eps=1e-12, gelu="erf", ln_fusion="auto", ffn_chain="auto"):
         """``weights``: dict with W_qkv [D,3D], b_qkv, W_o [D,D], b_o, g1, be1, W_1 [D,F], b_1,
-        W_2 [F,D], b_2, g2, be2 in the reference's [in, out] orientation, fp16 on the GPU."""
+        W_2 [F,D], b_2, g2, be2 in the reference's [in, out] orientation, fp16 on the GPU.
+        ``ffn_chain``: True / False / "auto" - the two FFN products as one launch with the 4 x hidden
+        intermediate on chip (``fused.gemm_act_gemm``); "auto" takes it up to
+        ``fused.CHAIN_MAX_ROWS`` rows (0 on MI355X: two launches measured faster at every size)."""
         self.n_heads = n_heads
+        self.ffn_chain = ffn_chain
         self.eps = eps
         # FFN activation: erf GELU (BERT, src/benchmk_end2end.py:81), tanh GELU (GPT, :25-26,144), ReLU (T5, :206)
         acts = {"erf": "gelu", "gelu": "gelu", "tanh": "gelu_tanh", "gelu_tanh": "gelu_tanh", "relu": "relu"}
@@ -65,6 +69,20 @@ class EncoderLayer:
         y = fused.gemm_bias_act(x, Wt, None, "none")
         return fused.bias_residual_layernorm(y, bias, residual, gamma, beta, self.eps)
 
+    def _chain(self, M):
+        if self.ffn_chain != "auto":
+            return bool(self.ffn_chain)
+        return (M <= fused.CHAIN_MAX_ROWS and not self._fuse(M) and
+                fused.chain_supported(M, self.hidden, self.W1.shape[0], self.hidden))
+
+    def _ffn(self, h):
+        M = h.numel() // h.shape[-1]
+        if self._chain(M):
+            y = fused.gemm_act_gemm(h, self.W1, self.b1, self.W2, None, self.act)
+            return fused.bias_residual_layernorm(y, self.b2, h, self.g2, self.be2, self.eps)
+        f = fused.gemm_bias_act(h, self.W1, self.b1, self.act)
+        return self._gemm_ln(f, self.W2, self.b2, h, self.g2, self.be2)
+
     def forward(self, x, lut, block=64):
         B, S, D = x.shape
         H = self.n_heads
@@ -73,8 +91,7 @@ class EncoderLayer:
         q, k, v = (qkv[..., t * D:(t + 1) * D].view(B, S, H, hd).permute(0, 2, 1, 3) for t in range(3))
         attn = block_attn(q, k, v, lut, block, block, out_layout="bshd")      # [B,S,D]
         h = self._gemm_ln(attn, self.Wo, self.bo, x, self.g1, self.be1)
-        f = fused.gemm_bias_act(h, self.W1, self.b1, self.act)
-        return self._gemm_ln(f, self.W2, self.b2, h, self.g2, self.be2)
+        return self._ffn(h)
 
     __call__ = forward
 
@@ -103,8 +120,8 @@ class EncoderStack:
     """``layers`` independent EncoderLayers applied in sequence (24 for the BERT-large /
     GPT-2-medium style stack)."""
 
-    def __init__(self, layer_weights, n_heads, eps=1e-12, gelu="erf", ln_fusion="auto"):
-        self.layers = [EncoderLayer(w, n_heads, eps, gelu, ln_fusion) for w in layer_weights]
+    def __init__(self, layer_weights, n_heads, eps=1e-12, gelu="erf", ln_fusion="auto", ffn_chain="auto"):
+        self.layers = [EncoderLayer(w, n_heads, eps, gelu, ln_fusion, ffn_chain) for w in layer_weights]
 
     def forward(self, x, lut, block=64):
         for layer in self.layers:

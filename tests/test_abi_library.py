@@ -76,6 +76,17 @@ def test_other_entry_points_argument_checks(lib):
     assert lib.stof_gemm_bias_act(P, P, None, P, 64, 64, 96, 96, 64, 0, None) == -2      # K % 64
     assert lib.stof_gemm_bias_act(P, P, None, P, 64, 64, 64, 64, 64, 9, None) == -3      # activation
     assert lib.stof_gemm_bias_act(P, P + 8, None, P, 64, 64, 64, 64, 64, 0, None) == -4
+    # chained GEMM + activation + GEMM: X, W1t, b1, W2t, b2, Y, M, K, F, H, ldx, ldy, act, workspace, bytes, stream
+    need = lib.stof_gemm_act_gemm_workspace_bytes(64, 128)
+    assert need >= 64 * 128 * 4 + 4 and lib.stof_gemm_act_gemm_workspace_bytes(0, 128) == 0
+    chain = lambda **kw: lib.stof_gemm_act_gemm(kw.get("X", P), P, None, P, None, P, 64, kw.get("K", 64), kw.get("F", 128),
+                                                kw.get("H", 128), 64, 128, kw.get("act", 1), kw.get("ws", P),
+                                                kw.get("wsb", need), None)
+    assert chain(ws=None) == -1
+    assert chain(K=96) == -2 and chain(F=192) == -2 and chain(H=64) == -2
+    assert chain(wsb=need - 1) == -2       # workspace too small
+    assert chain(act=9) == -3
+    assert chain(X=P + 8) == -4
     assert lib.stof_gemm_bias_res_ln(P, P, None, None, None, None, P, 64, 384, 64, 1e-5, None) == -3   # N
     assert lib.stof_gemm_bias_res_ln(P, P, None, None, None, None, P, 64, 768, 48, 1e-5, None) == -2   # K % 32
     assert lib.stof_rowwise_attn_fwd(P, P, P, P, 7, 0, 0, None, 1, 128, 12, 64, 0, -1, None) == -3
