@@ -19,11 +19,12 @@
 // Meant for small token counts (M <= ~1024), where two separate GEMM launches run at the latency
 // of their K loops on a few dozen workgroups: the chunk split gives M/64 * F/128 workgroups (192
 // at M 512, F 3072) and the second product a K of 128 per workgroup.
-// MEASURED (MI355X, M 512, K 768, F 3072, H 768): 79 us against 31 us for the two launches it
-// replaces (9 + 22 us), so no caller of this library selects it by default.  52 us remain without
-// the atomic adds (one workgroup of four waves per compute unit, a load of 24-32 KB awaited at
-// every step: the K loops run at the load latency) and the 9.4 M fp32 atomic adds (24 partial
-// results per output element) cost the other 27 us, which no pipelining of the loops removes.
+// MEASURED (MI355X, M 512, K 768, F 3072, H 768): 67 us against 31 us for the two launches it
+// replaces (9 + 22 us), so no caller of this library selects it by default.  About 40 us remain
+// without the atomic adds (one workgroup of four waves per compute unit, a load of 24-32 KB
+// awaited at every step: the K loops run at the load latency) and the 9.4 M fp32 atomic adds
+// (24 partial results per output element) cost the other 27 us, which no pipelining of the loops
+// removes.
 // Fewer partial results mean fewer workgroups (F / chunk of them per row block), each streaming
 // more of the 9.4 MB of weights through one compute unit; at this M the split that keeps the
 // intermediate on chip and the parallelism the chip needs exclude each other.
@@ -245,28 +246,29 @@ __global__ __launch_bounds__(256) void ffn_chain_kernel(const ChainParams p) {
   }
 
   // ---- 4. the last workgroup of this row block converts the sums
-  __threadfence();     // this thread's atomic adds are performed before the counter moves
+  // The sums live in device-scope atomics, which do not stay in this XCD's L2, so no cache
+  // write-back is needed before the counter moves (a fence of device scope would write back the
+  // whole L2 once per workgroup: measured 20+ us per launch).  Each thread waits for its own
+  // atomic adds to be acknowledged, the barrier collects the workgroup, then the counter moves.
+  __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0)
   __syncthreads();
   if (threadIdx.x == 0) {
-    const int prev = __hip_atomic_fetch_add(p.counters + mt, 1, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+    const int prev = __hip_atomic_fetch_add(p.counters + mt, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     s_last = (prev == p.chunks - 1);
   }
   __syncthreads();
   if (!s_last) return;
-  __threadfence();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");   // the reader drops what its caches hold of the sums
   const int quads = p.H / 4;
   for (int idx = threadIdx.x; idx < kRows * quads; idx += 256) {
     const int r = idx / quads, c = 4 * (idx % quads);
     const int m = m0 + r;
     if (m >= p.M) break;
     float* src = p.ws + (int64_t)m * p.H + c;
+    const floatx4 v4 = *reinterpret_cast<const floatx4*>(src);
     half4_t o;
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      float v = __hip_atomic_load(src + e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      if (p.b2) v += (float)p.b2[c + e];
-      o[e] = (half_t)v;
-    }
+    for (int e = 0; e < 4; ++e) o[e] = (half_t)(v4[e] + (p.b2 ? (float)p.b2[c + e] : 0.f));
     *reinterpret_cast<half4_t*>(p.Y + (int64_t)m * p.ldy + c) = o;
     *reinterpret_cast<floatx4*>(src) = floatx4{0.f, 0.f, 0.f, 0.f};   // the workspace goes back to zeros for the next call
   }

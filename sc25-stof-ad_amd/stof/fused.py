@@ -156,7 +156,7 @@ def triton_matmul_bias_layernorm(A, B, bias, eps=1e-5):
 
 # Rows up to which "auto" callers take the single-launch chained form.  0: never - measured on
 # MI355X it loses to two GEMM launches at every row count tried (M 256 / 512 / 1024 at K 768,
-# F 3072: 57 / 79 / 123 us against 30 / 31 / 35 us), see csrc/ffn_chain_gfx950.hip.
+# F 3072: 50 / 67 / 101 us against 30 / 31 / 35 us), see csrc/ffn_chain_gfx950.hip.
 CHAIN_MAX_ROWS = 0
 _chain_ws = {}            # (device index, stream handle) -> zeroed workspace tensor, grown on demand
 

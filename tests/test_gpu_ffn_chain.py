@@ -7,7 +7,7 @@ observed max abs error 3.9e-3 at (1, 512, 768, 3072) = one fp16 ulp of results o
 8).  The contributions of the F / 128 chunks are added with fp32 atomics, so two runs may differ
 in the last bit of an fp16 result; comparisons between runs allow one fp16 ulp.
 
-The single-launch form is NOT the faster one on MI355X (79 us against 31 us for two launches at
+The single-launch form is NOT the faster one on MI355X (67 us against 31 us for two launches at
 this size); it is opt-in, and the first test prints both times.
 """
 import pytest
