@@ -853,11 +853,16 @@ __device__ __forceinline__ void attn_group(const AttnParams& p, const int bh, co
       for (int r = 0; r < 16; ++r) oacc[dt][r] = oacc[dt][r] * fa + xo[(16 * dt + r) * 64 + lane] * fb;
   }
 
-  // ---- normalise and store: oacc[dt][r] = O[query j32][d = 32dt + 8(r/4) + 4g + r%4]
+  // ---- normalise and store: oacc[dt][r] = O[query j32][d = 32dt + 8(r/4) + 4g + r%4].  In that
+  // layout a store instruction would write 16 B into each of 32 rows (32 partial cache lines),
+  // so the wave's 32 x 64 block goes through 4 KB of LDS of its own (the tile buffers are free
+  // once every wave has left the walk; 16-byte chunks XOR-ed by the row so that the row-wise
+  // reads are conflict-free) and leaves as 4 stores of 8 full 128-byte rows each.
+  if (KS == 1) __syncthreads();   // (the key split has passed its own barriers above)
   if (!q_valid) return;
   const float l = pair_sum(l_run);
   const float inv = (l > 0.f) ? 1.0f / l : 0.f;   // no allowed key at all: zeros
-  half_t* orow = ob + (int64_t)j32 * p.os[2];
+  lds_byte* stage = (lds_byte*)(KS == 2 ? v_lds1 : (wave < 2 ? k_lds0 : k_lds1)) + (wave & 1) * 4096;   // (key split: waves 0 and 1 are left)
 #pragma unroll
   for (int dt = 0; dt < 2; ++dt)
 #pragma unroll
@@ -865,8 +870,14 @@ __device__ __forceinline__ void attn_group(const AttnParams& p, const int bh, co
       half4_t o4;
 #pragma unroll
       for (int e = 0; e < 4; ++e) o4[e] = to_elem<BF>(oacc[dt][4 * q4 + e] * inv);
-      *reinterpret_cast<half4_t*>(orow + 32 * dt + 8 * q4 + 4 * g) = o4;
+      *reinterpret_cast<__attribute__((address_space(3))) half4_t*>(stage + j32 * 128 + (((4 * dt + q4) ^ (j32 & 7)) << 4) + 8 * g) = o4;
     }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int t = 8 * i + (lane >> 3), c = lane & 7;
+    const half8_t o = *reinterpret_cast<const __attribute__((address_space(3))) half8_t*>(stage + t * 128 + ((c ^ (t & 7)) << 4));
+    *reinterpret_cast<half8_t*>(ob + (int64_t)t * p.os[2] + 8 * c) = o;
+  }
 }
 
 // Workgroups are handed to the 8 XCDs round-robin; give each XCD a contiguous range of
