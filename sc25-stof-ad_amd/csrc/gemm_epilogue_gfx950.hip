@@ -549,9 +549,10 @@ __global__ __launch_bounds__(512) void gemm_bias_res_ln_kernel(const LnGemmParam
 // Which form runs.
 //  * wide ring (256-token tiles, 3 stages) when its grid has at least kWideMinGroups workgroups
 //    (three per compute unit of an MI355X) and K is at least kWideMinK.  Measured at settled
-//    clocks, 8192 tokens: N 3072 K 1024 721 vs 673 TFLOP/s, N 4096 K 1024 706 vs 648, N 1024
-//    K 4096 882 vs 830, 8192^3 951 vs 864; with K 768 (N 3072: 564 vs 598) its longer ring fill
-//    and epilogue per workgroup are not paid back.  Deeper rings (one workgroup per compute
+//    clocks with the line-wise epilogue, 8192 tokens, wide vs 128 x 128: N 3072 K 768 47.5 vs
+//    48.8 us (with GELU 54.4 vs 56.8), N 3072 K 1024 59.3 vs 61.3, N 4096 K 1024 78.6 vs 80.8,
+//    N 1024 K 4096 75.9 vs 75.1; below 768 groups the 128 x 128 form wins (N 2304 K 768: 43.1
+//    vs 39.5 us; 4096 tokens x N 3072: 29.2 vs 27.4).  Deeper rings (one workgroup per compute
 //    unit) measured no faster; a 256 x 256 tile with eight waves gained 3-9 % only from N 4096
 //    up and is not built.
 //  * small ring (64-token tiles, 4 stages) when the 128 x 128 form would have at most
@@ -561,7 +562,7 @@ __global__ __launch_bounds__(512) void gemm_bias_res_ln_kernel(const LnGemmParam
 //  * the 128 x 128 double-buffered form otherwise.
 constexpr int kWideStages = 3;
 constexpr int kWideMinGroups = 768;
-constexpr int kWideMinK = 1024;
+constexpr int kWideMinK = 768;
 constexpr int kSmallStages = 4;
 constexpr int kSmallMaxTiles = 128;
 
