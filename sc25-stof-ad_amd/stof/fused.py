@@ -9,6 +9,7 @@ Reference-named entry points (same signatures as ``src/triton_template``):
 and the explicit forms the encoder layer uses:
 
 * ``gemm_bias_act(x, Wt, bias, act)``                          act(x @ Wt^T + bias)
+* ``gemm_bias_gelu(x, Wt, bias, approximate)``                 the same with torch's name for the GELU variant
 * ``gemm_act_gemm(x, W1t, b1, W2t, b2, act)``                  act(x @ W1t^T + b1) @ W2t^T + b2, one launch
 * ``gemm_bias_residual_layernorm(x, Wt, bias, residual, gamma, beta, eps)``
 * ``bias_residual_layernorm(x, bias, residual, gamma, beta, eps)``
@@ -114,6 +115,13 @@ def gemm_bias_act(x, Wt, bias=None, act="none", out=None):
                                         M, N, K, x2.stride(0), o2.stride(0), ACT[act], _stream(o2)),
           "stof_gemm_bias_act")
     return out
+
+
+def gemm_bias_gelu(x, Wt, bias=None, approximate="none", out=None):
+    """GELU(x @ Wt^T + bias) with torch's naming of the variant: ``approximate`` "none" (erf, BERT,
+    src/benchmk_end2end.py:81) or "tanh" (GPT, :25-26)."""
+    _require(approximate in ("none", "tanh"), f"approximate must be 'none' or 'tanh', got {approximate!r}")
+    return gemm_bias_act(x, Wt, bias, "gelu" if approximate == "none" else "gelu_tanh", out=out)
 
 
 def gemm_bias_residual_layernorm(x, Wt, bias, residual, gamma, beta, eps=1e-5, out=None):

@@ -92,6 +92,15 @@ def test_reference_named_fused_ops():
     _close(got, want, "matmul_batch")
 
 
+def test_gemm_bias_gelu_alias():
+    x = _rand(256, 128, seed=30); W = _rand(128, 256, seed=31, scale=0.05); b = _rand(256, seed=32, scale=0.5)
+    Wt = fused.pack_weight(W.cuda())
+    _close(fused.gemm_bias_gelu(x.cuda(), Wt, b.cuda()), oe.gemm_bias_act(x, W, b, "gelu"), "gelu erf")
+    _close(fused.gemm_bias_gelu(x.cuda(), Wt, b.cuda(), approximate="tanh"), oe.gemm_bias_act(x, W, b, "gelu_tanh"), "gelu tanh")
+    with pytest.raises(StofError):
+        fused.gemm_bias_gelu(x.cuda(), Wt, b.cuda(), approximate="fast")
+
+
 def test_fused_op_errors():
     x = _rand(64, 96, seed=20).cuda(); W = _rand(72, 96, seed=21).cuda()
     with pytest.raises(StofError):
