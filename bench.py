@@ -157,12 +157,12 @@ def bench_layer_c3(steps, warmup):
     maskg = mask.cuda().half()
     lut = pm.get_sparse_storage_batched(mask.float().cuda(), 64, 64)[1:]
     out = {}
-    for fusion in ("auto", "fused", "split"):
+    for fusion in ("auto", "fused", "cluster", "split"):
         layer = EncoderLayer(w, cfg.heads, eps=cfg.eps, ln_fusion=fusion)
         y = layer(x, lut)
         out[fusion + "_ms"], _ = time_region(lambda: layer(x, lut), steps, warmup)
         if fusion == "auto":
-            out["auto_runs"] = "fused" if layer._fuse(cfg.batch * cfg.seq) else "split"
+            out["auto_runs"] = layer._ln_form(cfg.batch * cfg.seq, cfg.hidden)
             y_auto = y
     with torch.no_grad():
         y_eager = eager_layer(x, w, maskg, cfg.heads, cfg.eps)
@@ -253,7 +253,8 @@ def bench_stack_c5(steps, warmup):
         eager_ms, _ = time_region(eager, max(steps // 2, 3), 2)
     gemm_flop = 2 * cfg.batch * cfg.seq * cfg.hidden * (3 * cfg.hidden + cfg.hidden + 2 * cfg.ffn) * cfg.layers
     return {"stack_ms": ms, "ms_per_layer": ms / cfg.layers, "eager_ms": eager_ms, "speedup_vs_eager": eager_ms / ms,
-            "gemm_tflops_at_stack_ms": gemm_flop / ms / 1e9, "layers": cfg.layers, "output_check": check}
+            "gemm_tflops_at_stack_ms": gemm_flop / ms / 1e9, "layers": cfg.layers,
+            "auto_runs": stack.layers[0]._ln_form(cfg.batch * cfg.seq, cfg.hidden), "output_check": check}
 
 
 def bench_dense_vs_sdpa(steps, warmup):

@@ -33,6 +33,7 @@
  *   stof_gemm_bias_res_ln      batch_matmul_bias_layernorm_kernel
  *                                                           src/triton_template/gemm_add_layernorm.py:78-144
  *                              and matmul + bias + residual + F.layer_norm, src/benchmk_end2end.py:73-76
+ *   stof_gemm_bias_res_ln_cluster  the same interfaces (a second launch form of the operator)
  */
 #ifndef STOF_ABI_H
 #define STOF_ABI_H
@@ -258,6 +259,29 @@ int stof_gemm_act_gemm(const void* X, const void* W1t, const void* b1, const voi
 int stof_gemm_bias_res_ln(const void* A, const void* Wt, const void* bias, const void* residual,
                           const void* gamma, const void* beta, void* C,
                           int64_t M, int64_t N, int64_t K, float eps, void* stream);
+
+/*
+ * The same operator as stof_gemm_bias_res_ln (gemm_add_layernorm.py:78-144; benchmk_end2end.py:73-76,
+ * 83-86) on 128 x 128 tiles: the N / 128 workgroups that share a block of 128 token rows
+ * exchange per-row statistics (mean and sum of squared deviations of their 128 columns) through
+ * `workspace`, so the pre-normalisation values still never reach HBM while the grid is N / 128
+ * times larger.  The form for token counts at which one workgroup per 64 rows leaves compute
+ * units idle (8192 tokens at hidden 768 / 1024).
+ * N in {256, 512, 768, 1024}; K % 64 == 0; M <= 2^21; A rows at pitch lda, residual rows at pitch
+ * ldr, C rows at pitch ldc (elements, multiples of 8); A, Wt, residual, C 16-byte aligned.
+ * bias / residual / gamma / beta may be NULL.
+ * workspace: stof_gemm_bias_res_ln_cluster_workspace_bytes(M, N) bytes (0 = shape not supported)
+ * of device memory, 16-byte aligned, that hold ZEROS at the first call; every call leaves them
+ * zero again, so one buffer serves any sequence of calls, of any shapes, that do not overlap in
+ * time (calls sharing a workspace on different streams race).  The first 4 bytes are an error
+ * word: a workgroup whose bounded wait for its partners ran out sets it to 1 (the output is
+ * then invalid); it is never set in normal operation and stays set until the caller clears it.
+ */
+int64_t stof_gemm_bias_res_ln_cluster_workspace_bytes(int64_t M, int64_t N);
+int stof_gemm_bias_res_ln_cluster(const void* A, const void* Wt, const void* bias, const void* residual,
+                                  const void* gamma, const void* beta, void* C,
+                                  int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldr, int64_t ldc,
+                                  float eps, void* workspace, int64_t workspace_bytes, void* stream);
 
 #ifdef __cplusplus
 }

@@ -546,6 +546,306 @@ __global__ __launch_bounds__(512) void gemm_bias_res_ln_kernel(const LnGemmParam
   }
 }
 
+// ------------------------------------------------------------------------------------------
+// The same operator on the 128 x 128 tiles of the bias / activation GEMM: the N / 128 workgroups
+// that share a block of 128 token rows (a "row-block cluster") exchange per-row statistics
+// through a small workspace instead of one workgroup owning the whole row.  The grid then fills
+// the chip at 8192 tokens (hidden 768: 384 workgroups instead of 128) and every workgroup brings
+// in one 128-wide slice of the weights, while the pre-normalisation values still never leave
+// the registers.
+//
+//  * wave (wm, wn) of a workgroup holds 64 token rows x 64 features.  After bias and residual
+//    (requested before the K loop, so their latency is hidden behind it) it forms mean and
+//    M2 = sum (x - mean)^2 of its 64 values per row (two passes in registers) and publishes them
+//    as ONE 8-byte word per row, stats[row block][part = 2 tn + wn][row], whose top bit (the sign
+//    of M2, never set by the arithmetic) says "valid";
+//  * it then reads the words of all 2 N / 128 parts of its rows until every one is valid - the
+//    word itself is the signal, so nothing has to be ordered against anything else -, merges
+//    them (equal counts: mean = average of the means, M2 = sum M2_i + 64 sum (mean_i - mean)^2),
+//    normalises its registers and stores through LDS as full 128-byte lines;
+//  * the words travel as relaxed device-scope atomic stores and loads: these are performed beyond
+//    the XCD's cache, so no cache write-back or invalidate is needed (a device-scope fence would
+//    write back the whole L2 of the XCD once per wave);
+//  * the wait is bounded: after kClusterSpinLimit polls the wave sets the error word of the
+//    workspace and goes on (its output rows are then wrong, the launch still ends).  The cluster's
+//    workgroups are 8 apart in dispatch order - round-robin over the 8 XCDs puts them on one XCD,
+//    where they share the activation rows in L2 - so with in-order dispatch the oldest unfinished
+//    cluster is always resident as a whole and finishes;
+//  * having stored its output, a wave counts itself out of its half row block (64 rows); the
+//    last one to leave puts the half's words and the counter back to zero, so the workspace
+//    serves the next call as it is.
+// ------------------------------------------------------------------------------------------
+struct LnClusterParams {
+  const half_t* A; const half_t* W; const half_t* bias; const half_t* res;
+  const half_t* gamma; const half_t* beta; half_t* C;
+  unsigned long long* stats;   // [tiles_m][2 * tiles_n][128] packed (mean, M2 | valid)
+  int* departed;               // [tiles_m * 2]
+  int* error;
+  int M, N, K; int lda, ldr, ldc; float eps; float inv_n;
+  int tiles_m, tiles_n;
+};
+
+constexpr int kClusterSpinLimit = 1 << 18;
+constexpr unsigned long long kStatsValid = 1ull << 63;
+
+template <int NT>   // NT = N / 128 workgroups per row block
+__global__ __launch_bounds__(256) void gemm_bias_res_ln_cluster_kernel(const LnClusterParams p) {
+  __shared__ __attribute__((aligned(1024))) unsigned char a_lds0[kGTile];
+  __shared__ __attribute__((aligned(1024))) unsigned char a_lds1[kGTile];
+  __shared__ __attribute__((aligned(1024))) unsigned char w_lds0[kGTile];
+  __shared__ __attribute__((aligned(1024))) unsigned char w_lds1[kGTile];
+  constexpr int kParts = 2 * NT;
+
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
+  const int j32 = lane & 31, g = lane >> 5;
+  const int wm = wave >> 1, wn = wave & 1;
+
+  // dispatch index -> (XCD x, i): the NT workgroups of a row block are consecutive on one XCD
+  const int x = blockIdx.x & 7, i = blockIdx.x >> 3;
+  const int tn = i % NT;
+  const int tm = (i / NT) * 8 + x;
+  if (tm >= p.tiles_m) return;   // (a whole cluster at a time: nobody waits for these)
+  const int m0 = tm * kGT, n0 = tn * kGT;
+  const int nb = n0 + 64 * wn;   // first feature of this wave
+
+  // Bias of this lane's columns, in the accumulator layout
+  // acc[ni][mi][r] = X[m0 + 64 wm + 32 mi + j32][nb + 32 ni + 8 (r / 4) + 4 g + r % 4]
+  // (requested inside the K loop, so that neither the first tile's wait nor the epilogue sees
+  // the latency).
+  half4_t bv[2][4];
+  auto request_bias = [&]() {
+#pragma unroll
+    for (int ni = 0; ni < 2; ++ni)
+#pragma unroll
+      for (int q4 = 0; q4 < 4; ++q4) {
+        bv[ni][q4] = half4_t{(half_t)0.f, (half_t)0.f, (half_t)0.f, (half_t)0.f};
+        if (p.bias) bv[ni][q4] = *reinterpret_cast<const half4_t*>(p.bias + nb + 32 * ni + 8 * q4 + 4 * g);
+      }
+  };
+  // The residual tile (128 rows x 256 B) comes in like one more operand tile: as full lines,
+  // direct to LDS, into the stage that the last K tile does not use, while that tile is being
+  // multiplied.  (Read from global memory in the accumulator layout it would be 8 bytes out of
+  // each of 32 rows per instruction, on the address path that already limits the K loop: measured
+  // +3 us on the 8192 x 768 x 768 product.)  Rows 0-63 go to the stage's A buffer, rows 64-127 to
+  // its W buffer; 16-byte chunk c of row r sits at chunk position c ^ (r & 15).
+  auto issue_residual = [&](lds_byte* ad, lds_byte* wd) {
+    if (!p.res) return;
+    lds_byte* dst = (wave < 2 ? ad : wd) + (wave & 1) * 8192;
+#pragma unroll
+    for (int t = 0; t < 8; ++t) {
+      const int row = 32 * wave + 4 * t + (lane >> 4);
+      const int chunk = (lane & 15) ^ (row & 15);
+      const int m = min(m0 + row, p.M - 1);
+      dma16(p.res + (int64_t)m * p.ldr + n0 + 8 * chunk, dst + t * 1024);
+    }
+  };
+
+  const half_t* a_src[4]; const half_t* w_src[4];
+#pragma unroll
+  for (int ii = 0; ii < 4; ++ii) {
+    const int trow = 8 * (4 * wave + ii) + (lane >> 3);
+    const int chunk = (lane & 7) ^ swz(trow);
+    const int am = min(m0 + trow, p.M - 1);       // rows past the edge re-read the last row
+    a_src[ii] = p.A + (int64_t)am * p.lda + 8 * chunk;
+    w_src[ii] = p.W + (int64_t)(n0 + trow) * p.K + 8 * chunk;
+  }
+  auto issue = [&](int kt, lds_byte* ad, lds_byte* wd) {
+#pragma unroll
+    for (int ii = 0; ii < 4; ++ii) dma16(a_src[ii] + kt * kGK, ad + (4 * wave + ii) * 1024);
+#pragma unroll
+    for (int ii = 0; ii < 4; ++ii) dma16(w_src[ii] + kt * kGK, wd + (4 * wave + ii) * 1024);
+  };
+  int rd[4];
+#pragma unroll
+  for (int ks = 0; ks < 4; ++ks) rd[ks] = j32 * 128 + (((2 * ks + g) ^ swz(j32)) << 4);
+
+  floatx16 acc[2][2];   // [feature tile ni][token tile mi]
+#pragma unroll
+  for (int a = 0; a < 2; ++a)
+#pragma unroll
+    for (int b = 0; b < 2; ++b)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.f;
+
+  auto compute = [&](const lds_byte* at, const lds_byte* wt) {
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+      half8_t xa[2], wb[2];
+#pragma unroll
+      for (int mi = 0; mi < 2; ++mi) xa[mi] = lds_frag(at, (64 * wm + 32 * mi) * 128 + rd[ks]);
+#pragma unroll
+      for (int ni = 0; ni < 2; ++ni) wb[ni] = lds_frag(wt, (64 * wn + 32 * ni) * 128 + rd[ks]);
+#pragma unroll
+      for (int ni = 0; ni < 2; ++ni)
+#pragma unroll
+        for (int mi = 0; mi < 2; ++mi) acc[ni][mi] = mfma32(wb[ni], xa[mi], acc[ni][mi]);
+    }
+  };
+
+  const int nk = p.K / kGK;
+  const int res_at = nk > 2 ? 2 : 0;
+  issue(0, (lds_byte*)a_lds0, (lds_byte*)w_lds0);
+  for (int kt = 0; kt < nk; kt += 2) {
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+    __syncthreads();
+    if (kt + 1 < nk) issue(kt + 1, (lds_byte*)a_lds1, (lds_byte*)w_lds1);
+    else issue_residual((lds_byte*)a_lds1, (lds_byte*)w_lds1);   // tile kt is the last one
+    if (kt == res_at) request_bias();
+    compute((const lds_byte*)a_lds0, (const lds_byte*)w_lds0);
+    if (kt + 1 < nk) {   // (no early exit from the loop: a second exit makes the compiler copy the accumulators)
+      __builtin_amdgcn_s_waitcnt(0x0F70);
+      __syncthreads();
+      if (kt + 2 < nk) issue(kt + 2, (lds_byte*)a_lds0, (lds_byte*)w_lds0);
+      else issue_residual((lds_byte*)a_lds0, (lds_byte*)w_lds0);   // tile kt + 1 is the last one
+      compute((const lds_byte*)a_lds1, (const lds_byte*)w_lds1);
+    }
+  }
+  // The residual sits in the stage that did not hold the last tile; the other stage, free after
+  // the barrier below, becomes the staging area of the output.
+  const bool last_in_0 = (nk & 1) != 0;
+  const lds_byte* res_lds = (const lds_byte*)(last_in_0 ? (wm ? w_lds1 : a_lds1) : (wm ? w_lds0 : a_lds0));
+  lds_byte* stage = (lds_byte*)(last_in_0 ? a_lds0 : a_lds1) + wave * 4096;
+  __builtin_amdgcn_s_waitcnt(0x0F70);   // this wave's share of the residual tile has landed
+  __syncthreads();   // every wave is done with the operand tiles: they become the store staging
+
+  // ---- bias + residual; statistics of this wave's 64 features per row
+  float wmean[2], wm2[2];
+#pragma unroll
+  for (int mi = 0; mi < 2; ++mi) {
+    half4_t rv[2][4];
+#pragma unroll
+    for (int ni = 0; ni < 2; ++ni)
+#pragma unroll
+      for (int q4 = 0; q4 < 4; ++q4) {
+        const int rowl = 32 * mi + j32, c = 8 * wn + 4 * ni + q4;
+        rv[ni][q4] = half4_t{(half_t)0.f, (half_t)0.f, (half_t)0.f, (half_t)0.f};
+        if (p.res) rv[ni][q4] = *reinterpret_cast<const __attribute__((address_space(3))) half4_t*>(res_lds + rowl * 256 + ((c ^ (rowl & 15)) << 4) + 8 * g);
+      }
+    float s = 0.f;
+#pragma unroll
+    for (int ni = 0; ni < 2; ++ni)
+#pragma unroll
+      for (int q4 = 0; q4 < 4; ++q4)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const float v = acc[ni][mi][4 * q4 + e] + (float)bv[ni][q4][e] + (float)rv[ni][q4][e];
+          acc[ni][mi][4 * q4 + e] = v;
+          s += v;
+        }
+    wmean[mi] = pair_sum(s) * (1.0f / 64.0f);
+    float d2 = 0.f;
+#pragma unroll
+    for (int ni = 0; ni < 2; ++ni)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) { const float d = acc[ni][mi][r] - wmean[mi]; d2 += d * d; }
+    wm2[mi] = pair_sum(d2);
+  }
+
+  // ---- publish; lane (j32, g) speaks for row 64 wm + 32 g + j32 of the row block
+  const int row_l = 64 * wm + 32 * g + j32;
+  unsigned long long* my_stats = p.stats + ((int64_t)tm * kParts) * kGT + row_l;
+  {
+    const float pm = g ? wmean[1] : wmean[0], pq = g ? wm2[1] : wm2[0];
+    const unsigned long long word = ((unsigned long long)__builtin_bit_cast(unsigned, pq) << 32) | __builtin_bit_cast(unsigned, pm);
+    __hip_atomic_store(my_stats + (int64_t)(2 * tn + wn) * kGT, word | kStatsValid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+  // gamma and beta are requested here: they arrive while the wave waits for the other parts
+  half4_t gv[2][4], tv[2][4];
+#pragma unroll
+  for (int ni = 0; ni < 2; ++ni)
+#pragma unroll
+    for (int q4 = 0; q4 < 4; ++q4) {
+      const int n = nb + 32 * ni + 8 * q4 + 4 * g;
+      gv[ni][q4] = half4_t{(half_t)1.f, (half_t)1.f, (half_t)1.f, (half_t)1.f};
+      tv[ni][q4] = half4_t{(half_t)0.f, (half_t)0.f, (half_t)0.f, (half_t)0.f};
+      if (p.gamma) gv[ni][q4] = *reinterpret_cast<const half4_t*>(p.gamma + n);
+      if (p.beta) tv[ni][q4] = *reinterpret_cast<const half4_t*>(p.beta + n);
+    }
+
+  // ---- collect the parts of this lane's row: read all of them until all are valid
+  unsigned long long word[kParts];
+  {
+    int polls = 0;
+    for (;;) {
+      bool ok = true;
+#pragma unroll
+      for (int pt = 0; pt < kParts; ++pt) {
+        word[pt] = __hip_atomic_load(my_stats + (int64_t)pt * kGT, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        ok = ok && (word[pt] & kStatsValid) != 0;
+      }
+      if (!__any(!ok)) break;
+      if (++polls >= kClusterSpinLimit) {
+        if (lane == 0) __hip_atomic_store(p.error, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        break;
+      }
+      __builtin_amdgcn_s_sleep(4);
+    }
+  }
+  float mean_own = 0.f, m2 = 0.f;
+#pragma unroll
+  for (int pt = 0; pt < kParts; ++pt) {
+    mean_own += __builtin_bit_cast(float, (unsigned)(word[pt] & 0xffffffffull));
+    m2 += __builtin_bit_cast(float, (unsigned)((word[pt] & ~kStatsValid) >> 32));
+  }
+  mean_own *= 1.0f / (float)kParts;
+  float spread = 0.f;
+#pragma unroll
+  for (int pt = 0; pt < kParts; ++pt) {
+    const float d = __builtin_bit_cast(float, (unsigned)(word[pt] & 0xffffffffull)) - mean_own;
+    spread += d * d;
+  }
+  m2 += 64.0f * spread;
+  const float rstd_own = 1.0f / sqrtf(m2 * p.inv_n + p.eps);
+  const float mean_other = xchg32(mean_own), rstd_other = xchg32(rstd_own);
+  float mean[2], rstd[2];
+  mean[0] = g ? mean_other : mean_own; mean[1] = g ? mean_own : mean_other;
+  rstd[0] = g ? rstd_other : rstd_own; rstd[1] = g ? rstd_own : rstd_other;
+
+  // ---- normalise and store: each 32 x 64 block through 4 KB of LDS of the wave's own, out as
+  // full 128-byte lines (see store_wave_block)
+#pragma unroll
+  for (int mi = 0; mi < 2; ++mi) {
+#pragma unroll
+    for (int ni = 0; ni < 2; ++ni)
+#pragma unroll
+      for (int q4 = 0; q4 < 4; ++q4) {
+        half4_t o;
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          o[e] = (half_t)((acc[ni][mi][4 * q4 + e] - mean[mi]) * rstd[mi] * (float)gv[ni][q4][e] + (float)tv[ni][q4][e]);
+        *reinterpret_cast<__attribute__((address_space(3))) half4_t*>(stage + j32 * 128 + (((4 * ni + q4) ^ (j32 & 7)) << 4) + 8 * g) = o;
+      }
+#pragma unroll
+    for (int ii = 0; ii < 4; ++ii) {
+      const int t = 8 * ii + (lane >> 3), c = lane & 7;
+      const half8_t o = *reinterpret_cast<const __attribute__((address_space(3))) half8_t*>(stage + t * 128 + ((c ^ (t & 7)) << 4));
+      const int m = m0 + 64 * wm + 32 * mi + t;
+      if (m < p.M) *reinterpret_cast<half8_t*>(p.C + (int64_t)m * p.ldc + nb + 8 * c) = o;
+    }
+  }
+
+  // ---- leave; the last wave of the half row block zeroes its words and the counter.  (Every
+  // wave that counts itself out has read all the parts, so nobody reads them after this.)
+  int* dep = p.departed + (2 * tm + wm);
+  int prev = 0;
+  if (lane == 0) prev = __hip_atomic_fetch_add(dep, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  prev = __builtin_amdgcn_readfirstlane(prev);
+  if (prev == kParts - 1) {
+#pragma unroll
+    for (int pt = 0; pt < kParts; ++pt)
+      __hip_atomic_store(my_stats + (int64_t)pt * kGT, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (lane == 0) __hip_atomic_store(dep, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+}
+
+// Workspace: error word (first 16 bytes), the counters of kClusterMaxRows / 128 row blocks, then
+// the statistics.  The counter area has one size for every problem, so that a workspace that has
+// served one shape can serve any other.  All of it is zero between calls.
+constexpr int64_t kClusterMaxRows = 1 << 21;
+constexpr int64_t kClusterStatsOffset = 16 + (kClusterMaxRows / kGT) * 8 + 240;   // a multiple of 256
+static_assert(kClusterStatsOffset % 256 == 0, "statistics start on a 256-byte boundary");
+
 // Which form runs.
 //  * wide ring (256-token tiles, 3 stages) when its grid has at least kWideMinGroups workgroups
 //    (three per compute unit of an MI355X) and K is at least kWideMinK.  Measured at settled
@@ -632,6 +932,46 @@ extern "C" int stof_gemm_bias_res_ln(const void* A, const void* Wt, const void* 
     case 512: hipLaunchKernelGGL(gemm_bias_res_ln_kernel<2>, grid, block, 0, st, p); break;
     case 768: hipLaunchKernelGGL(gemm_bias_res_ln_kernel<3>, grid, block, 0, st, p); break;
     default: hipLaunchKernelGGL(gemm_bias_res_ln_kernel<4>, grid, block, 0, st, p); break;
+  }
+  return stof_check_launch();
+}
+
+extern "C" int64_t stof_gemm_bias_res_ln_cluster_workspace_bytes(int64_t M, int64_t N) {
+  if (M <= 0 || M > kClusterMaxRows || N <= 0 || N % kGT != 0) return 0;
+  return kClusterStatsOffset + ((M + kGT - 1) / kGT) * (2 * (N / kGT)) * kGT * 8;
+}
+
+extern "C" int stof_gemm_bias_res_ln_cluster(const void* A, const void* Wt, const void* bias, const void* residual,
+                                             const void* gamma, const void* beta, void* C,
+                                             int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldr, int64_t ldc,
+                                             float eps, void* workspace, int64_t workspace_bytes, void* stream) {
+  if (!A || !Wt || !C || !workspace) return STOF_ERR_NULL_POINTER;
+  if (M <= 0 || K <= 0 || K % kGK != 0 || M > kClusterMaxRows || K > (1 << 30) || lda < K || ldc < N || (residual && ldr < N))
+    return STOF_ERR_BAD_SHAPE;
+  if (N != 256 && N != 512 && N != 768 && N != 1024) return STOF_ERR_UNSUPPORTED;
+  if (!stof_aligned16(A) || !stof_aligned16(Wt) || !stof_aligned16(C) || ((uintptr_t)bias & 7) ||
+      !stof_aligned16(residual) || ((uintptr_t)gamma & 7) || ((uintptr_t)beta & 7) || ((uintptr_t)workspace & 15) ||
+      lda % 8 != 0 || ldc % 8 != 0 || ldr % 8 != 0)
+    return STOF_ERR_MISALIGNED;
+  if (workspace_bytes < stof_gemm_bias_res_ln_cluster_workspace_bytes(M, N)) return STOF_ERR_BAD_SHAPE;
+  LnClusterParams p;
+  p.A = (const half_t*)A; p.W = (const half_t*)Wt; p.bias = (const half_t*)bias; p.res = (const half_t*)residual;
+  p.gamma = (const half_t*)gamma; p.beta = (const half_t*)beta; p.C = (half_t*)C;
+  p.tiles_m = (int)((M + kGT - 1) / kGT); p.tiles_n = (int)(N / kGT);
+  p.error = reinterpret_cast<int*>(workspace);
+  p.departed = p.error + 4;
+  p.stats = reinterpret_cast<unsigned long long*>(reinterpret_cast<char*>(workspace) + kClusterStatsOffset);
+  p.M = (int)M; p.N = (int)N; p.K = (int)K; p.lda = (int)lda; p.ldr = (int)ldr; p.ldc = (int)ldc;
+  p.eps = eps; p.inv_n = 1.0f / (float)N;
+  const int64_t groups = (int64_t)((p.tiles_m + 7) / 8) * 8 * p.tiles_n;
+  if (groups > (1 << 30)) return STOF_ERR_BAD_SHAPE;
+  const dim3 grid((unsigned)groups), block(256);
+  hipStream_t st = (hipStream_t)stream;
+  switch (p.tiles_n) {
+    case 2: hipLaunchKernelGGL(gemm_bias_res_ln_cluster_kernel<2>, grid, block, 0, st, p); break;
+    case 4: hipLaunchKernelGGL(gemm_bias_res_ln_cluster_kernel<4>, grid, block, 0, st, p); break;
+    case 6: hipLaunchKernelGGL(gemm_bias_res_ln_cluster_kernel<6>, grid, block, 0, st, p); break;
+    default: hipLaunchKernelGGL(gemm_bias_res_ln_cluster_kernel<8>, grid, block, 0, st, p); break;
   }
   return stof_check_launch();
 }

@@ -39,6 +39,9 @@ _SIGNATURES = {
     "stof_gemm_act_gemm": (c_int, [_P, _P, _P, _P, _P, _P, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64,
                                    c_int, _P, c_int64, _P]),
     "stof_gemm_bias_res_ln": (c_int, [_P, _P, _P, _P, _P, _P, _P, c_int64, c_int64, c_int64, c_float, _P]),
+    "stof_gemm_bias_res_ln_cluster_workspace_bytes": (c_int64, [c_int64, c_int64]),
+    "stof_gemm_bias_res_ln_cluster": (c_int, [_P, _P, _P, _P, _P, _P, _P, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64,
+                                              c_float, _P, c_int64, _P]),
 }
 
 

@@ -124,8 +124,41 @@ def gemm_bias_gelu(x, Wt, bias=None, approximate="none", out=None):
     return gemm_bias_act(x, Wt, bias, "gelu" if approximate == "none" else "gelu_tanh", out=out)
 
 
-def gemm_bias_residual_layernorm(x, Wt, bias, residual, gamma, beta, eps=1e-5, out=None):
-    """LN(x @ Wt^T + bias + residual) * gamma + beta with the row owned by one workgroup."""
+_cluster_ws = {}          # (device index, stream handle) -> zeroed workspace tensor, grown on demand
+
+
+def cluster_supported(N, K):
+    """Shapes the row-block-cluster form of the LayerNorm GEMM takes."""
+    return N in (256, 512, 768, 1024) and K % 64 == 0
+
+
+def _cluster_workspace(dev, stream, nbytes):
+    """Workspace of stof_gemm_bias_res_ln_cluster, one per (device, stream): its counters start
+    as zeros and every call leaves them zero again; calls on one stream do not overlap."""
+    key = (dev.index, stream)
+    ws = _cluster_ws.get(key)
+    if ws is None or ws.numel() < nbytes:
+        ws = torch.zeros(max(nbytes, 1 << 21), dtype=torch.uint8, device=dev)
+        _cluster_ws[key] = ws
+    return ws
+
+
+def cluster_exchange_failed(dev=None):
+    """True if a wait inside any cluster-form launch on ``dev`` ran out (its output is then
+    invalid): the first word of the workspace.  Synchronises the device; for tests and debugging."""
+    dev = torch.device("cuda", torch.cuda.current_device()) if dev is None else torch.device(dev)
+    torch.cuda.synchronize(dev)
+    return any(bool(ws[:4].view(torch.int32).item()) for (d, _), ws in _cluster_ws.items() if d == dev.index)
+
+
+def gemm_bias_residual_layernorm(x, Wt, bias, residual, gamma, beta, eps=1e-5, out=None, form="row"):
+    """LN(x @ Wt^T + bias + residual) * gamma + beta; the pre-normalisation values stay on chip.
+
+    ``form="row"``: one workgroup owns the whole row of N features (stof_gemm_bias_res_ln).
+    ``form="cluster"``: the N / 128 workgroups of a block of 128 token rows each own 128 features
+    and exchange per-row statistics through a small workspace (stof_gemm_bias_res_ln_cluster):
+    the form for token counts at which one workgroup per 64 rows leaves compute units idle."""
+    _require(form in ("row", "cluster"), f"unknown form {form!r}")
     x = _f16c("x", x); Wt = _f16c("Wt", Wt)
     bias = _f16c("bias", bias, True); residual = _f16c("residual", residual, True)
     gamma = _f16c("gamma", gamma, True); beta = _f16c("beta", beta, True)
@@ -134,10 +167,23 @@ def gemm_bias_residual_layernorm(x, Wt, bias, residual, gamma, beta, eps=1e-5, o
     M = x.numel() // K
     _require(Wt.dim() == 2 and Wt.shape[1] == K, f"Wt must be [N, {K}]")
     _require(residual is None or residual.numel() == M * N, "residual must be [..., N] matching x's rows")
+    for name, t in (("bias", bias), ("gamma", gamma), ("beta", beta)):
+        _require(t is None or t.numel() == N, f"{name} must have {N} elements")
     if out is None:
         out = torch.empty(x.shape[:-1] + (N,), dtype=torch.float16, device=x.device)
-    check(_lib.lib().stof_gemm_bias_res_ln(x.data_ptr(), Wt.data_ptr(), _p(bias), _p(residual),
-                                           _p(gamma), _p(beta), out.data_ptr(), M, N, K, float(eps), _stream(out)),
+    lib = _lib.lib()
+    st = _stream(out)
+    if form == "cluster":
+        _require(cluster_supported(N, K), f"unsupported shape for the cluster form: N {N}, K {K}")
+        nbytes = lib.stof_gemm_bias_res_ln_cluster_workspace_bytes(M, N)
+        ws = _cluster_workspace(x.device, st, nbytes)
+        check(lib.stof_gemm_bias_res_ln_cluster(x.data_ptr(), Wt.data_ptr(), _p(bias), _p(residual), _p(gamma), _p(beta),
+                                                out.data_ptr(), M, N, K, K, N, N, float(eps),
+                                                ws.data_ptr(), ws.numel(), st),
+              "stof_gemm_bias_res_ln_cluster")
+        return out
+    check(lib.stof_gemm_bias_res_ln(x.data_ptr(), Wt.data_ptr(), _p(bias), _p(residual),
+                                    _p(gamma), _p(beta), out.data_ptr(), M, N, K, float(eps), st),
           "stof_gemm_bias_res_ln")
     return out
 

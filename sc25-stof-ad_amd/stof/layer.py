@@ -12,14 +12,20 @@ runs end to end on its own hidden state:
 
 Five launches per layer, no permute / contiguous copies, no standalone elementwise kernels.
 ``ln_fusion`` selects how the two LayerNorm GEMMs run: "fused" = LayerNorm in the GEMM
-epilogue (one workgroup owns the full row), "split" = tiled GEMM followed by the
-bias+residual+LayerNorm kernel.  "auto" is a fixed rule on the shape (the reference likewise
-switches its fused GEMM+LN per shape, data/triton_perf.csv), not a run-time tuner.
+epilogue with one workgroup owning the full row, "cluster" = LayerNorm in the epilogue of the
+128 x 128-tile GEMM, the workgroups of a row block exchanging row statistics, "split" = tiled
+GEMM followed by the bias+residual+LayerNorm kernel.  "auto" is a fixed rule on the shape (the
+reference likewise switches its fused GEMM+LN per shape, data/triton_perf.csv), not a run-time
+tuner.
 """
 import torch
 
 from . import fused
 from .ops import block_attn
+
+
+def _compute_units():
+    return torch.cuda.get_device_properties(torch.cuda.current_device()).multi_processor_count
 
 
 class EncoderLayer:
@@ -47,32 +53,49 @@ class EncoderLayer:
         self.g2, self.be2 = w["g2"].contiguous(), w["be2"].contiguous()
         self.hidden = self.Wo.shape[0]
 
-    def _fuse(self, M):
-        if self.ln_fusion in ("fused", "split"):
-            return self.ln_fusion == "fused"
+    def _ln_form(self, M, K):
+        """How a LayerNorm GEMM of M rows and reduction length K runs: "fused" (one workgroup per
+        64 rows owns the whole row), "cluster" (128 x 128 tiles, the workgroups of a row block
+        exchange row statistics) or "split" (tiled GEMM, then the bias+residual+LayerNorm kernel)."""
+        if self.ln_fusion in ("fused", "cluster", "split"):
+            return self.ln_fusion
+        # Cluster form: its grid of (M / 128) x (hidden / 128) workgroups must fill the chip without
+        # exceeding what is resident at once (two per compute unit), because a workgroup holds its
+        # slot while it waits for its partners.  Measured on MI355X, cluster vs split, 8192 rows:
+        # hidden 768 K 768 / 3072 23.7 vs 28.5 / 55.1 vs 58.8 us, hidden 1024 K 1024 / 4096 32.1 vs
+        # 34.3 / 80.7 vs 85.8 us; at 12288 rows x hidden 768 (1.1 rounds) 108.8 vs 95.6 us.
+        tiles = ((M + 127) // 128) * (self.hidden // 128)
+        if fused.cluster_supported(self.hidden, K) and 192 <= tiles <= 2 * _compute_units():
+            return "cluster"
         # One workgroup per 64 rows streams the whole weight matrix, so the fused kernel needs many
         # row blocks per compute unit (or a small matrix) to beat the tiled GEMM followed by the
-        # LayerNorm kernel.  Measured on MI355X for N = K and N = K / 4: hidden 256 fused wins from
-        # 2048 rows up (10 vs 19 us at 8192); hidden 512 from 32768 rows; hidden 768 / 1024 from
-        # 65536 rows (513 vs 640 us, 915 vs 1188 us at K = 4N), below that the split form wins
-        # (hidden 768, 8192 rows: 41 vs 28 us and 109 vs 60 us).
+        # LayerNorm kernel.  Measured on MI355X for N = K and N = K / 4: hidden 512 from 32768
+        # rows; hidden 768 / 1024 from 65536 rows (513 vs 640 us, 915 vs 1188 us at K = 4N), below
+        # that the split form wins (hidden 768, 8192 rows: 41 vs 28 us and 109 vs 60 us).
         if self.hidden <= 256:
-            return True
+            return "fused" if M >= 32768 or self.hidden < 256 else "split"
         if self.hidden <= 512:
-            return M >= 32768
-        return M >= 65536
+            return "fused" if M >= 32768 else "split"
+        return "fused" if M >= 65536 else "split"
+
+    def pre_ln_stored(self, M):
+        """True if the products that feed the two LayerNorms are stored as fp16 tensors for M token
+        rows (the split form), False if they stay in registers (fused and cluster forms)."""
+        return self._ln_form(M, self.hidden) == "split"
 
     def _gemm_ln(self, x, Wt, bias, residual, gamma, beta):
         M = x.numel() // x.shape[-1]
-        if self._fuse(M):
-            return fused.gemm_bias_residual_layernorm(x, Wt, bias, residual, gamma, beta, self.eps)
-        y = fused.gemm_bias_act(x, Wt, None, "none")
-        return fused.bias_residual_layernorm(y, bias, residual, gamma, beta, self.eps)
+        form = self._ln_form(M, x.shape[-1])
+        if form == "split":
+            y = fused.gemm_bias_act(x, Wt, None, "none")
+            return fused.bias_residual_layernorm(y, bias, residual, gamma, beta, self.eps)
+        return fused.gemm_bias_residual_layernorm(x, Wt, bias, residual, gamma, beta, self.eps,
+                                                  form="cluster" if form == "cluster" else "row")
 
     def _chain(self, M):
         if self.ffn_chain != "auto":
             return bool(self.ffn_chain)
-        return (M <= fused.CHAIN_MAX_ROWS and not self._fuse(M) and
+        return (M <= fused.CHAIN_MAX_ROWS and self._ln_form(M, self.W1.shape[0]) == "split" and
                 fused.chain_supported(M, self.hidden, self.W1.shape[0], self.hidden))
 
     def _ffn(self, h):

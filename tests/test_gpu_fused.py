@@ -167,7 +167,7 @@ def _layer_checks(got, want16, want32, what, fp32_bound, valid=None):
 
 
 @pytest.mark.timeout(300)
-@pytest.mark.parametrize("fusion", ["fused", "split", "auto"])
+@pytest.mark.parametrize("fusion", ["fused", "cluster", "split", "auto"])
 @pytest.mark.parametrize("B", [4, 16])
 def test_encoder_layer_c3(fusion, B):
     """BERT-base layer (hidden 768, 12 heads, FFN 3072, eps 1e-12), per-sample padding x
@@ -179,8 +179,7 @@ def test_encoder_layer_c3(fusion, B):
     lut = pm.get_sparse_storage_batched(mask.float().cuda(), 64, 64)[1:]
     layer = EncoderLayer({k: v.cuda() for k, v in w.items()}, H, eps=1e-12, ln_fusion=fusion)
     got = layer(x.cuda(), lut)
-    runs_fused = layer._fuse(B * S)
-    want16 = oe.bert_layer(x, w, mask.float(), H, eps=1e-12, round_fp16=True if runs_fused else "split")
+    want16 = oe.bert_layer(x, w, mask.float(), H, eps=1e-12, round_fp16="split" if layer.pre_ln_stored(B * S) else True)
     want32 = oe.bert_layer(x, w, mask.float(), H, eps=1e-12)
     valid = torch.arange(S)[None, :] < L[:, None]          # rows past the sample length are don't-care
     _layer_checks(got, want16, want32, f"C3 layer B{B} {fusion}", 5e-3, valid)   # observed 2.9e-3 (B4), 3.3e-3 (B16)
@@ -196,7 +195,7 @@ def test_encoder_layer_gpt_and_t5_activations(act):
     lut = pm.get_sparse_storage(mask[:1].float().cuda(), 64, 64)[1:]
     layer = EncoderLayer({k: v.cuda() for k, v in w.items()}, H, eps=1e-12, gelu=act)
     got = layer(x.cuda(), lut)
-    mode = True if layer._fuse(B * S) else "split"
+    mode = "split" if layer.pre_ln_stored(B * S) else True
     _layer_checks(got, oe.bert_layer(x, w, mask.float(), H, eps=1e-12, gelu=act, round_fp16=mode),
                   oe.bert_layer(x, w, mask.float(), H, eps=1e-12, gelu=act), f"layer {act}", 5e-3)   # observed 3.5e-3
     with pytest.raises(ValueError):
@@ -211,7 +210,7 @@ def test_encoder_stack_two_layers_c5_shape_reduced():
     lut = pm.get_sparse_storage(mask.float().cuda(), 64, 64)[1:]
     stack = EncoderStack([{k: v.cuda() for k, v in w.items()} for w in ws], H, eps=1e-12)
     got = stack(x.cuda(), lut)
-    mode = True if stack.layers[0]._fuse(B * S) else "split"
+    mode = "split" if stack.layers[0].pre_ln_stored(B * S) else True
     want16 = want32 = x
     for w in ws:
         want16 = oe.bert_layer(want16, w, mask.float(), H, eps=1e-12, round_fp16=mode)
@@ -240,7 +239,7 @@ def test_encoder_stack_c5_full_size():
         y = layer(x, lut)
         if i in checked:
             print(f"C5 layer {i + 1}", flush=True)
-            mode = True if layer._fuse(cfg.batch * cfg.seq) else "split"
+            mode = "split" if layer.pre_ln_stored(cfg.batch * cfg.seq) else True
             xin = x.cpu()
             want16 = oe.bert_layer(xin, w, mask.float()[None], cfg.heads, eps=cfg.eps, round_fp16=mode)
             want32 = oe.bert_layer(xin, w, mask.float()[None], cfg.heads, eps=cfg.eps)
@@ -268,7 +267,7 @@ def test_captured_stack_replays_match_eager_launches():
         got = run(x).clone()
         torch.cuda.synchronize()
         assert torch.equal(got, want), f"replay {i} differs from the eager result"
-    mode = True if stack.layers[0]._fuse(B * S) else "split"
+    mode = "split" if stack.layers[0].pre_ln_stored(B * S) else True
     want0 = xs[0].cpu()
     for w in ws:
         want0 = oe.bert_layer(want0, w, mask.float(), H, eps=1e-12, round_fp16=mode)

@@ -1,0 +1,58 @@
+"""GPU parity of the row-block-cluster form of GEMM + bias + residual + LayerNorm against the
+CPU oracle.  Tolerance: |got - want| <= 2e-3 + 1e-2 * |want|."""
+import pytest
+import torch
+
+from oracle import encoder as oe
+from stof import fused
+
+pytestmark = pytest.mark.gpu
+
+
+def _close(got, want, what="", atol=2e-3, rtol=1e-2):
+    got = got.float().cpu(); want = want.float().cpu()
+    assert got.shape == want.shape
+    err = (got - want).abs()
+    bad = err > atol + rtol * want.abs()
+    assert not bool(bad.any()), f"{what}: {int(bad.sum())} out of tolerance, max abs err {float(err.max()):.3e}"
+
+
+def _rand(*shape, seed=0, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(*shape, generator=g) * scale).half()
+
+
+# (8192, 768, 768) / (8192, 768, 3072) / (8192, 1024, 4096): the encoder shapes (one resident round);
+# (1000, 1024, 1024): ragged last row block; (7, 256, 64): a single partly filled cluster;
+# (40000, 512, 128): more clusters than fit on the chip at once (the wait relies on dispatch order);
+# eps 1e-12 with a row offset of 30: statistics that a one-pass variance would lose
+@pytest.mark.parametrize("M,N,K", [(8192, 768, 768), (8192, 768, 3072), (8192, 1024, 4096), (1000, 1024, 1024),
+                                   (7, 256, 64), (40000, 512, 128)])
+@pytest.mark.parametrize("eps", [1e-5, 1e-12])
+def test_gemm_ln_cluster_matches_oracle(M, N, K, eps):
+    print(f"gemm_ln cluster M{M} N{N} K{K} eps{eps}", flush=True)
+    x = _rand(M, K, seed=6); W = _rand(K, N, seed=7, scale=0.05); b = _rand(N, seed=8, scale=0.5)
+    r = _rand(M, N, seed=9); gm = (1 + 0.1 * _rand(N, seed=10).float()).half(); bt = _rand(N, seed=11, scale=0.1)
+    if eps == 1e-12:
+        r = (r.float() + 30.0).half()
+    args = (x.cuda(), fused.pack_weight(W.cuda()), b.cuda(), r.cuda(), gm.cuda(), bt.cuda(), eps)
+    got = fused.gemm_bias_residual_layernorm(*args, form="cluster")
+    assert not fused.cluster_exchange_failed()
+    _close(got, oe.gemm_bias_residual_layernorm(x, W, b, r, gm, bt, eps), "cluster")
+    # a second call on the same workspace (its counters must be back at zero), equal bit for bit
+    again = fused.gemm_bias_residual_layernorm(*args, form="cluster")
+    assert not fused.cluster_exchange_failed()
+    assert torch.equal(got, again)
+
+
+def test_gemm_ln_cluster_optional_operands_and_errors():
+    x = _rand(300, 128, seed=1); W = _rand(128, 256, seed=2, scale=0.1)
+    got = fused.gemm_bias_residual_layernorm(x.cuda(), fused.pack_weight(W.cuda()), None, None, None, None, 1e-5, form="cluster")
+    zero_n, one_n = torch.zeros(256).half(), torch.ones(256).half()
+    _close(got, oe.gemm_bias_residual_layernorm(x, W, zero_n, torch.zeros(300, 256).half(), one_n, zero_n, 1e-5), "no optional operands")
+    with pytest.raises(fused.StofError):
+        fused.gemm_bias_residual_layernorm(x.cuda()[:, :96].contiguous(), fused.pack_weight(W.cuda()[:96]), None, None, None, None,
+                                           1e-5, form="cluster")   # K % 64 != 0
+    Wbad = _rand(128, 384, seed=3)
+    with pytest.raises(fused.StofError):
+        fused.gemm_bias_residual_layernorm(x.cuda(), fused.pack_weight(Wbad.cuda()), None, None, None, None, 1e-5, form="cluster")
