@@ -295,8 +295,7 @@ __global__ __launch_bounds__(256, 2) void gemm_bias_act_ring_kernel(const GemmPa
 
   // Fragment reads are written as asm: the compiler orders LDS reads it can see after every
   // direct-to-LDS load it cannot prove disjoint, which drains the ring.  The ring's own
-  // counter waits cover that dependency; the LDS counter is waited on by hand, fenced so that
-  // nothing that uses a fragment can be scheduled above its wait.
+  // counter waits cover that dependency; the LDS counter is waited on by hand (lds_wait).
   auto frags = [&](uint32_t wa, uint32_t aa, half8_t (&wbk)[2], half8_t (&xak)[MI]) {
     if constexpr (MI == 4) {
       asm volatile(
@@ -319,10 +318,24 @@ __global__ __launch_bounds__(256, 2) void gemm_bias_act_ring_kernel(const GemmPa
           : "v"(wa), "v"(aa));
     }
   };
-  auto lds_wait = [&](bool one_set_in_flight) {   // wait for all fragment reads, or all but the MI + 2 of the latest set
-    __builtin_amdgcn_sched_barrier(0);
-    if (!one_set_in_flight) __builtin_amdgcn_s_waitcnt(0xC07F);   // lgkmcnt(0)
-    else __builtin_amdgcn_s_waitcnt(0xC07F | ((MI + 2) << 8));    // lgkmcnt(MI + 2)
+  // Wait for the fragment reads of one set: all reads (newer_in_flight false) or all but the
+  // MI + 2 reads of the set requested last.  The wait is an asm statement that names the
+  // fragments it covers as read-write operands, so every use of them depends on it and neither
+  // the scheduler nor the register allocator can move a use (or a copy) above the wait.  The LDS
+  // counter is shared with scalar loads, which return out of order: an outstanding one can only
+  // make this wait longer, never shorter, because LDS reads return in order among themselves.
+  auto lds_wait = [&](bool newer_in_flight, half8_t (&wbk)[2], half8_t (&xak)[MI]) {
+    __builtin_amdgcn_sched_barrier(0);   // (keeps the software pipeline in the order written)
+    if constexpr (MI == 4) {
+      if (newer_in_flight) asm volatile("s_waitcnt lgkmcnt(6)" : "+v"(wbk[0]), "+v"(wbk[1]), "+v"(xak[0]), "+v"(xak[1]), "+v"(xak[2]), "+v"(xak[3]));
+      else asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(wbk[0]), "+v"(wbk[1]), "+v"(xak[0]), "+v"(xak[1]), "+v"(xak[2]), "+v"(xak[3]));
+    } else if constexpr (MI == 2) {
+      if (newer_in_flight) asm volatile("s_waitcnt lgkmcnt(4)" : "+v"(wbk[0]), "+v"(wbk[1]), "+v"(xak[0]), "+v"(xak[1]));
+      else asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(wbk[0]), "+v"(wbk[1]), "+v"(xak[0]), "+v"(xak[1]));
+    } else {
+      if (newer_in_flight) asm volatile("s_waitcnt lgkmcnt(3)" : "+v"(wbk[0]), "+v"(wbk[1]), "+v"(xak[0]));
+      else asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(wbk[0]), "+v"(wbk[1]), "+v"(xak[0]));
+    }
     __builtin_amdgcn_sched_barrier(0);
   };
   auto mfmas = [&](const half8_t (&wbk)[2], const half8_t (&xak)[MI]) {
@@ -356,9 +369,9 @@ __global__ __launch_bounds__(256, 2) void gemm_bias_act_ring_kernel(const GemmPa
   for (int t = 0; t < nk; ++t) {
     const int ns = (cs + 1 == NS) ? 0 : cs + 1;
     frags(w_rd + cs * kWTile + rd[1], a_rd + cs * kATile + rd[1], wb1, xa1);
-    lds_wait(true);
+    lds_wait(true, wb0, xa0);
     mfmas(wb0, xa0);
-    lds_wait(false);
+    lds_wait(false, wb1, xa1);
     if (t + 1 < nk) {
       // tiles t+1 .. t+NS-1 are outstanding; all but the first may stay in flight
       if (t + NS - 1 < nk) __builtin_amdgcn_s_waitcnt(vmcnt_imm(kLoads * (NS - 2)));
