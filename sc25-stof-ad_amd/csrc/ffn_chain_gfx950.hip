@@ -50,27 +50,6 @@ __device__ __forceinline__ void dma16(const half_t* src, lds_byte* dst) {
   __builtin_amdgcn_global_load_lds((gptr_t*)src, (__attribute__((address_space(3))) void*)dst, 16, 0, 0);
 }
 
-// erf by Abramowitz-Stegun 7.1.26 (|error| <= 1.5e-7), as in the bias / activation GEMM
-__device__ __forceinline__ float fast_erf(float x) {
-  const float a = fabsf(x);
-  const float t = __builtin_amdgcn_rcpf(__builtin_fmaf(0.3275911f, a, 1.0f));
-  float y = __builtin_fmaf(1.061405429f, t, -1.453152027f);
-  y = __builtin_fmaf(y, t, 1.421413741f);
-  y = __builtin_fmaf(y, t, -0.284496736f);
-  y = __builtin_fmaf(y, t, 0.254829592f);
-  y = y * t * __builtin_amdgcn_exp2f(-1.4426950408889634f * a * a);
-  return copysignf(1.0f - y, x);
-}
-template <int ACT> __device__ __forceinline__ float activate(float x) {
-  if (ACT == STOF_ACT_GELU_ERF) return 0.5f * x * (1.0f + fast_erf(x * 0.70710678118654752f));
-  if (ACT == STOF_ACT_GELU_TANH) {
-    const float u = 0.7978845608028654f * (x + 0.044715f * x * x * x);
-    return x * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-2.8853900817779268f * u));
-  }
-  if (ACT == STOF_ACT_RELU) return fmaxf(x, 0.f);
-  return x;
-}
-
 struct ChainParams {
   const half_t* X; const half_t* W1; const half_t* b1; const half_t* W2; const half_t* b2; half_t* Y;
   float* ws; int* counters;

@@ -25,6 +25,37 @@ __device__ __forceinline__ float wave_sum(float x) {
   return x;
 }
 
+// GELU(x) = x * Phi(x), Phi the standard normal distribution function.  Both variants are
+// evaluated as x * sigmoid(p(x)) = x / (1 + exp2(-log2(e) p(x))) with p an odd polynomial:
+//  * erf form (torch approximate="none"): p(x) = x (a0 + a1 x^2 + a2 x^4), the coefficients a
+//    weighted least-squares fit of x * sigmoid(p(x)) to x * Phi(x) that levels the error over
+//    |x| <= 9: |error| <= 2.6e-5 everywhere (a fifth of the spacing of the fp16 output at the
+//    argument where it peaks, x = -0.56), against 4.7e-4 for the tanh formula.  x^2 is held at
+//    81 (a2 < 0, so p would turn round at |x| = 11; beyond 9 the sigmoid is 0 or 1 in fp32).
+//    One reciprocal, one exp2, seven multiply-adds: half the instructions of an erf evaluation
+//    (Abramowitz-Stegun 7.1.26: 17), which is what the epilogue of the FFN GEMM spends its time on;
+//  * tanh form (approximate="tanh"): 0.5 x (1 + tanh(u)) = x * sigmoid(2u) exactly,
+//    u = sqrt(2/pi) (x + 0.044715 x^3), i.e. p(x) = x (2 sqrt(2/pi) + 2 sqrt(2/pi) 0.044715 x^2).
+__device__ __forceinline__ float stof_gelu_erf(float x) {
+  constexpr float kNegLog2e = -1.4426950408889634f;
+  constexpr float a0 = 1.5950157578067197f, a1 = 0.07401130113566103f, a2 = -0.0007030349551266337f;
+  const float x2 = fminf(x * x, 81.0f);
+  const float q = x * __builtin_fmaf(x2, __builtin_fmaf(x2, kNegLog2e * a2, kNegLog2e * a1), kNegLog2e * a0);
+  return x * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(q));
+}
+__device__ __forceinline__ float stof_gelu_tanh(float x) {
+  constexpr float k0 = -1.4426950408889634f * 2.0f * 0.7978845608028654f;
+  const float q = x * __builtin_fmaf(x * x, k0 * 0.044715f, k0);
+  return x * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(q));
+}
+// Activation selector of the GEMM epilogues (STOF_ACT_*).
+template <int ACT> __device__ __forceinline__ float activate(float x) {
+  if (ACT == STOF_ACT_GELU_ERF) return stof_gelu_erf(x);
+  if (ACT == STOF_ACT_GELU_TANH) return stof_gelu_tanh(x);
+  if (ACT == STOF_ACT_RELU) return fmaxf(x, 0.f);
+  return x;
+}
+
 static inline int stof_check_launch() {
   return hipGetLastError() == hipSuccess ? STOF_OK : STOF_ERR_LAUNCH;
 }

@@ -60,6 +60,22 @@ def test_gemm_strided_rows_and_no_bias():
     _close(fused.gemm_bias_act(x.cuda()[:, :64].contiguous(), ident.cuda(), None, "none"), x[:, :64], "identity")
 
 
+@pytest.mark.parametrize("act,approximate", [("gelu", "none"), ("gelu_tanh", "tanh")])
+def test_gelu_epilogue_pointwise(act, approximate):
+    """The epilogue's GELU on a dense grid of arguments (identity weights, so the product hands x
+    through unchanged): within 4e-5 + one fp16 rounding of torch's fp32 GELU, including the range
+    beyond |x| = 9 where the erf form holds its polynomial argument, and the fp16 extremes."""
+    K = 64
+    grid = torch.linspace(-12, 12, 64 * 1023)
+    x = torch.cat([grid, torch.tensor([-65504., -1000., -40., -11.5, 11.5, 40., 1000., 65504.] * 8)]).half().view(-1, K)
+    ident = torch.eye(K).half()
+    got = fused.gemm_bias_act(x.cuda(), ident.cuda(), None, act).float().cpu()
+    want = torch.nn.functional.gelu(x.float(), approximate=approximate)
+    err = (got - want).abs()
+    bound = 4e-5 + want.abs() * 2.0 ** -11
+    assert bool((err <= bound).all()), f"max excess {float((err - bound).max()):.3e} at x = {float(x.flatten()[int((err - bound).argmax())])}"
+
+
 # ---- GEMM + bias + residual + LayerNorm -------------------------------------------------------
 
 @pytest.mark.parametrize("M,N,K", [(8192, 768, 768), (2048, 768, 3072), (1000, 1024, 1024), (64, 512, 128), (7, 256, 32)])
