@@ -56,3 +56,33 @@ def test_gemm_ln_cluster_optional_operands_and_errors():
     Wbad = _rand(128, 384, seed=3)
     with pytest.raises(fused.StofError):
         fused.gemm_bias_residual_layernorm(x.cuda(), fused.pack_weight(Wbad.cuda()), None, None, None, None, 1e-5, form="cluster")
+
+
+def test_gemm_ln_cluster_in_a_captured_graph():
+    """The cluster form recorded into a HIP graph (workspace allocated and zero-filled by torch
+    inside the capture): every replay, with eager launches and synchronisation between the
+    replays, reproduces the eager result bit for bit."""
+    M, N, K = 4096, 768, 768
+    xs = [_rand(M, K, seed=20 + i).cuda() for i in range(3)]
+    W = fused.pack_weight(_rand(K, N, seed=30, scale=0.05).cuda()); b = _rand(N, seed=31, scale=0.5).cuda()
+    r = _rand(M, N, seed=32).cuda(); gm = (1 + 0.1 * _rand(N, seed=33).float()).half().cuda(); bt = _rand(N, seed=34, scale=0.1).cuda()
+    run = lambda x: fused.gemm_bias_residual_layernorm(x, W, b, r, gm, bt, 1e-12, form="cluster")
+    xin = xs[0].clone()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        run(xin)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        y = run(xin)
+    for i, x in enumerate(xs):
+        print(f"graph replay {i}", flush=True)
+        want = run(x)
+        torch.cuda.synchronize()
+        xin.copy_(x)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(y, want), f"replay {i} differs from the eager result"
+    assert not fused.cluster_exchange_failed()
