@@ -264,17 +264,24 @@ __device__ __forceinline__ void attn_group(const AttnParams& p, const int bh, co
   bool warm = false;       // every lane of the wave has a finite running max
   constexpr float kSumLimit = 16384.f;   // 32 probabilities of at most 2^kLazy sum to 2^13
 
+  // K and V of this (batch, head) as buffer resources: a tile load is then the resource (scalar
+  // registers, set up once), the tile's byte offset (one scalar multiply) and the lane's 32-bit
+  // offset inside a tile - no 64-bit address arithmetic per tile.  The byte span of a head is below
+  // 2^31 (checked by the host), and the resource's extent is that span, so an offset beyond the
+  // tensor would read zeros instead of faulting.
+  const uint32_t k_tile_bytes = (uint32_t)(kBN * 2 * p.ks[2]), v_tile_bytes = (uint32_t)(kBN * 2 * p.vs[2]);
+  const __amdgpu_buffer_rsrc_t k_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<half_t*>(kb), 0, (int)(((int64_t)(p.S - 1) * p.ks[2] + kD) * 2), 0x00020000);
+  const __amdgpu_buffer_rsrc_t v_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<half_t*>(vb), 0, (int)(((int64_t)(p.S - 1) * p.vs[2] + kD) * 2), 0x00020000);
   auto issue_tile = [&](int col, lds_byte* kdst, lds_byte* vdst) {
-    const char* kt = reinterpret_cast<const char*>(kb + (int64_t)col * kBN * p.ks[2]);
-    const char* vt = reinterpret_cast<const char*>(vb + (int64_t)col * kBN * p.vs[2]);
+    const uint32_t kt = (uint32_t)col * k_tile_bytes, vt = (uint32_t)col * v_tile_bytes;
     lds_byte* kd = kdst + (kDma * wave) * 1024;
     lds_byte* vd = vdst + (kDma * wave) * 1024;
 #pragma unroll
     for (int i = 0; i < kDma; ++i)
-      __builtin_amdgcn_global_load_lds((gptr_t*)(kt + k_src[i]), (__attribute__((address_space(3))) void*)(kd + i * 1024), 16, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(k_rsrc, (__attribute__((address_space(3))) void*)(kd + i * 1024), 16, k_src[i], kt, 0, 0);
 #pragma unroll
     for (int i = 0; i < kDma; ++i)
-      __builtin_amdgcn_global_load_lds((gptr_t*)(vt + v_src[i]), (__attribute__((address_space(3))) void*)(vd + i * 1024), 16, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(v_rsrc, (__attribute__((address_space(3))) void*)(vd + i * 1024), 16, v_src[i], vt, 0, 0);
   };
 
   // ---- merged walk over the group's rows, wave-uniform and identical in every wave.
@@ -361,20 +368,19 @@ __device__ __forceinline__ void attn_group(const AttnParams& p, const int bh, co
     // issues the loads of K(i+2) and V(i+1) into the buffers iteration i-1 read last.
     enum { kValid = 1, kMine = 2, kMask = 4 };   // tile flags: listed by the walk, used by this wave's row, needs its element mask
     struct Tile { int col, slot, f; };
-    const uint32_t k_tile_bytes = (uint32_t)(kBN * 2 * p.ks[2]), v_tile_bytes = (uint32_t)(kBN * 2 * p.vs[2]);   // < 2^28: strides_ok
     auto dma_k = [&](int col, lds_byte* kdst) {
-      const char* kt = reinterpret_cast<const char*>(kb) + (uint64_t)(uint32_t)col * k_tile_bytes;
+      const uint32_t kt = (uint32_t)col * k_tile_bytes;
       lds_byte* kd = kdst + (kDma * wave) * 1024;
 #pragma unroll
       for (int i = 0; i < kDma; ++i)
-        __builtin_amdgcn_global_load_lds((gptr_t*)(kt + k_src[i]), (__attribute__((address_space(3))) void*)(kd + i * 1024), 16, 0, 0);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(k_rsrc, (__attribute__((address_space(3))) void*)(kd + i * 1024), 16, k_src[i], kt, 0, 0);
     };
     auto dma_v = [&](int col, lds_byte* vdst) {
-      const char* vt = reinterpret_cast<const char*>(vb) + (uint64_t)(uint32_t)col * v_tile_bytes;
+      const uint32_t vt = (uint32_t)col * v_tile_bytes;
       lds_byte* vd = vdst + (kDma * wave) * 1024;
 #pragma unroll
       for (int i = 0; i < kDma; ++i)
-        __builtin_amdgcn_global_load_lds((gptr_t*)(vt + v_src[i]), (__attribute__((address_space(3))) void*)(vd + i * 1024), 16, 0, 0);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(v_rsrc, (__attribute__((address_space(3))) void*)(vd + i * 1024), 16, v_src[i], vt, 0, 0);
     };
     // element-mask word of this lane's query for a tile (requested when the tile enters the queue)
     auto request_bits = [&](const Tile& t) -> uint64_t {
@@ -1154,6 +1160,10 @@ bool strides_ok(const int64_t s[3]) {
   return (s[0] % 8 == 0) && (s[1] % 8 == 0) && (s[2] % 8 == 0) && s[2] >= kD && s[2] < (1 << 20);
 }
 
+// K and V tiles are addressed with 32-bit byte offsets from the start of their (batch, head):
+// the rows of one head must span less than 2^31 bytes.
+bool span_ok(int64_t seq_len, int64_t row_stride) { return ((seq_len - 1) * row_stride + kD) * 2 < ((int64_t)1 << 31); }
+
 }  // namespace
 
 extern "C" int stof_attn_set_launch_form(int form) {
@@ -1188,6 +1198,7 @@ extern "C" int stof_block_attn_fwd(
   if (!stof_aligned16(q) || !stof_aligned16(k) || !stof_aligned16(v) || !stof_aligned16(out)) return STOF_ERR_MISALIGNED;
   if (!strides_ok(q_strides) || !strides_ok(k_strides) || !strides_ok(v_strides) || !strides_ok(out_strides))
     return STOF_ERR_MISALIGNED;
+  if (!span_ok(seq_len, k_strides[2]) || !span_ok(seq_len, v_strides[2])) return STOF_ERR_BAD_SHAPE;
   if ((int64_t)nQ * batch_size * head_num > (int64_t)1 << 30) return STOF_ERR_BAD_SHAPE;
 
   AttnParams p;
@@ -1218,7 +1229,7 @@ extern "C" int stof_rowwise_attn_fwd(
   if (kind == STOF_ROW_SLIDING && bandwidth <= 0) return STOF_ERR_BAD_SHAPE;
   if (!stof_aligned16(q) || !stof_aligned16(k) || !stof_aligned16(v) || !stof_aligned16(out)) return STOF_ERR_MISALIGNED;
   const int nQ = seq_len / kBM;
-  if ((int64_t)nQ * batch_size * head_num > (int64_t)1 << 30) return STOF_ERR_BAD_SHAPE;
+  if ((int64_t)nQ * batch_size * head_num > (int64_t)1 << 30 || !span_ok(seq_len, kD)) return STOF_ERR_BAD_SHAPE;
   AttnParams p;
   p.q = (const half_t*)q; p.k = (const half_t*)k; p.v = (const half_t*)v; p.out = (half_t*)out;
   p.prp = nullptr; p.pci = nullptr; p.pbits = nullptr; p.lrp = nullptr; p.lci = nullptr;
