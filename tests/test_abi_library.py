@@ -89,6 +89,20 @@ def test_other_entry_points_argument_checks(lib):
     assert chain(X=P + 8) == -4
     assert lib.stof_gemm_bias_res_ln(P, P, None, None, None, None, P, 64, 384, 64, 1e-5, None) == -3   # N
     assert lib.stof_gemm_bias_res_ln(P, P, None, None, None, None, P, 64, 768, 48, 1e-5, None) == -2   # K % 32
+    # cluster form: A, Wt, bias, residual, gamma, beta, C, M, N, K, lda, ldr, ldc, eps, workspace, bytes, stream
+    cneed = lib.stof_gemm_bias_res_ln_cluster_workspace_bytes(8192, 768)
+    assert cneed >= 64 * 12 * 128 * 8 and cneed % 256 == 0
+    assert lib.stof_gemm_bias_res_ln_cluster_workspace_bytes(8192, 384) == 8192 // 128 * 6 * 1024 + lib.stof_gemm_bias_res_ln_cluster_workspace_bytes(128, 128) - 2048
+    assert lib.stof_gemm_bias_res_ln_cluster_workspace_bytes(8192, 100) == 0          # N % 128
+    assert lib.stof_gemm_bias_res_ln_cluster_workspace_bytes((1 << 21) + 1, 768) == 0   # more rows than the counter area holds
+    cl = lambda **kw: lib.stof_gemm_bias_res_ln_cluster(kw.get("A", P), P, None, kw.get("res", None), None, None, P, kw.get("M", 8192),
+                                                        kw.get("N", 768), kw.get("K", 768), kw.get("lda", 768), kw.get("ldr", 768), kw.get("ldc", 768), 1e-5,
+                                                        kw.get("ws", P), kw.get("wsb", cneed), None)
+    assert cl(ws=None) == -1
+    assert cl(K=96) == -2 and cl(lda=512) == -2 and cl(M=(1 << 21) + 1) == -2
+    assert cl(wsb=cneed - 1) == -2          # workspace too small
+    assert cl(N=384) == -3 and cl(N=2048, ldc=2048) == -3
+    assert cl(A=P + 8) == -4 and cl(res=P + 8) == -4 and cl(res=P, ldr=772) == -4
     assert lib.stof_rowwise_attn_fwd(P, P, P, P, 7, 0, 0, None, 1, 128, 12, 64, 0, -1, None) == -3
     assert lib.stof_rowwise_attn_fwd(P, P, P, P, 2, 0, 0, None, 1, 128, 12, 64, 0, -1, None) == -1            # mask kind, no bits
     assert lib.stof_rowwise_attn_fwd(P, P, P, P, 1, 1, 0, None, 1, 128, 12, 64, 0, -1, None) == -2            # band <= 0
