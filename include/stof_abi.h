@@ -278,6 +278,10 @@ int stof_gemm_bias_res_ln(const void* A, const void* Wt, const void* bias, const
  * then invalid); it is never set in normal operation and stays set until the caller clears it.
  */
 int64_t stof_gemm_bias_res_ln_cluster_workspace_bytes(int64_t M, int64_t N);
+/* Number of polls after which a wave of the cluster kernel stops waiting for its partners and sets the
+ * error word (process-wide; 0 restores the default of 2^18, about a tenth of a second).  Meant for
+ * tests of that path: with a limit of 1 a launch ends normally with the error word set. */
+int stof_gemm_bias_res_ln_cluster_set_spin_limit(int polls);
 int stof_gemm_bias_res_ln_cluster(const void* A, const void* Wt, const void* bias, const void* residual,
                                   const void* gamma, const void* beta, void* C,
                                   int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldr, int64_t ldc,

@@ -554,7 +554,7 @@ __global__ __launch_bounds__(512) void gemm_bias_res_ln_kernel(const LnGemmParam
 //  * the words travel as relaxed device-scope atomic stores and loads: these are performed beyond
 //    the XCD's cache, so no cache write-back or invalidate is needed (a device-scope fence would
 //    write back the whole L2 of the XCD once per wave);
-//  * the wait is bounded: after kClusterSpinLimit polls the wave sets the error word of the
+//  * the wait is bounded: after a fixed number of polls (2^18; stof_gemm_bias_res_ln_cluster_set_spin_limit) the wave sets the error word of the
 //    workspace and goes on (its output rows are then wrong, the launch still ends).  The cluster's
 //    workgroups are 8 apart in dispatch order - round-robin over the 8 XCDs puts them on one XCD,
 //    where they share the activation rows in L2 - so with in-order dispatch the oldest unfinished
@@ -570,10 +570,11 @@ struct LnClusterParams {
   int* departed;               // [tiles_m * 2]
   int* error;
   int M, N, K; int lda, ldr, ldc; float eps; float inv_n;
-  int tiles_m, tiles_n;
+  int tiles_m, tiles_n; int spin_limit;
 };
 
-constexpr int kClusterSpinLimit = 1 << 18;
+constexpr int kClusterSpinLimit = 1 << 18;   // default number of polls before a wave gives up
+int g_cluster_spin_limit = kClusterSpinLimit;
 constexpr unsigned long long kStatsValid = 1ull << 63;
 
 template <int NT>   // NT = N / 128 workgroups per row block
@@ -763,7 +764,7 @@ __global__ __launch_bounds__(256) void gemm_bias_res_ln_cluster_kernel(const LnC
         ok = ok && (word[pt] & kStatsValid) != 0;
       }
       if (!__any(!ok)) break;
-      if (++polls >= kClusterSpinLimit) {
+      if (++polls >= p.spin_limit) {
         if (lane == 0) __hip_atomic_store(p.error, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         break;
       }
@@ -929,6 +930,12 @@ extern "C" int64_t stof_gemm_bias_res_ln_cluster_workspace_bytes(int64_t M, int6
   return kClusterStatsOffset + ((M + kGT - 1) / kGT) * (2 * (N / kGT)) * kGT * 8;
 }
 
+extern "C" int stof_gemm_bias_res_ln_cluster_set_spin_limit(int polls) {
+  if (polls < 0) return STOF_ERR_BAD_SHAPE;
+  g_cluster_spin_limit = polls == 0 ? kClusterSpinLimit : polls;
+  return STOF_OK;
+}
+
 extern "C" int stof_gemm_bias_res_ln_cluster(const void* A, const void* Wt, const void* bias, const void* residual,
                                              const void* gamma, const void* beta, void* C,
                                              int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldr, int64_t ldc,
@@ -950,7 +957,7 @@ extern "C" int stof_gemm_bias_res_ln_cluster(const void* A, const void* Wt, cons
   p.departed = p.error + 4;
   p.stats = reinterpret_cast<unsigned long long*>(reinterpret_cast<char*>(workspace) + kClusterStatsOffset);
   p.M = (int)M; p.N = (int)N; p.K = (int)K; p.lda = (int)lda; p.ldr = (int)ldr; p.ldc = (int)ldc;
-  p.eps = eps; p.inv_n = 1.0f / (float)N;
+  p.eps = eps; p.inv_n = 1.0f / (float)N; p.spin_limit = g_cluster_spin_limit;
   const int64_t groups = (int64_t)((p.tiles_m + 7) / 8) * 8 * p.tiles_n;
   if (groups > (1 << 30)) return STOF_ERR_BAD_SHAPE;
   const dim3 grid((unsigned)groups), block(256);

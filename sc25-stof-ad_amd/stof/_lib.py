@@ -40,6 +40,7 @@ _SIGNATURES = {
                                    c_int, _P, c_int64, _P]),
     "stof_gemm_bias_res_ln": (c_int, [_P, _P, _P, _P, _P, _P, _P, c_int64, c_int64, c_int64, c_float, _P]),
     "stof_gemm_bias_res_ln_cluster_workspace_bytes": (c_int64, [c_int64, c_int64]),
+    "stof_gemm_bias_res_ln_cluster_set_spin_limit": (c_int, [c_int]),
     "stof_gemm_bias_res_ln_cluster": (c_int, [_P, _P, _P, _P, _P, _P, _P, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64,
                                               c_float, _P, c_int64, _P]),
 }

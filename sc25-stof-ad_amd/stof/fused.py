@@ -151,6 +151,14 @@ def cluster_exchange_failed(dev=None):
     return any(bool(ws[:4].view(torch.int32).item()) for (d, _), ws in _cluster_ws.items() if d == dev.index)
 
 
+def clear_cluster_exchange_error(dev=None):
+    """Put the error word of every cluster workspace on ``dev`` back to zero."""
+    dev = torch.device("cuda", torch.cuda.current_device()) if dev is None else torch.device(dev)
+    for (d, _), ws in _cluster_ws.items():
+        if d == dev.index:
+            ws[:4].zero_()
+
+
 def gemm_bias_residual_layernorm(x, Wt, bias, residual, gamma, beta, eps=1e-5, out=None, form="row"):
     """LN(x @ Wt^T + bias + residual) * gamma + beta; the pre-normalisation values stay on chip.
 

@@ -86,3 +86,30 @@ def test_gemm_ln_cluster_in_a_captured_graph():
         torch.cuda.synchronize()
         assert torch.equal(y, want), f"replay {i} differs from the eager result"
     assert not fused.cluster_exchange_failed()
+
+
+def test_gemm_ln_cluster_bounded_wait_gives_up_and_recovers():
+    """The wait for the partners is bounded: with a limit of one poll some waves of a launch give up
+    (the kernel still ends normally, the error word is set, the output is not to be used); with the
+    default limit restored and the word cleared the same workspace serves the next call."""
+    from stof import _lib
+    M, N, K = 8192, 768, 768
+    x = _rand(M, K, seed=40); W = _rand(K, N, seed=41, scale=0.05); b = _rand(N, seed=42, scale=0.5)
+    r = _rand(M, N, seed=43); gm = (1 + 0.1 * _rand(N, seed=44).float()).half(); bt = _rand(N, seed=45, scale=0.1)
+    args = (x.cuda(), fused.pack_weight(W.cuda()), b.cuda(), r.cuda(), gm.cuda(), bt.cuda(), 1e-5)
+    want = oe.gemm_bias_residual_layernorm(x, W, b, r, gm, bt, 1e-5)
+    _close(fused.gemm_bias_residual_layernorm(*args, form="cluster"), want, "before")
+    lib = _lib.lib()
+    try:
+        assert lib.stof_gemm_bias_res_ln_cluster_set_spin_limit(1) == 0
+        for _ in range(5):                       # (a single launch in which every wave finds its partners at once is conceivable)
+            fused.gemm_bias_residual_layernorm(*args, form="cluster")
+        torch.cuda.synchronize()                 # the launches end although waves gave up
+        assert fused.cluster_exchange_failed()
+    finally:
+        assert lib.stof_gemm_bias_res_ln_cluster_set_spin_limit(0) == 0
+    fused.clear_cluster_exchange_error()
+    assert not fused.cluster_exchange_failed()
+    _close(fused.gemm_bias_residual_layernorm(*args, form="cluster"), want, "after")
+    assert not fused.cluster_exchange_failed()
+    assert lib.stof_gemm_bias_res_ln_cluster_set_spin_limit(-1) == -2
