@@ -660,6 +660,7 @@ __device__ __forceinline__ void attn_group(const AttnParams& p, const int bh, co
       build_table();
     }
   } else {
+    float raise_at = -INFINITY;   // (running max) * c + kLazy: a tile max above it raises the running max
     // one key block: kt/vt hold the current tile, the next tile's loads go to kn/vn
     auto step = [&](const Step cur, const Step nxt, const lds_byte* kt, const lds_byte* vt, lds_byte* kn, lds_byte* vn) {
       // The row mask of a partial tile is fetched first so that its latency hides behind
@@ -759,12 +760,17 @@ __device__ __forceinline__ void attn_group(const AttnParams& p, const int bh, co
 #pragma unroll
           for (int r = 0; r < 16; ++r) mx = fmaxf(mx, sacc[mt][r]);
         mx = pair_max(mx);
-        const float m_new = (mx * p.c > m_run * p.c + kLazy || m_run == -INFINITY) ? mx : m_run;
+        // Nothing to do unless some lane's tile max exceeds its threshold (running max + kLazy, in
+        // log2 units; -inf for a row that has seen no key, so its first finite score gets here):
+        // one multiply and one compare on the common path.
+        if (!__any(mx * p.c > raise_at)) return;
+        const float m_new = (mx * p.c > raise_at) ? mx : m_run;
         // A row that has seen no allowed key yet has m_new == -inf: subtract 0 instead, so
         // that its probabilities are exp2(-inf) = 0 and no inf - inf appears.
         const float m_sub = (m_new == -INFINITY) ? 0.f : m_new;
         const float alpha = __builtin_amdgcn_exp2f((m_run - m_sub) * p.c);
         mc_run = m_sub * p.c;
+        raise_at = m_new * p.c + kLazy;
         l_run *= alpha;   // per-lane partial sum; the two halves are added at the end
         m_run = m_new;
         if (__any(alpha != 1.0f)) {
@@ -773,7 +779,6 @@ __device__ __forceinline__ void attn_group(const AttnParams& p, const int bh, co
 #pragma unroll
             for (int r = 0; r < 16; ++r) oacc[dt][r] *= alpha;
         }
-        warm = !__any(m_run == -INFINITY);
       };
       half8_t pf[kMT][2];   // [key sub-tile][half]: B operand of O^T = V^T . P^T
       auto probabilities = [&]() -> float {
