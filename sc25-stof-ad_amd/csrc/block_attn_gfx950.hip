@@ -13,7 +13,7 @@
 //    the two 32-key halves of every tile, so the chain of key blocks of a long row, which
 //    sets the run time there, takes half as long; partial results are merged through LDS;
 //  * K/V tiles travel HBM/L2 -> LDS with the asynchronous direct-to-LDS loads
-//    (global_load_lds_dwordx4), double buffered: the loads of block t+1 are issued before
+//    (buffer_load_dwordx4 ... lds), double buffered: the loads of block t+1 are issued before
 //    the math of block t, no VGPRs are used for staging and one barrier per block suffices;
 //  * scores are produced TRANSPOSED, S^T = K . Q^T, with v_mfma_f32_32x32x16_f16.  In the
 //    32x32 accumulator layout a lane holds 32 keys of ONE query (lane & 31), so the
