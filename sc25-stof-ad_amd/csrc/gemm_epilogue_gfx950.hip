@@ -860,22 +860,23 @@ constexpr int64_t kClusterStatsOffset = 16 + (kClusterMaxRows / kGT) * 8 + 240; 
 static_assert(kClusterStatsOffset % 256 == 0, "statistics start on a 256-byte boundary");
 
 // Which form runs.
-//  * wide ring (256-token tiles, 3 stages) when its grid has at least kWideMinGroups workgroups
-//    (three per compute unit of an MI355X) and K is at least kWideMinK.  Measured at settled
-//    clocks with the line-wise epilogue, 8192 tokens, wide vs 128 x 128: N 3072 K 768 47.5 vs
-//    48.8 us (with GELU 54.4 vs 56.8), N 3072 K 1024 59.3 vs 61.3, N 4096 K 1024 78.6 vs 80.8,
-//    N 1024 K 4096 75.9 vs 75.1; below 768 groups the 128 x 128 form wins (N 2304 K 768: 43.1
-//    vs 39.5 us; 4096 tokens x N 3072: 29.2 vs 27.4).  Deeper rings (one workgroup per compute
-//    unit) measured no faster; a 256 x 256 tile with eight waves gained 3-9 % only from N 4096
-//    up and is not built.
+//  * the 128 x 128 double-buffered form for almost everything.  With its tile loads through buffer
+//    resources (no 64-bit vector add per load) it is the fastest form from 4096 to 32768 rows at every
+//    N and K measured, settled clocks, 128 x 128 vs wide ring: 8192 rows N 3072 K 768 45.8 vs 48.0 us,
+//    N 2304 K 768 36.2 vs 41.4, N 4096 K 1024 75.3 vs 76.5, N 1024 K 4096 67.3 vs 73.3, 8192^3 1042
+//    vs 1095 us (1055 TFLOP/s), 16384 x 4096 x 4096 547 vs 562 us;
+//  * wide ring (256-token tiles, 3 stages) from kWideMinRows rows on, when its grid has at least
+//    kWideMinGroups workgroups and K is at least kWideMinK: 65536 rows x N 3072 x K 768 433 vs 470 us
+//    (at 32768 rows the two tie: 187 vs 185 us).  Before the buffer-resource loads it was the form
+//    for every grid of 768+ workgroups (+3-8 %);
 //  * small ring (64-token tiles, 4 stages) when the 128 x 128 form would have at most
 //    kSmallMaxTiles workgroups.  GPU time, N x K of the BERT-base layer: 512 tokens 14.4 -> 8.9,
 //    14.0 -> 8.4, 14.5 -> 10.6, 36.0 -> 22.9 us; 2048 tokens x N 768: 14.2 -> 8.9, 36.9 -> 23.2 us;
 //    from 192 tiles on (4096 tokens x N 768, 2048 x N 2304) the two are within 5 % either way.
-//  * the 128 x 128 double-buffered form otherwise.
 constexpr int kWideStages = 3;
 constexpr int kWideMinGroups = 768;
 constexpr int kWideMinK = 768;
+constexpr int kWideMinRows = 49152;
 constexpr int kSmallStages = 4;
 constexpr int kSmallMaxTiles = 128;
 
@@ -910,7 +911,7 @@ extern "C" int stof_gemm_bias_act(const void* A, const void* Wt, const void* bia
   p.M = (int)M; p.N = (int)N; p.K = (int)K; p.lda = (int)lda; p.ldc = (int)ldc;
   hipStream_t st = (hipStream_t)stream;
   const int64_t wide_groups = ((M + kWTok - 1) / kWTok) * ((N + kWFeat - 1) / kWFeat);
-  if (wide_groups >= kWideMinGroups && K >= kWideMinK) return launch_ring<kWideStages, 4>(p, act, st);
+  if (wide_groups >= kWideMinGroups && K >= kWideMinK && M >= kWideMinRows) return launch_ring<kWideStages, 4>(p, act, st);
   const int64_t tiles128 = ((M + kGT - 1) / kGT) * ((N + kGT - 1) / kGT);
   if (tiles128 <= kSmallMaxTiles) return launch_ring<kSmallStages, 1>(p, act, st);
   p.tiles_m = (int)((M + kGT - 1) / kGT); p.tiles_n = (int)((N + kGT - 1) / kGT);

@@ -29,14 +29,15 @@ def _rand(*shape, seed=0, scale=1.0):
 # ---- GEMM + bias + activation -----------------------------------------------------------------
 
 # Three launch forms behind one entry point:
-#  wide ring (grids of 768+ workgroups of 256 x 128, K >= 1024): (8192, 3072, 1024) full tiles,
-#    (8155, 3080, 1024) ragged token / feature edges, (8292, 3072, 1088) a K loop whose length is not
-#    a multiple of the ring depth;
-#  128 x 128 double-buffered: (8192, 3072, 768) has the grid of the wide form but not the K,
-#    (2100, 2312, 192) ragged edges on both sides;
+#  128 x 128 double-buffered (the default): (8192, 3072, 1024) and (8192, 3072, 768) full tiles at the
+#    encoder's shapes, (8155, 3080, 1024) and (2100, 2312, 192) ragged token / feature edges,
+#    (8292, 3072, 1088) an odd number of K tiles;
+#  wide ring (from 49152 rows, grids of 768+ workgroups of 256 x 128, K >= 768): (49152, 512, 768) full
+#    tiles, (49155, 520, 832) ragged edges and a K loop whose length is not a multiple of the ring depth;
 #  small ring (at most 128 tiles of 128 x 128): (300, 768, 3072) long K loop, (64, 2304, 768),
 #    (1, 8, 64) fewer K tiles than ring stages, (129, 136, 128) ragged edges.
 @pytest.mark.parametrize("M,N,K", [(8192, 3072, 1024), (8155, 3080, 1024), (8292, 3072, 1088), (8192, 3072, 768),
+                                   (49152, 512, 768), (49155, 520, 832),
                                    (2100, 2312, 192), (300, 768, 3072), (64, 2304, 768), (1, 8, 64), (129, 136, 128)])
 @pytest.mark.parametrize("act", ["none", "gelu", "gelu_tanh", "relu"])
 def test_gemm_bias_act(M, N, K, act):
@@ -52,10 +53,10 @@ def test_gemm_strided_rows_and_no_bias():
     W = _rand(128, 72, seed=5, scale=0.1)
     got = fused.gemm_bias_act(xs, fused.pack_weight(W.cuda()), None, "none")
     _close(got, x[:, :128].float() @ W.float(), "strided")
-    big = _rand(8192, 1088, seed=15)              # wide form, row pitch 1088, K = 1024
-    Wb = _rand(1024, 3072, seed=16, scale=0.05)
-    _close(fused.gemm_bias_act(big.cuda()[:, :1024], fused.pack_weight(Wb.cuda()), None, "none"),
-           big[:, :1024].float() @ Wb.float(), "strided, wide form")
+    big = _rand(49152, 832, seed=15)             # wide form, row pitch 832, K = 768
+    Wb = _rand(768, 512, seed=16, scale=0.05)
+    _close(fused.gemm_bias_act(big.cuda()[:, :768], fused.pack_weight(Wb.cuda()), None, "none"),
+           big[:, :768].float() @ Wb.float(), "strided, wide form")
     ident = torch.eye(64).half()                  # closed form: W = I returns the input
     _close(fused.gemm_bias_act(x.cuda()[:, :64].contiguous(), ident.cuda(), None, "none"), x[:, :64], "identity")
 
