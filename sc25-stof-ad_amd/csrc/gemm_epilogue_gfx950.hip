@@ -158,18 +158,26 @@ __global__ __launch_bounds__(256) void gemm_bias_act_kernel(const GemmParams p) 
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
+  // Fragments of k-step ks + 1 are requested before the MFMAs of k-step ks are issued (two sets of
+  // fragment registers), so the LDS latency of a k-step hides behind the previous one's products.
   auto compute = [&](const lds_byte* at, const lds_byte* wt) {
+    half8_t xa[2][2], wb[2][2];
+    auto fetch = [&](int ks, int set) {
+#pragma unroll
+      for (int mi = 0; mi < 2; ++mi) xa[set][mi] = lds_frag(at, (64 * wm + 32 * mi) * 128 + rd[ks]);
+#pragma unroll
+      for (int ni = 0; ni < 2; ++ni) wb[set][ni] = lds_frag(wt, (64 * wn + 32 * ni) * 128 + rd[ks]);
+    };
+    fetch(0, 0);
 #pragma unroll
     for (int ks = 0; ks < 4; ++ks) {
-      half8_t xa[2], wb[2];
-#pragma unroll
-      for (int mi = 0; mi < 2; ++mi) xa[mi] = lds_frag(at, (64 * wm + 32 * mi) * 128 + rd[ks]);
-#pragma unroll
-      for (int ni = 0; ni < 2; ++ni) wb[ni] = lds_frag(wt, (64 * wn + 32 * ni) * 128 + rd[ks]);
+      if (ks + 1 < 4) fetch(ks + 1, (ks + 1) & 1);
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int ni = 0; ni < 2; ++ni)
 #pragma unroll
-        for (int mi = 0; mi < 2; ++mi) acc[ni][mi] = mfma32(wb[ni], xa[mi], acc[ni][mi]);
+        for (int mi = 0; mi < 2; ++mi) acc[ni][mi] = mfma32(wb[ks & 1][ni], xa[ks & 1][mi], acc[ni][mi]);
+      __builtin_amdgcn_sched_barrier(0);
     }
   };
 
@@ -681,18 +689,26 @@ __global__ __launch_bounds__(256) void gemm_bias_res_ln_cluster_kernel(const LnC
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.f;
 
+  // Fragments of k-step ks + 1 are requested before the MFMAs of k-step ks are issued (two sets of
+  // fragment registers), so the LDS latency of a k-step hides behind the previous one's products.
   auto compute = [&](const lds_byte* at, const lds_byte* wt) {
+    half8_t xa[2][2], wb[2][2];
+    auto fetch = [&](int ks, int set) {
+#pragma unroll
+      for (int mi = 0; mi < 2; ++mi) xa[set][mi] = lds_frag(at, (64 * wm + 32 * mi) * 128 + rd[ks]);
+#pragma unroll
+      for (int ni = 0; ni < 2; ++ni) wb[set][ni] = lds_frag(wt, (64 * wn + 32 * ni) * 128 + rd[ks]);
+    };
+    fetch(0, 0);
 #pragma unroll
     for (int ks = 0; ks < 4; ++ks) {
-      half8_t xa[2], wb[2];
-#pragma unroll
-      for (int mi = 0; mi < 2; ++mi) xa[mi] = lds_frag(at, (64 * wm + 32 * mi) * 128 + rd[ks]);
-#pragma unroll
-      for (int ni = 0; ni < 2; ++ni) wb[ni] = lds_frag(wt, (64 * wn + 32 * ni) * 128 + rd[ks]);
+      if (ks + 1 < 4) fetch(ks + 1, (ks + 1) & 1);
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int ni = 0; ni < 2; ++ni)
 #pragma unroll
-        for (int mi = 0; mi < 2; ++mi) acc[ni][mi] = mfma32(wb[ni], xa[mi], acc[ni][mi]);
+        for (int mi = 0; mi < 2; ++mi) acc[ni][mi] = mfma32(wb[ks & 1][ni], xa[ks & 1][mi], acc[ni][mi]);
+      __builtin_amdgcn_sched_barrier(0);
     }
   };
 
