@@ -60,6 +60,27 @@ struct GemmParams {
   int tiles_m, tiles_n;
 };
 
+// Workgroup index -> output tile.  Workgroups go round-robin to the 8 XCDs, each with an L2 of
+// its own, and about 64 of them run on an XCD at a time.  XCD x = index % 8 owns the token tiles
+// tm = 8 q + x and takes its tiles in bands of kRasterRows values of q, feature tile after feature
+// tile inside a band: the 64 workgroups in flight on an XCD then cover 8 token tiles x 8 feature
+// tiles and bring 8 + 8 operand tiles through its L2 instead of 64 + 1 (token tile after token
+// tile for one feature tile re-read the activations once per feature tile from memory:
+// 65536 x 3072 x 768 470 us = 660 TFLOP/s where 8192 rows reach 840).
+// The grid is 8 * ceil(tiles_m / 8) * tiles_n; false = padding of the last token tiles.
+constexpr int kRasterRows = 8;
+__device__ __forceinline__ bool raster_tile(int index, int tiles_m, int tiles_n, int& tm, int& tn) {
+  const int x = index & 7, i = index >> 3;
+  const int rows_x = (tiles_m + 7) >> 3;
+  const int band = i / (kRasterRows * tiles_n), r = i - band * (kRasterRows * tiles_n);
+  const int first = band * kRasterRows;
+  const int rows = min(kRasterRows, rows_x - first);
+  tn = r / rows;
+  tm = 8 * (first + r - tn * rows) + x;
+  return tm < tiles_m;
+}
+inline unsigned raster_grid(int tiles_m, int tiles_n) { return 8u * (unsigned)((tiles_m + 7) / 8) * (unsigned)tiles_n; }
+
 // Epilogue of the bias / activation GEMMs for one wave: acc[ni][mi][r] is
 // C[m_base + 32 mi + j32][n_base + 32 ni + 8 (r / 4) + 4 g + r % 4].  In this layout a store
 // instruction would write 16 B into each of 32 rows, 32 partial cache lines per instruction
@@ -122,10 +143,8 @@ __global__ __launch_bounds__(256) void gemm_bias_act_kernel(const GemmParams p) 
   const int j32 = lane & 31, g = lane >> 5;
   const int wm = wave >> 1, wn = wave & 1;
 
-  // Consecutive workgroups share the weight tile (same tn) and walk the token tiles, so the
-  // weight tile stays hot in L2 while activations stream.
-  const int tm = blockIdx.x % p.tiles_m;
-  const int tn = blockIdx.x / p.tiles_m;
+  int tm, tn;
+  if (!raster_tile(blockIdx.x, p.tiles_m, p.tiles_n, tm, tn)) return;
   const int m0 = tm * kGT, n0 = tn * kGT;
 
   // DMA: 16 instructions of 8 rows per operand tile; wave w issues 4w..4w+3.
@@ -201,18 +220,19 @@ __global__ __launch_bounds__(256) void gemm_bias_act_kernel(const GemmParams p) 
 }
 
 // ------------------------------------------------------------------------------------------
-// Ring forms of the same GEMM: tile (64 * MI tokens) x 128 (features) x 32 (K), 4 waves as
+// Ring form of the same GEMM: tile (64 * MI tokens) x 128 (features) x 32 (K), 4 waves as
 // 2 x 2, each (32 * MI) tokens x 64 features = MI x 2 MFMA tiles.  The K loop is a ring of NS
 // stages filled by direct-to-LDS loads and is software pipelined inside the wave.
-//   MI = 4, NS = 3 (wide): 256-token tiles; a wave reads 6 fragments for 8 MFMAs per k-step
-//     (0.75 KB of LDS per MFMA instead of 1 KB) and a workgroup brings in 24 KB per 2.1 MFLOP
-//     (85 FLOP per byte over the L2 -> LDS path instead of 64): the form for large grids.
-//   MI = 1, NS = 4 (small): 64-token tiles, four times the workgroups of the 128 x 128 form and
-//     three tiles in flight per workgroup: the form for token counts that give the 128 x 128
-//     form less than one workgroup per two compute units, where the K loop of each workgroup
-//     runs at the latency of its loads (512 tokens, N 768, K 3072: 36 -> 23 us).
+//   MI = 1, NS = 4 (small) is the one that is launched: 64-token tiles, four times the workgroups
+//     of the 128 x 128 form and three tiles in flight per workgroup: the form for token counts
+//     that give the 128 x 128 form less than one workgroup per two compute units, where the K
+//     loop of each workgroup runs at the latency of its loads (512 tokens, N 768, K 3072:
+//     36 -> 23 us).
+//   MI = 4, NS = 3 (256-token tiles; 0.75 KB of LDS reads per MFMA instead of 1 KB, 85 FLOP per
+//     byte over the L2 -> LDS path instead of 64) was the form for large grids until the
+//     128 x 128 form got buffer-resource loads and the banded tile order; the kernel still
+//     supports it, the library no longer instantiates it.
 // ------------------------------------------------------------------------------------------
-constexpr int kWTok = 256;     // tokens per workgroup of the wide form (MI = 4)
 constexpr int kWFeat = 128;
 
 // 64-byte rows: chunk c of row r sits at position c ^ ((r >> 2) & 3); 16 rows fill 1 KB.
@@ -239,8 +259,8 @@ __global__ __launch_bounds__(256, 2) void gemm_bias_act_ring_kernel(const GemmPa
   const int j32 = lane & 31, g = lane >> 5;
   const int wf = wave >> 1, wt = wave & 1;   // feature half (64), token half (32 * MI)
 
-  const int tm = blockIdx.x % p.tiles_m;
-  const int tn = blockIdx.x / p.tiles_m;
+  int tm, tn;
+  if (!raster_tile(blockIdx.x, p.tiles_m, p.tiles_n, tm, tn)) return;
   const int m0 = tm * kTok, n0 = tn * kWFeat;
 
   // Loads: one instruction = 16 rows of 64 B.  A tile: 4 * MI instructions (MI per wave), W
@@ -428,23 +448,25 @@ __global__ __launch_bounds__(512) void gemm_bias_res_ln_kernel(const LnGemmParam
   // (its OWN feature rows: wave w reads back exactly what it loaded, plus the shared A tile);
   // A tile: 4 instructions, issued by waves 0..3.
   const int drow = lane >> 2;                    // row within the instruction's 16
-  const half_t* w_src[2 * NC];
+  uint32_t w_off[2 * NC];
 #pragma unroll
   for (int i = 0; i < 2 * NC; ++i) {
     const int trow = 16 * (2 * NC * wave + i) + drow;     // feature index (< N)
     const int chunk = (lane & 3) ^ swz4(trow);
-    w_src[i] = p.W + (int64_t)trow * p.K + 8 * chunk;
+    w_off[i] = (uint32_t)trow * (uint32_t)(p.K * 2) + 16 * chunk;
   }
-  const half_t* a_src;
+  uint32_t a_off;
   {
     const int trow = 16 * (wave & 3) + drow;
     const int chunk = (lane & 3) ^ swz4(trow);
-    a_src = p.A + (int64_t)min(m0 + trow, p.M - 1) * p.K + 8 * chunk;
+    a_off = (uint32_t)min(trow, p.M - 1 - m0) * (uint32_t)(p.K * 2) + 16 * chunk;
   }
+  const __amdgpu_buffer_rsrc_t a_rs = tile_rsrc(p.A + (int64_t)m0 * p.K), w_rs = tile_rsrc(p.W);
   auto issue = [&](int kt, lds_byte* wd, lds_byte* ad) {
+    const uint32_t koff = (uint32_t)kt * (kLK * 2);
 #pragma unroll
-    for (int i = 0; i < 2 * NC; ++i) dma16(w_src[i] + kt * kLK, wd + (2 * NC * wave + i) * 1024);
-    if (wave < 4) dma16(a_src + kt * kLK, ad + wave * 1024);
+    for (int i = 0; i < 2 * NC; ++i) dma16b(w_rs, w_off[i], koff, wd + (2 * NC * wave + i) * 1024);
+    if (wave < 4) dma16b(a_rs, a_off, koff, ad + wave * 1024);
   };
   // fragment read: row (32*t + j32), chunk 2*ks + g of 4, row pitch 64 B
   int rd[2];
@@ -588,8 +610,11 @@ __global__ __launch_bounds__(512) void gemm_bias_res_ln_kernel(const LnGemmParam
 //  * the wait is bounded: after a fixed number of polls (2^18; stof_gemm_bias_res_ln_cluster_set_spin_limit) the wave sets the error word of the
 //    workspace and goes on (its output rows are then wrong, the launch still ends).  The cluster's
 //    workgroups are 8 apart in dispatch order - round-robin over the 8 XCDs puts them on one XCD,
-//    where they share the activation rows in L2 - so with in-order dispatch the oldest unfinished
-//    cluster is always resident as a whole and finishes;
+//    where they share the activation rows in L2.  The grid never exceeds two workgroups per
+//    compute unit, which all run at once, and each walks over several tiles when there are more:
+//    a workgroup then only waits for workgroups that are running.  (One workgroup per tile, with
+//    more tiles than the chip holds, did run into the limit: once in some forty launches of
+//    65536 x 1024 x 4096 a resident workgroup waited for one that had not been started.);
 //  * having stored its output, a wave counts itself out of its half row block (64 rows); the
 //    last one to leave puts the half's words and the counter back to zero, so the workspace
 //    serves the next call as it is.
@@ -602,6 +627,7 @@ struct LnClusterParams {
   int* error;
   int M, N, K; int lda, ldr, ldc; float eps; float inv_n;
   int tiles_m, tiles_n; int spin_limit;
+  int total_groups;            // tiles of the walk: tiles_m rounded up to 8, times tiles_n
 };
 
 constexpr int kClusterSpinLimit = 1 << 18;   // default number of polls before a wave gives up
@@ -621,11 +647,21 @@ __global__ __launch_bounds__(256) void gemm_bias_res_ln_cluster_kernel(const LnC
   const int j32 = lane & 31, g = lane >> 5;
   const int wm = wave >> 1, wn = wave & 1;
 
-  // dispatch index -> (XCD x, i): the NT workgroups of a row block are consecutive on one XCD
-  const int x = blockIdx.x & 7, i = blockIdx.x >> 3;
+  int rd[4];
+#pragma unroll
+  for (int ks = 0; ks < 4; ++ks) rd[ks] = j32 * 128 + (((2 * ks + g) ^ swz(j32)) << 4);
+
+  // The grid is never larger than what the chip holds at once (see the launch), and a workgroup
+  // walks over tiles blockIdx, blockIdx + gridDim, ... (gridDim a multiple of 8, so a workgroup
+  // stays with the token tiles of its XCD).  A workgroup only ever waits for workgroups that are
+  // running, and no wait can close a circle: tile v waits for its partners v' < v + 8 NT, whose
+  // workgroups first had to finish tile v' - gridDim < v (gridDim >= 8 NT), and so on downwards.
+  for (int vb = blockIdx.x; vb < p.total_groups; vb += gridDim.x) {
+  // tile index -> (XCD x, i): the NT workgroups of a row block are consecutive on one XCD
+  const int x = vb & 7, i = vb >> 3;
   const int tn = i % NT;
   const int tm = (i / NT) * 8 + x;
-  if (tm >= p.tiles_m) return;   // (a whole cluster at a time: nobody waits for these)
+  if (tm >= p.tiles_m) continue;   // (a whole cluster at a time: nobody waits for these)
   const int m0 = tm * kGT, n0 = tn * kGT;
   const int nb = n0 + 64 * wn;   // first feature of this wave
 
@@ -677,10 +713,6 @@ __global__ __launch_bounds__(256) void gemm_bias_res_ln_cluster_kernel(const LnC
 #pragma unroll
     for (int ii = 0; ii < 4; ++ii) dma16b(w_rs, w_off[ii], koff, wd + (4 * wave + ii) * 1024);
   };
-  int rd[4];
-#pragma unroll
-  for (int ks = 0; ks < 4; ++ks) rd[ks] = j32 * 128 + (((2 * ks + g) ^ swz(j32)) << 4);
-
   floatx16 acc[2][2];   // [feature tile ni][token tile mi]
 #pragma unroll
   for (int a = 0; a < 2; ++a)
@@ -866,6 +898,8 @@ __global__ __launch_bounds__(256) void gemm_bias_res_ln_cluster_kernel(const LnC
       __hip_atomic_store(my_stats + (int64_t)pt * kGT, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     if (lane == 0) __hip_atomic_store(dep, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
+  __syncthreads();   // the staging areas are operand buffers again
+  }
 }
 
 // Workspace: error word (first 16 bytes), the counters of kClusterMaxRows / 128 row blocks, then
@@ -877,22 +911,17 @@ static_assert(kClusterStatsOffset % 256 == 0, "statistics start on a 256-byte bo
 
 // Which form runs.
 //  * the 128 x 128 double-buffered form for almost everything.  With its tile loads through buffer
-//    resources (no 64-bit vector add per load) it is the fastest form from 4096 to 32768 rows at every
-//    N and K measured, settled clocks, 128 x 128 vs wide ring: 8192 rows N 3072 K 768 45.8 vs 48.0 us,
-//    N 2304 K 768 36.2 vs 41.4, N 4096 K 1024 75.3 vs 76.5, N 1024 K 4096 67.3 vs 73.3, 8192^3 1042
-//    vs 1095 us (1055 TFLOP/s), 16384 x 4096 x 4096 547 vs 562 us;
-//  * wide ring (256-token tiles, 3 stages) from kWideMinRows rows on, when its grid has at least
-//    kWideMinGroups workgroups and K is at least kWideMinK: 65536 rows x N 3072 x K 768 433 vs 470 us
-//    (at 32768 rows the two tie: 187 vs 185 us).  Before the buffer-resource loads it was the form
-//    for every grid of 768+ workgroups (+3-8 %);
+//    resources (no 64-bit vector add per load) and the banded tile order it is the fastest form
+//    from 4096 rows up at every N and K measured (settled clocks, us, rows x N x K, against the
+//    ring form with 256-token tiles and 3 stages): 8192 x 3072 x 768 45.6 vs 48.0, 8192 x 2304 x 768
+//    36.2 vs 41.4, 8192 x 1024 x 4096 64.5 vs 73.3, 32768 x 3072 x 768 167 vs 185, 65536 x 3072 x 768
+//    361 vs 372, 65536 x 768 x 3072 327 vs 359, 65536 x 1024 x 4096 549 vs 606 (1000 TFLOP/s),
+//    8192^3 1042 vs 1095.  (Before these two changes the 256-token ring was the form for every
+//    grid of 768+ workgroups, by 3-8 %; it is no longer chosen.);
 //  * small ring (64-token tiles, 4 stages) when the 128 x 128 form would have at most
 //    kSmallMaxTiles workgroups.  GPU time, N x K of the BERT-base layer: 512 tokens 14.4 -> 8.9,
 //    14.0 -> 8.4, 14.5 -> 10.6, 36.0 -> 22.9 us; 2048 tokens x N 768: 14.2 -> 8.9, 36.9 -> 23.2 us;
 //    from 192 tiles on (4096 tokens x N 768, 2048 x N 2304) the two are within 5 % either way.
-constexpr int kWideStages = 3;
-constexpr int kWideMinGroups = 768;
-constexpr int kWideMinK = 768;
-constexpr int kWideMinRows = 49152;
 constexpr int kSmallStages = 4;
 constexpr int kSmallMaxTiles = 128;
 
@@ -900,7 +929,7 @@ template <int NS, int MI>
 int launch_ring(GemmParams& p, int act, hipStream_t st) {
   p.tiles_m = (p.M + 64 * MI - 1) / (64 * MI);
   p.tiles_n = (p.N + kWFeat - 1) / kWFeat;
-  const dim3 grid((unsigned)(p.tiles_m * p.tiles_n)), block(256);
+  const dim3 grid(raster_grid(p.tiles_m, p.tiles_n)), block(256);
   switch (act) {
     case STOF_ACT_NONE: hipLaunchKernelGGL((gemm_bias_act_ring_kernel<STOF_ACT_NONE, NS, MI>), grid, block, 0, st, p); break;
     case STOF_ACT_GELU_ERF: hipLaunchKernelGGL((gemm_bias_act_ring_kernel<STOF_ACT_GELU_ERF, NS, MI>), grid, block, 0, st, p); break;
@@ -926,12 +955,11 @@ extern "C" int stof_gemm_bias_act(const void* A, const void* Wt, const void* bia
   p.A = (const half_t*)A; p.W = (const half_t*)Wt; p.bias = (const half_t*)bias; p.C = (half_t*)C;
   p.M = (int)M; p.N = (int)N; p.K = (int)K; p.lda = (int)lda; p.ldc = (int)ldc;
   hipStream_t st = (hipStream_t)stream;
-  const int64_t wide_groups = ((M + kWTok - 1) / kWTok) * ((N + kWFeat - 1) / kWFeat);
-  if (wide_groups >= kWideMinGroups && K >= kWideMinK && M >= kWideMinRows) return launch_ring<kWideStages, 4>(p, act, st);
+  if (((M + 63) / 64) * ((N + kGT - 1) / kGT) > (1 << 30)) return STOF_ERR_BAD_SHAPE;   // the grid is a 32-bit count
   const int64_t tiles128 = ((M + kGT - 1) / kGT) * ((N + kGT - 1) / kGT);
   if (tiles128 <= kSmallMaxTiles) return launch_ring<kSmallStages, 1>(p, act, st);
   p.tiles_m = (int)((M + kGT - 1) / kGT); p.tiles_n = (int)((N + kGT - 1) / kGT);
-  const dim3 grid((unsigned)(p.tiles_m * p.tiles_n)), block(256);
+  const dim3 grid(raster_grid(p.tiles_m, p.tiles_n)), block(256);
   switch (act) {
     case STOF_ACT_NONE: hipLaunchKernelGGL(gemm_bias_act_kernel<STOF_ACT_NONE>, grid, block, 0, st, p); break;
     case STOF_ACT_GELU_ERF: hipLaunchKernelGGL(gemm_bias_act_kernel<STOF_ACT_GELU_ERF>, grid, block, 0, st, p); break;
@@ -965,6 +993,20 @@ extern "C" int stof_gemm_bias_res_ln(const void* A, const void* Wt, const void* 
   }
   return stof_check_launch();
 }
+
+namespace {
+constexpr int kClusterGroupsPerCu = 2;
+int cluster_compute_units() {
+  static int cus = 0;
+  if (cus == 0) {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+      n = 256;
+    cus = n;
+  }
+  return cus;
+}
+}  // namespace
 
 extern "C" int64_t stof_gemm_bias_res_ln_cluster_workspace_bytes(int64_t M, int64_t N) {
   if (M <= 0 || M > kClusterMaxRows || N <= 0 || N % kGT != 0) return 0;
@@ -1001,7 +1043,12 @@ extern "C" int stof_gemm_bias_res_ln_cluster(const void* A, const void* Wt, cons
   p.eps = eps; p.inv_n = 1.0f / (float)N; p.spin_limit = g_cluster_spin_limit;
   const int64_t groups = (int64_t)((p.tiles_m + 7) / 8) * 8 * p.tiles_n;
   if (groups > (1 << 30)) return STOF_ERR_BAD_SHAPE;
-  const dim3 grid((unsigned)groups), block(256);
+  p.total_groups = (int)groups;
+  // Two workgroups fit a compute unit (64 KB of LDS each), so a grid of at most that many
+  // (a multiple of 8) is running as a whole from the start.
+  const int64_t resident = ((int64_t)kClusterGroupsPerCu * cluster_compute_units()) / 8 * 8;
+  if (resident < 8 * p.tiles_n) return STOF_ERR_UNSUPPORTED;   // a device too small to hold one cluster per XCD
+  const dim3 grid((unsigned)(groups < resident ? groups : resident)), block(256);
   hipStream_t st = (hipStream_t)stream;
   switch (p.tiles_n) {
     case 2: hipLaunchKernelGGL(gemm_bias_res_ln_cluster_kernel<2>, grid, block, 0, st, p); break;

@@ -68,7 +68,7 @@ def pack_weight(W):
     return Wt
 
 
-def bias_residual_layernorm(x, bias, residual, gamma, beta, eps=1e-5, return_stats=False):
+def bias_residual_layernorm(x, bias, residual, gamma, beta, eps=1e-5, return_stats=False, out=None):
     """LN(x + bias + residual) * gamma + beta over the last dim; any operand but x may be None."""
     x = _f16c("x", x)
     N = x.shape[-1]
@@ -78,7 +78,8 @@ def bias_residual_layernorm(x, bias, residual, gamma, beta, eps=1e-5, return_sta
     for name, t in (("bias", bias), ("gamma", gamma), ("beta", beta)):
         _require(t is None or t.numel() == N, f"{name} must have {N} elements")
     _require(residual is None or residual.shape == x.shape, "residual must have x's shape")
-    y = torch.empty_like(x)
+    _require(out is None or (out.shape == x.shape and out.dtype == x.dtype and out.is_contiguous()), "out must be contiguous, with x's shape")
+    y = torch.empty_like(x) if out is None else out
     mean = rstd = None
     if return_stats:
         mean = torch.empty(M, dtype=torch.float32, device=x.device)
@@ -159,14 +160,45 @@ def clear_cluster_exchange_error(dev=None):
             ws[:4].zero_()
 
 
-def gemm_bias_residual_layernorm(x, Wt, bias, residual, gamma, beta, eps=1e-5, out=None, form="row"):
-    """LN(x @ Wt^T + bias + residual) * gamma + beta; the pre-normalisation values stay on chip.
+# From this many 128 x 128 output tiles on, the LayerNorm GEMM runs its cluster form.  Measured on
+# MI355X, us, cluster / GEMM then LayerNorm kernel / row form, rows x N x K: 8192 x 768 x 768
+# 22.3 / 26.0 / 42.5, 8192 x 768 x 3072 51.9 / 53.0 / 112, 8192 x 1024 x 4096 74.4 / 79.5 / 197,
+# 16384 x 768 x 768 37.9 / 42.2 / 49.0, 65536 x 1024 x 1024 221 / 237 / 288, 65536 x 512 x 512
+# 61 / 78 / 84; with K = 4 N the two-launch form is level with it or up to 7 % ahead from 32768
+# rows on (32768 x 768 x 3072 207 / 193 / 277, 32768 x 1024 x 4096 320 / 309 / 503, 65536 x 768 x 3072
+# 394 / 394 / 558: with several tiles per workgroup each tile's wait for its partners costs more
+# than the LayerNorm kernel's second pass).  Below, the tiled GEMM
+# runs its 64-token form, which the cluster kernel has no counterpart of: 2048 x 768 x 3072
+# (96 tiles) 38 / 28 / 108.  The row form (one workgroup per 64 rows streams the whole weight
+# matrix) is level with the others only at N 256.
+CLUSTER_MIN_TILES = 192
+
+
+def ln_gemm_form(M, N, K):
+    """How ``form="auto"`` runs a LayerNorm GEMM of M rows: "cluster", or "split" (tiled GEMM, then
+    the bias+residual+LayerNorm kernel; the pre-normalisation values pass through HBM as fp16), or
+    "row" where K is a multiple of 32 but not of 64, which only that kernel takes."""
+    tiles = ((M + 127) // 128) * (N // 128)
+    if cluster_supported(N, K) and tiles >= CLUSTER_MIN_TILES:
+        return "cluster"
+    return "split" if K % 64 == 0 else "row"
+
+
+def gemm_bias_residual_layernorm(x, Wt, bias, residual, gamma, beta, eps=1e-5, out=None, form="auto"):
+    """LN(x @ Wt^T + bias + residual) * gamma + beta.
 
     ``form="row"``: one workgroup owns the whole row of N features (stof_gemm_bias_res_ln).
     ``form="cluster"``: the N / 128 workgroups of a block of 128 token rows each own 128 features
-    and exchange per-row statistics through a small workspace (stof_gemm_bias_res_ln_cluster):
-    the form for token counts at which one workgroup per 64 rows leaves compute units idle."""
-    _require(form in ("row", "cluster"), f"unknown form {form!r}")
+    and exchange per-row statistics through a small workspace (stof_gemm_bias_res_ln_cluster).
+    In both the pre-normalisation values stay in registers.
+    ``form="split"``: stof_gemm_bias_act, then stof_bias_residual_layernorm.
+    ``form="auto"``: ``ln_gemm_form`` chooses."""
+    _require(form in ("auto", "row", "cluster", "split"), f"unknown form {form!r}")
+    if form == "auto":
+        form = ln_gemm_form(x.numel() // x.shape[-1], Wt.shape[0], x.shape[-1])
+    if form == "split":
+        y = gemm_bias_act(x, Wt, None, "none")
+        return bias_residual_layernorm(y, bias, None if residual is None else residual.reshape(y.shape), gamma, beta, eps, out=out)
     x = _f16c("x", x); Wt = _f16c("Wt", Wt)
     bias = _f16c("bias", bias, True); residual = _f16c("residual", residual, True)
     gamma = _f16c("gamma", gamma, True); beta = _f16c("beta", beta, True)

@@ -24,10 +24,6 @@ from . import fused
 from .ops import block_attn
 
 
-def _compute_units():
-    return torch.cuda.get_device_properties(torch.cuda.current_device()).multi_processor_count
-
-
 class EncoderLayer:
     def __init__(self, weights, n_heads, eps=1e-12, gelu="erf", ln_fusion="auto", ffn_chain="auto"):
         """``weights``: dict with W_qkv [D,3D], b_qkv, W_o [D,D], b_o, g1, be1, W_1 [D,F], b_1,
@@ -56,27 +52,11 @@ class EncoderLayer:
     def _ln_form(self, M, K):
         """How a LayerNorm GEMM of M rows and reduction length K runs: "fused" (one workgroup per
         64 rows owns the whole row), "cluster" (128 x 128 tiles, the workgroups of a row block
-        exchange row statistics) or "split" (tiled GEMM, then the bias+residual+LayerNorm kernel)."""
+        exchange row statistics) or "split" (tiled GEMM, then the bias+residual+LayerNorm kernel);
+        "auto" follows ``fused.ln_gemm_form``."""
         if self.ln_fusion in ("fused", "cluster", "split"):
             return self.ln_fusion
-        # Cluster form: its grid of (M / 128) x (hidden / 128) workgroups must fill the chip without
-        # exceeding what is resident at once (two per compute unit), because a workgroup holds its
-        # slot while it waits for its partners.  Measured on MI355X, cluster vs split, 8192 rows:
-        # hidden 768 K 768 / 3072 23.7 vs 28.5 / 55.1 vs 58.8 us, hidden 1024 K 1024 / 4096 32.1 vs
-        # 34.3 / 80.7 vs 85.8 us; at 12288 rows x hidden 768 (1.1 rounds) 108.8 vs 95.6 us.
-        tiles = ((M + 127) // 128) * (self.hidden // 128)
-        if fused.cluster_supported(self.hidden, K) and 192 <= tiles <= 2 * _compute_units():
-            return "cluster"
-        # One workgroup per 64 rows streams the whole weight matrix, so the fused kernel needs many
-        # row blocks per compute unit (or a small matrix) to beat the tiled GEMM followed by the
-        # LayerNorm kernel.  Measured on MI355X for N = K and N = K / 4: hidden 512 from 32768
-        # rows; hidden 768 / 1024 from 65536 rows (513 vs 640 us, 915 vs 1188 us at K = 4N), below
-        # that the split form wins (hidden 768, 8192 rows: 41 vs 28 us and 109 vs 60 us).
-        if self.hidden <= 256:
-            return "fused" if M >= 32768 or self.hidden < 256 else "split"
-        if self.hidden <= 512:
-            return "fused" if M >= 32768 else "split"
-        return "fused" if M >= 65536 else "split"
+        return fused.ln_gemm_form(M, self.hidden, K)
 
     def pre_ln_stored(self, M):
         """True if the products that feed the two LayerNorms are stored as fp16 tensors for M token
@@ -84,13 +64,9 @@ class EncoderLayer:
         return self._ln_form(M, self.hidden) == "split"
 
     def _gemm_ln(self, x, Wt, bias, residual, gamma, beta):
-        M = x.numel() // x.shape[-1]
-        form = self._ln_form(M, x.shape[-1])
-        if form == "split":
-            y = fused.gemm_bias_act(x, Wt, None, "none")
-            return fused.bias_residual_layernorm(y, bias, residual, gamma, beta, self.eps)
+        form = self._ln_form(x.numel() // x.shape[-1], x.shape[-1])
         return fused.gemm_bias_residual_layernorm(x, Wt, bias, residual, gamma, beta, self.eps,
-                                                  form="cluster" if form == "cluster" else "row")
+                                                  form="row" if form == "fused" else form)
 
     def _chain(self, M):
         if self.ffn_chain != "auto":

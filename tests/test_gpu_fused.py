@@ -81,12 +81,13 @@ def test_gelu_epilogue_pointwise(act, approximate):
 
 @pytest.mark.parametrize("M,N,K", [(8192, 768, 768), (2048, 768, 3072), (1000, 1024, 1024), (64, 512, 128), (7, 256, 32)])
 @pytest.mark.parametrize("eps", [1e-5, 1e-12])
-def test_gemm_bias_residual_layernorm(M, N, K, eps):
-    print(f"gemm_ln M{M} N{N} K{K}", flush=True)
+@pytest.mark.parametrize("form", ["row", "auto"])
+def test_gemm_bias_residual_layernorm(M, N, K, eps, form):
+    print(f"gemm_ln M{M} N{N} K{K} {form}", flush=True)
     x = _rand(M, K, seed=6); W = _rand(K, N, seed=7, scale=0.05); b = _rand(N, seed=8, scale=0.5)
     r = _rand(M, N, seed=9); gm = (1 + 0.1 * _rand(N, seed=10).float()).half(); bt = _rand(N, seed=11, scale=0.1)
     got = fused.gemm_bias_residual_layernorm(x.cuda(), fused.pack_weight(W.cuda()), b.cuda(), r.cuda(),
-                                             gm.cuda(), bt.cuda(), eps)
+                                             gm.cuda(), bt.cuda(), eps, form=form)
     _close(got, oe.gemm_bias_residual_layernorm(x, W, b, r, gm, bt, eps), "gemm_ln")
 
 
@@ -123,7 +124,13 @@ def test_fused_op_errors():
     with pytest.raises(StofError):
         fused.gemm_bias_act(x, W, None, "none")                                    # K % 64 != 0
     with pytest.raises(StofError):
-        fused.gemm_bias_residual_layernorm(_rand(64, 128).cuda(), _rand(384, 128).cuda(), None, None, None, None)  # N = 384
+        fused.gemm_bias_residual_layernorm(_rand(64, 128).cuda(), _rand(384, 128).cuda(), None, None, None, None, form="row")  # N = 384
+    with pytest.raises(StofError):
+        fused.gemm_bias_residual_layernorm(_rand(64, 128).cuda(), _rand(384, 128).cuda(), None, None, None, None, form="cluster")
+    x2 = _rand(64, 128, seed=22); W2 = _rand(128, 384, seed=23, scale=0.05)     # "auto" takes the two-launch form there
+    ones, zeros = torch.ones(384).half(), torch.zeros(384).half()
+    _close(fused.gemm_bias_residual_layernorm(x2.cuda(), fused.pack_weight(W2.cuda()), None, None, None, None),
+           oe.gemm_bias_residual_layernorm(x2, W2, zeros, torch.zeros(64, 384).half(), ones, zeros, 1e-5), "gemm_ln N 384")
     with pytest.raises(StofError):
         fused.gemm_bias_act(x.float(), W, None, "none")
 

@@ -24,7 +24,7 @@ def _rand(*shape, seed=0, scale=1.0):
 
 # (8192, 768, 768) / (8192, 768, 3072) / (8192, 1024, 4096): the encoder shapes (one resident round);
 # (1000, 1024, 1024): ragged last row block; (7, 256, 64): a single partly filled cluster;
-# (40000, 512, 128): more clusters than fit on the chip at once (the wait relies on dispatch order);
+# (40000, 512, 128): more tiles than workgroups (each workgroup walks over several tiles);
 # eps 1e-12 with a row offset of 30: statistics that a one-pass variance would lose
 @pytest.mark.parametrize("M,N,K", [(8192, 768, 768), (8192, 768, 3072), (8192, 1024, 4096), (1000, 1024, 1024),
                                    (7, 256, 64), (40000, 512, 128)])
@@ -43,6 +43,25 @@ def test_gemm_ln_cluster_matches_oracle(M, N, K, eps):
     again = fused.gemm_bias_residual_layernorm(*args, form="cluster")
     assert not fused.cluster_exchange_failed()
     assert torch.equal(got, again)
+
+
+def test_gemm_ln_cluster_many_tiles_long_k_repeated():
+    """Eight times more tiles than the chip holds workgroups, a long K loop, forty launches: no
+    wait may run out (a workgroup only waits for workgroups that are running) and every launch
+    gives the bits of the first, which agrees with the tiled GEMM followed by the LayerNorm
+    kernel within the fp16 rounding of that path's intermediate."""
+    M, N, K = 32768, 1024, 2048
+    x = _rand(M, K, seed=50).cuda(); Wt = fused.pack_weight(_rand(K, N, seed=51, scale=0.05).cuda())
+    b = _rand(N, seed=52, scale=0.5).cuda(); r = _rand(M, N, seed=53).cuda()
+    gm = (1 + 0.1 * _rand(N, seed=54).float()).half().cuda(); bt = _rand(N, seed=55, scale=0.1).cuda()
+    first = fused.gemm_bias_residual_layernorm(x, Wt, b, r, gm, bt, 1e-5, form="cluster").clone()
+    _close(first, fused.gemm_bias_residual_layernorm(x, Wt, b, r, gm, bt, 1e-5, form="split"), "cluster vs split", atol=6e-3)
+    out = torch.empty_like(first)
+    for i in range(40):
+        fused.gemm_bias_residual_layernorm(x, Wt, b, r, gm, bt, 1e-5, out=out, form="cluster")
+        if i % 8 == 7:
+            assert torch.equal(out, first), f"launch {i} differs"
+    assert not fused.cluster_exchange_failed()
 
 
 def test_gemm_ln_cluster_optional_operands_and_errors():
