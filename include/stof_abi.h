@@ -30,6 +30,7 @@
  *   stof_gemm_bias_act         the first product + bias + GELU of triton_matmul_batch_kernel
  *                                                           src/triton_template/gemm_gemm.py:99-150
  *                              and matmul + bias (+ F.gelu)  src/benchmk_end2end.py:80-81
+ *   stof_gemm_bias_act_splitk  the same interfaces (a second launch form: K split over workgroups)
  *   stof_gemm_bias_res_ln      batch_matmul_bias_layernorm_kernel
  *                                                           src/triton_template/gemm_add_layernorm.py:78-144
  *                              and matmul + bias + residual + F.layer_norm, src/benchmk_end2end.py:73-76
@@ -232,6 +233,30 @@ int stof_bias_res_ln(const void* x, const void* bias, const void* residual,
 int stof_gemm_bias_act(const void* A, const void* Wt, const void* bias, void* C,
                        int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldc,
                        int act, void* stream);
+
+/*
+ * The same operator (src/triton_template/gemm_gemm.py:99-150, src/benchmk_end2end.py:80-81) with
+ * the K dimension split over `splits` workgroups per tile of 64 rows x 128 features, for shapes
+ * with few output tiles and a long K (a BERT-base FFN-out product at 512 tokens is 48 tiles and
+ * K = 3072: one workgroup per tile leaves four compute units in five without work).  Each
+ * workgroup leaves fp32 partial sums in `workspace`; the one that finishes last adds them in the
+ * order of the splits (so the result does not depend on the order of arrival), applies bias and
+ * activation and writes C.  Arguments and rules as stof_gemm_bias_act, plus:
+ *   splits      2 .. 8 (fewer are used when K / 32 has fewer than that many k-tiles);
+ *   workspace   at least stof_gemm_bias_act_splitk_workspace_bytes(M, N, splits) bytes, 16-byte
+ *               aligned, ZERO at first use; every call leaves its counters zero again, so one
+ *               workspace serves any sequence of calls on one stream (calls that overlap in time
+ *               need workspaces of their own).  At most 4096 tiles (else STOF_ERR_UNSUPPORTED).
+ * stof_gemm_bias_act_splitk_plan returns the number of splits this library would use for a shape,
+ * 1 where stof_gemm_bias_act is the form to call (its rule: the plain form would run at most 128
+ * tiles of 128 x 128, the split grid stays within 256 workgroups and 4 splits, and every split
+ * keeps at least 24 k-tiles of 32).
+ */
+int stof_gemm_bias_act_splitk_plan(int64_t M, int64_t N, int64_t K);
+int64_t stof_gemm_bias_act_splitk_workspace_bytes(int64_t M, int64_t N, int splits);
+int stof_gemm_bias_act_splitk(const void* A, const void* Wt, const void* bias, void* C,
+                              int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldc,
+                              int act, int splits, void* workspace, int64_t workspace_bytes, void* stream);
 
 /*
  * Y[M,H] = act( X[M,K] @ W1^T + b1[F] ) @ W2^T (+ b2[H]) in ONE launch, W1 given as W1t[F,K] and W2

@@ -58,6 +58,8 @@ struct GemmParams {
   const half_t* A; const half_t* W; const half_t* bias; half_t* C;
   int M, N, K; int lda, ldc;
   int tiles_m, tiles_n;
+  // split-K launches only: workgroup (tile, z) multiplies k-tiles [z * nk_split, (z + 1) * nk_split)
+  float* partials; int* counters; int splits; int nk_split;
 };
 
 // Workgroup index -> output tile.  Workgroups go round-robin to the 8 XCDs, each with an L2 of
@@ -241,9 +243,10 @@ __device__ __forceinline__ int swz4(int row) { return (row >> 2) & 3; }
 // s_waitcnt immediate that waits for the vector-memory counter only (lgkmcnt 15, expcnt 7)
 constexpr int vmcnt_imm(int n) { return (n & 15) | ((n >> 4) << 14) | 0x0F70; }
 
-template <int ACT, int NS, int MI>
+template <int ACT, int NS, int MI, bool SK = false>
 __global__ __launch_bounds__(256, 2) void gemm_bias_act_ring_kernel(const GemmParams p) {
   static_assert(MI == 1 || MI == 2 || MI == 4, "token tiles per wave");
+  static_assert(!SK || MI == 1, "the split-K epilogue is written for the 64-token form");
   constexpr int kK = 32;
   constexpr int kTok = 64 * MI;           // tokens per workgroup: two waves of MI 32-token tiles
   constexpr int kLoads = MI + 2;          // load instructions per wave per tile
@@ -259,9 +262,13 @@ __global__ __launch_bounds__(256, 2) void gemm_bias_act_ring_kernel(const GemmPa
   const int j32 = lane & 31, g = lane >> 5;
   const int wf = wave >> 1, wt = wave & 1;   // feature half (64), token half (32 * MI)
 
+  // split-K: the grid is `splits` copies of the tile grid, copy z takes the z-th range of k-tiles
+  const int tile_grid = (int)(8u * (unsigned)((p.tiles_m + 7) / 8) * (unsigned)p.tiles_n);
+  const int z = SK ? (int)blockIdx.x / tile_grid : 0;
   int tm, tn;
-  if (!raster_tile(blockIdx.x, p.tiles_m, p.tiles_n, tm, tn)) return;
+  if (!raster_tile((int)blockIdx.x - z * tile_grid, p.tiles_m, p.tiles_n, tm, tn)) return;
   const int m0 = tm * kTok, n0 = tn * kWFeat;
+  const int kt_first = SK ? z * p.nk_split : 0;
 
   // Loads: one instruction = 16 rows of 64 B.  A tile: 4 * MI instructions (MI per wave), W
   // tile: 8 (2 per wave).  Rows past the edge re-read the last row.  Addresses are a wave-uniform tile
@@ -287,7 +294,7 @@ __global__ __launch_bounds__(256, 2) void gemm_bias_act_ring_kernel(const GemmPa
   const half_t* w_first = p.W + (int64_t)n0 * p.K;
   const __amdgpu_buffer_rsrc_t a_rs = tile_rsrc(a_first), w_rs = tile_rsrc(w_first);
   auto issue = [&](int kt, int stage) {
-    const uint32_t koff = (uint32_t)kt * (kK * 2);
+    const uint32_t koff = (uint32_t)(kt_first + kt) * (kK * 2);
     lds_byte* ad = (lds_byte*)a_lds + stage * kATile;
     lds_byte* wd = (lds_byte*)w_lds + stage * kWTile;
     if constexpr (MI == 1) {
@@ -380,7 +387,7 @@ __global__ __launch_bounds__(256, 2) void gemm_bias_act_ring_kernel(const GemmPa
   const uint32_t a_rd = (uint32_t)(uintptr_t)(lds_byte*)a_lds + (uint32_t)(32 * MI * wt) * 64;
   half8_t xa0[MI], wb0[2], xa1[MI], wb1[2];   // fragments of k-step 0 / k-step 1 of a tile
 
-  const int nk = p.K / kK;
+  const int nk = SK ? min(p.nk_split, p.K / kK - kt_first) : p.K / kK;
 #pragma unroll
   for (int s0 = 0; s0 < NS; ++s0)
     if (s0 < nk) issue(s0, s0);
@@ -412,7 +419,65 @@ __global__ __launch_bounds__(256, 2) void gemm_bias_act_ring_kernel(const GemmPa
   }
 
   wg_barrier();   // every wave has read its last fragments (and no load is in flight): the ring is free
-  store_wave_block<ACT, MI>(p, acc, (lds_byte*)a_lds + wave * 4096, m0 + 32 * MI * wt, n0 + 64 * wf, lane);
+  if constexpr (SK) {
+    // Each wave hands its 32 x 64 partial sums (32 floats per lane) to the wave of the same place
+    // in the split that finishes last: 8-byte device-scope stores (written through to memory, 512
+    // contiguous bytes per instruction), a wait until they are acknowledged, then one count on the
+    // (tile, wave) counter.  The wave that counts last adds the partial sums in the order of z -
+    // its own from registers - so the result does not depend on which split came last, applies
+    // the epilogue, and puts the counter back to zero for the next launch.
+    typedef unsigned long long u64;
+    const int64_t tile = (int64_t)tm * p.tiles_n + tn;
+    u64* mine = reinterpret_cast<u64*>(p.partials) + ((tile * p.splits + z) * 4 + wave) * 1024 + lane;
+#pragma unroll
+    for (int ni = 0; ni < 2; ++ni)
+#pragma unroll
+      for (int r = 0; r < 16; r += 2) {
+        // (through scalar copies: a bit cast applied directly to a vector element reads element 0)
+        const float lo = acc[ni][0][r], hi = acc[ni][0][r + 1];
+        const u64 v = ((u64)__builtin_bit_cast(unsigned, hi) << 32) | __builtin_bit_cast(unsigned, lo);
+        __hip_atomic_store(mine + (8 * ni + (r >> 1)) * 64, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+    // (relaxed atomics to different addresses are not ordered for the compiler: the empty asm
+    // statements keep the stores above the wait, the count below it and the reads below the count)
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
+    asm volatile("" ::: "memory");
+    int* counter = p.counters + tile * 4 + wave;
+    int before = 0;
+    if (lane == 0) before = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    before = __builtin_amdgcn_readfirstlane(before);
+    asm volatile("" ::: "memory");
+    if (before != p.splits - 1) return;
+    floatx16 sum[2][1];
+#pragma unroll
+    for (int ni = 0; ni < 2; ++ni)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) sum[ni][0][r] = 0.f;
+    const u64* slot0 = reinterpret_cast<const u64*>(p.partials) + ((tile * p.splits) * 4 + wave) * 1024 + lane;
+    for (int zz = 0; zz < p.splits; ++zz) {
+      if (zz == z) {
+#pragma unroll
+        for (int ni = 0; ni < 2; ++ni)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) sum[ni][0][r] += acc[ni][0][r];
+      } else {
+        const u64* src = slot0 + (int64_t)zz * 4 * 1024;
+#pragma unroll
+        for (int ni = 0; ni < 2; ++ni)
+#pragma unroll
+          for (int r = 0; r < 16; r += 2) {
+            const u64 v = __hip_atomic_load(src + (8 * ni + (r >> 1)) * 64, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            sum[ni][0][r] += __builtin_bit_cast(float, (unsigned)(v & 0xffffffffull));
+            sum[ni][0][r + 1] += __builtin_bit_cast(float, (unsigned)(v >> 32));
+          }
+      }
+    }
+    if (lane == 0) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    store_wave_block<ACT, 1>(p, sum, (lds_byte*)a_lds + wave * 4096, m0 + 32 * wt, n0 + 64 * wf, lane);
+  } else {
+    store_wave_block<ACT, MI>(p, acc, (lds_byte*)a_lds + wave * 4096, m0 + 32 * MI * wt, n0 + 64 * wf, lane);
+  }
 }
 
 // ------------------------------------------------------------------------------------------
@@ -954,6 +1019,7 @@ extern "C" int stof_gemm_bias_act(const void* A, const void* Wt, const void* bia
   GemmParams p;
   p.A = (const half_t*)A; p.W = (const half_t*)Wt; p.bias = (const half_t*)bias; p.C = (half_t*)C;
   p.M = (int)M; p.N = (int)N; p.K = (int)K; p.lda = (int)lda; p.ldc = (int)ldc;
+  p.partials = nullptr; p.counters = nullptr; p.splits = 1; p.nk_split = 0;
   hipStream_t st = (hipStream_t)stream;
   if (((M + 63) / 64) * ((N + kGT - 1) / kGT) > (1 << 30)) return STOF_ERR_BAD_SHAPE;   // the grid is a 32-bit count
   const int64_t tiles128 = ((M + kGT - 1) / kGT) * ((N + kGT - 1) / kGT);
@@ -965,6 +1031,78 @@ extern "C" int stof_gemm_bias_act(const void* A, const void* Wt, const void* bia
     case STOF_ACT_GELU_ERF: hipLaunchKernelGGL(gemm_bias_act_kernel<STOF_ACT_GELU_ERF>, grid, block, 0, st, p); break;
     case STOF_ACT_GELU_TANH: hipLaunchKernelGGL(gemm_bias_act_kernel<STOF_ACT_GELU_TANH>, grid, block, 0, st, p); break;
     case STOF_ACT_RELU: hipLaunchKernelGGL(gemm_bias_act_kernel<STOF_ACT_RELU>, grid, block, 0, st, p); break;
+    default: return STOF_ERR_UNSUPPORTED;
+  }
+  return stof_check_launch();
+}
+
+// ---- split-K form of the 64-token ring GEMM, for few output tiles and a long K ----------------
+// Workspace: one counter per (tile, wave) for up to kSplitMaxTiles tiles (a fixed area, so that a
+// workspace that served one shape can serve another; zero between calls), then the partial sums,
+// 32 KB per (tile, split).
+constexpr int64_t kSplitMaxTiles = 4096;
+constexpr int64_t kSplitPartialsOffset = kSplitMaxTiles * 4 * 4;
+constexpr int kSplitMaxSplits = 8;       // what the entry point takes
+// What the plan chooses.  Measured on MI355X (us; one workgroup per tile, then 2 / 3 / 4 / 6 / 8 splits), GELU
+// epilogue: 512 x 768 x 3072 22.2 | 15.7 13.7 13.9 19.6 17.0; 128 x 768 x 3072 21.3 | 14.8 13.0 12.7 18.1 15.9;
+// 512 x 1024 x 4096 27.7 | 18.6 16.5 17.3 20.3 21.4; 1024 x 768 x 3072 21.8 | 15.9 22.8 17.7 22.0 20.9;
+// 2048 x 768 x 3072 22.3 | 24.6 27.3 25.3; 512 x 768 x 768 7.7 | 8.6 8.7 8.9; 512 x 2304 x 768 8.3 | 12.4 12.0:
+// it pays while the grid stays within one workgroup per compute unit and a split keeps 24 k-tiles;
+// the hand-over (stores acknowledged, count, reads) costs about 5 us.
+constexpr int kSplitPlanMaxSplits = 4;
+constexpr int kSplitMinKTiles = 24;      // k-tiles of 32 per split at least
+constexpr int kSplitTargetGroups = 256;  // one workgroup per compute unit
+
+// How many ways stof_gemm_bias_act_splitk should split K for this shape; 1 = the plain form is the
+// one to use.  Only where the plain GEMM runs its 64-token form (at most kSmallMaxTiles tiles of
+// 128 x 128): there a workgroup's K loop runs at the latency of its loads and most compute units
+// have no workgroup at all.
+extern "C" int stof_gemm_bias_act_splitk_plan(int64_t M, int64_t N, int64_t K) {
+  if (M <= 0 || N <= 0 || K <= 0 || K % kGK != 0) return 1;
+  const int64_t tiles128 = ((M + kGT - 1) / kGT) * ((N + kGT - 1) / kGT);
+  if (tiles128 > kSmallMaxTiles) return 1;
+  const int64_t tiles64 = ((M + 63) / 64) * ((N + kWFeat - 1) / kWFeat);
+  int64_t splits = kSplitTargetGroups / tiles64;
+  if (splits > (K / 32) / kSplitMinKTiles) splits = (K / 32) / kSplitMinKTiles;
+  if (splits > kSplitPlanMaxSplits) splits = kSplitPlanMaxSplits;
+  return splits < 2 ? 1 : (int)splits;
+}
+
+extern "C" int64_t stof_gemm_bias_act_splitk_workspace_bytes(int64_t M, int64_t N, int splits) {
+  if (M <= 0 || N <= 0 || splits < 1 || splits > kSplitMaxSplits) return 0;
+  const int64_t tiles64 = ((M + 63) / 64) * ((N + kWFeat - 1) / kWFeat);
+  if (tiles64 > kSplitMaxTiles) return 0;
+  return kSplitPartialsOffset + tiles64 * splits * (64 * kWFeat * 4);
+}
+
+extern "C" int stof_gemm_bias_act_splitk(const void* A, const void* Wt, const void* bias, void* C,
+                                         int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldc,
+                                         int act, int splits, void* workspace, int64_t workspace_bytes, void* stream) {
+  if (!A || !Wt || !C || !workspace) return STOF_ERR_NULL_POINTER;
+  if (M <= 0 || N <= 0 || K <= 0 || K % kGK != 0 || N % 8 != 0 || lda < K || ldc < N) return STOF_ERR_BAD_SHAPE;
+  if (K > (1 << 30) || splits < 2 || splits > kSplitMaxSplits) return STOF_ERR_BAD_SHAPE;
+  const int64_t tiles64 = ((M + 63) / 64) * ((N + kWFeat - 1) / kWFeat);
+  if (tiles64 > kSplitMaxTiles) return STOF_ERR_UNSUPPORTED;
+  if (!stof_aligned16(A) || !stof_aligned16(Wt) || !stof_aligned16(C) || (bias && ((uintptr_t)bias & 7)) ||
+      ((uintptr_t)workspace & 15) || lda % 8 != 0 || ldc % 8 != 0)
+    return STOF_ERR_MISALIGNED;
+  if (workspace_bytes < stof_gemm_bias_act_splitk_workspace_bytes(M, N, splits)) return STOF_ERR_BAD_SHAPE;
+  GemmParams p;
+  p.A = (const half_t*)A; p.W = (const half_t*)Wt; p.bias = (const half_t*)bias; p.C = (half_t*)C;
+  p.M = (int)M; p.N = (int)N; p.K = (int)K; p.lda = (int)lda; p.ldc = (int)ldc;
+  p.tiles_m = (int)((M + 63) / 64); p.tiles_n = (int)((N + kWFeat - 1) / kWFeat);
+  const int nk = (int)(K / 32);
+  p.nk_split = (nk + splits - 1) / splits;
+  p.splits = (nk + p.nk_split - 1) / p.nk_split;   // (every split has at least one k-tile)
+  p.counters = reinterpret_cast<int*>(workspace);
+  p.partials = reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) + kSplitPartialsOffset);
+  const dim3 grid(raster_grid(p.tiles_m, p.tiles_n) * (unsigned)p.splits), block(256);
+  hipStream_t st = (hipStream_t)stream;
+  switch (act) {
+    case STOF_ACT_NONE: hipLaunchKernelGGL((gemm_bias_act_ring_kernel<STOF_ACT_NONE, kSmallStages, 1, true>), grid, block, 0, st, p); break;
+    case STOF_ACT_GELU_ERF: hipLaunchKernelGGL((gemm_bias_act_ring_kernel<STOF_ACT_GELU_ERF, kSmallStages, 1, true>), grid, block, 0, st, p); break;
+    case STOF_ACT_GELU_TANH: hipLaunchKernelGGL((gemm_bias_act_ring_kernel<STOF_ACT_GELU_TANH, kSmallStages, 1, true>), grid, block, 0, st, p); break;
+    case STOF_ACT_RELU: hipLaunchKernelGGL((gemm_bias_act_ring_kernel<STOF_ACT_RELU, kSmallStages, 1, true>), grid, block, 0, st, p); break;
     default: return STOF_ERR_UNSUPPORTED;
   }
   return stof_check_launch();

@@ -38,6 +38,10 @@ _SIGNATURES = {
     "stof_gemm_act_gemm_workspace_bytes": (c_int64, [c_int64, c_int64]),
     "stof_gemm_act_gemm": (c_int, [_P, _P, _P, _P, _P, _P, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64,
                                    c_int, _P, c_int64, _P]),
+    "stof_gemm_bias_act_splitk_plan": (c_int, [c_int64, c_int64, c_int64]),
+    "stof_gemm_bias_act_splitk_workspace_bytes": (c_int64, [c_int64, c_int64, c_int]),
+    "stof_gemm_bias_act_splitk": (c_int, [_P, _P, _P, _P, c_int64, c_int64, c_int64, c_int64, c_int64, c_int, c_int,
+                                          _P, c_int64, _P]),
     "stof_gemm_bias_res_ln": (c_int, [_P, _P, _P, _P, _P, _P, _P, c_int64, c_int64, c_int64, c_float, _P]),
     "stof_gemm_bias_res_ln_cluster_workspace_bytes": (c_int64, [c_int64, c_int64]),
     "stof_gemm_bias_res_ln_cluster_set_spin_limit": (c_int, [c_int]),

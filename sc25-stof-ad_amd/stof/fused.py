@@ -95,9 +95,28 @@ def triton_batched_bias_layernorm(x, bias, weight, bias_ln, eps=1e-5):
     return bias_residual_layernorm(x, bias, None, weight, bias_ln, eps)
 
 
-def gemm_bias_act(x, Wt, bias=None, act="none", out=None):
-    """act(x @ Wt^T + bias): x [..., K] (rows may be strided), Wt [N, K], bias [N]."""
+_splitk_ws = {}           # (device index, stream handle) -> zeroed workspace tensor, grown on demand
+
+
+def _splitk_workspace(dev, stream, nbytes):
+    """A workspace for stof_gemm_bias_act_splitk, one per (device, stream), zero at first use:
+    every call leaves its counters zero again, and calls on one stream do not overlap."""
+    key = (dev.index, stream)
+    ws = _splitk_ws.get(key)
+    if ws is None or ws.numel() < nbytes:
+        ws = torch.zeros(max(nbytes, 1 << 23), dtype=torch.uint8, device=dev)
+        _splitk_ws[key] = ws
+    return ws
+
+
+def gemm_bias_act(x, Wt, bias=None, act="none", out=None, splits=None):
+    """act(x @ Wt^T + bias): x [..., K] (rows may be strided), Wt [N, K], bias [N].
+
+    ``splits``: None = the library's rule (stof_gemm_bias_act_splitk_plan: K split over several
+    workgroups per tile where the output has few tiles and K is long), 1 = one workgroup per tile
+    (stof_gemm_bias_act), 2 .. 8 = that many splits (stof_gemm_bias_act_splitk)."""
     _require(act in ACT, f"unknown activation {act!r}")
+    _require(splits is None or 1 <= int(splits) <= 8, "splits must be None or 1 .. 8")
     _require(x.is_cuda and x.dtype == torch.float16, "x must be a CUDA float16 tensor")
     Wt = _f16c("Wt", Wt); bias = _f16c("bias", bias, True)
     K = x.shape[-1]
@@ -112,8 +131,21 @@ def gemm_bias_act(x, Wt, bias=None, act="none", out=None):
         out = torch.empty(x.shape[:-1] + (N,), dtype=torch.float16, device=x.device)
     o2 = out.view(-1, N)
     _require(o2.shape[0] == M and o2.stride(1) == 1, "out must be [..., N] with contiguous rows")
-    check(_lib.lib().stof_gemm_bias_act(x2.data_ptr(), Wt.data_ptr(), _p(bias), o2.data_ptr(),
-                                        M, N, K, x2.stride(0), o2.stride(0), ACT[act], _stream(o2)),
+    lib = _lib.lib()
+    st = _stream(o2)
+    if splits is None:
+        splits = lib.stof_gemm_bias_act_splitk_plan(M, N, K)
+    if splits > 1:
+        nbytes = lib.stof_gemm_bias_act_splitk_workspace_bytes(M, N, splits)
+        _require(nbytes > 0, f"shape not supported by the split-K form: M {M}, N {N}")
+        ws = _splitk_workspace(x.device, st, nbytes)
+        check(lib.stof_gemm_bias_act_splitk(x2.data_ptr(), Wt.data_ptr(), _p(bias), o2.data_ptr(),
+                                            M, N, K, x2.stride(0), o2.stride(0), ACT[act], int(splits),
+                                            ws.data_ptr(), ws.numel(), st),
+              "stof_gemm_bias_act_splitk")
+        return out
+    check(lib.stof_gemm_bias_act(x2.data_ptr(), Wt.data_ptr(), _p(bias), o2.data_ptr(),
+                                 M, N, K, x2.stride(0), o2.stride(0), ACT[act], st),
           "stof_gemm_bias_act")
     return out
 

@@ -76,6 +76,22 @@ def test_other_entry_points_argument_checks(lib):
     assert lib.stof_gemm_bias_act(P, P, None, P, 64, 64, 96, 96, 64, 0, None) == -2      # K % 64
     assert lib.stof_gemm_bias_act(P, P, None, P, 64, 64, 64, 64, 64, 9, None) == -3      # activation
     assert lib.stof_gemm_bias_act(P, P + 8, None, P, 64, 64, 64, 64, 64, 0, None) == -4
+    # split-K form: A, Wt, bias, C, M, N, K, lda, ldc, act, splits, workspace, bytes, stream
+    assert lib.stof_gemm_bias_act_splitk_plan(512, 768, 3072) == 4       # 48 tiles of 64 x 128, 96 k-tiles
+    assert lib.stof_gemm_bias_act_splitk_plan(1024, 768, 3072) == 2      # 96 tiles: two splits stay within 256 workgroups
+    assert lib.stof_gemm_bias_act_splitk_plan(512, 768, 768) == 1        # 24 k-tiles: too short to split
+    assert lib.stof_gemm_bias_act_splitk_plan(2048, 768, 3072) == 1      # 192 tiles already
+    assert lib.stof_gemm_bias_act_splitk_plan(8192, 3072, 768) == 1 and lib.stof_gemm_bias_act_splitk_plan(512, 768, 100) == 1
+    sneed = lib.stof_gemm_bias_act_splitk_workspace_bytes(512, 768, 4)
+    assert sneed == 4096 * 16 + 48 * 4 * 64 * 128 * 4
+    assert lib.stof_gemm_bias_act_splitk_workspace_bytes(512, 768, 9) == 0 and lib.stof_gemm_bias_act_splitk_workspace_bytes(1 << 20, 768, 2) == 0
+    sk = lambda **kw: lib.stof_gemm_bias_act_splitk(kw.get("A", P), P, None, P, kw.get("M", 512), 768, kw.get("K", 3072), 3072, 768,
+                                                    kw.get("act", 0), kw.get("splits", 4), kw.get("ws", P), kw.get("wsb", sneed), None)
+    assert sk(ws=None) == -1
+    assert sk(K=3088) == -2 and sk(splits=1) == -2 and sk(splits=9) == -2
+    assert sk(wsb=sneed - 1) == -2         # workspace too small
+    assert sk(act=9) == -3 and sk(M=1 << 20, wsb=1 << 40) == -3      # more tiles than the counter area holds
+    assert sk(A=P + 8) == -4 and sk(ws=P + 8) == -4
     # chained GEMM + activation + GEMM: X, W1t, b1, W2t, b2, Y, M, K, F, H, ldx, ldy, act, workspace, bytes, stream
     need = lib.stof_gemm_act_gemm_workspace_bytes(64, 128)
     assert need >= 64 * 128 * 4 + 4 and lib.stof_gemm_act_gemm_workspace_bytes(0, 128) == 0

@@ -28,14 +28,14 @@ def _rand(*shape, seed=0, scale=1.0):
 
 # ---- GEMM + bias + activation -----------------------------------------------------------------
 
-# Three launch forms behind one entry point:
+# Launch forms behind fused.gemm_bias_act:
 #  128 x 128 double-buffered (the default): (8192, 3072, 1024) and (8192, 3072, 768) full tiles at the
 #    encoder's shapes, (8155, 3080, 1024) and (2100, 2312, 192) ragged token / feature edges,
-#    (8292, 3072, 1088) an odd number of K tiles;
-#  wide ring (from 49152 rows, grids of 768+ workgroups of 256 x 128, K >= 768): (49152, 512, 768) full
-#    tiles, (49155, 520, 832) ragged edges and a K loop whose length is not a multiple of the ring depth;
-#  small ring (at most 128 tiles of 128 x 128): (300, 768, 3072) long K loop, (64, 2304, 768),
-#    (1, 8, 64) fewer K tiles than ring stages, (129, 136, 128) ragged edges.
+#    (8292, 3072, 1088) an odd number of K tiles; (49152, 512, 768) and (49155, 520, 832): more token
+#    tiles than resident workgroups (several bands of the tile order, padded last band);
+#  small ring (at most 128 tiles of 128 x 128): (64, 2304, 768), (1, 8, 64) fewer K tiles than ring
+#    stages, (129, 136, 128) ragged edges;
+#  split-K on the small ring (few tiles, long K; the library's rule picks it): (300, 768, 3072).
 @pytest.mark.parametrize("M,N,K", [(8192, 3072, 1024), (8155, 3080, 1024), (8292, 3072, 1088), (8192, 3072, 768),
                                    (49152, 512, 768), (49155, 520, 832),
                                    (2100, 2312, 192), (300, 768, 3072), (64, 2304, 768), (1, 8, 64), (129, 136, 128)])
@@ -45,6 +45,38 @@ def test_gemm_bias_act(M, N, K, act):
     x = _rand(M, K, seed=1); W = _rand(K, N, seed=2, scale=0.05); b = _rand(N, seed=3, scale=0.5)
     got = fused.gemm_bias_act(x.cuda(), fused.pack_weight(W.cuda()), b.cuda(), act)
     _close(got, oe.gemm_bias_act(x, W, b, act), f"gemm {act}")
+
+
+# splits 1 = one workgroup per tile.  (129, 136, 128): 4 k-tiles, so 3 splits become 2 of 2 k-tiles;
+# (1, 8, 64): 2 k-tiles; (512, 768, 3072): the FFN-out product of a 512-token BERT-base layer;
+# (200, 520, 1088): ragged edges, 34 k-tiles over 8 splits (5 + 5 + ... + 4).
+@pytest.mark.parametrize("M,N,K", [(512, 768, 3072), (200, 520, 1088), (129, 136, 128), (1, 8, 64)])
+@pytest.mark.parametrize("splits", [1, 2, 3, 8])
+def test_gemm_split_k(M, N, K, splits):
+    print(f"gemm split-K M{M} N{N} K{K} splits {splits}", flush=True)
+    x = _rand(M, K, seed=1); W = _rand(K, N, seed=2, scale=0.05); b = _rand(N, seed=3, scale=0.5)
+    xg, Wt, bg = x.cuda(), fused.pack_weight(W.cuda()), b.cuda()
+    for act in ("none", "gelu"):
+        got = fused.gemm_bias_act(xg, Wt, bg, act, splits=splits)
+        _close(got, oe.gemm_bias_act(x, W, b, act), f"split-K {act}")
+        # the partial sums are added in the order of the splits, whichever finishes last: same bits every time
+        for _ in range(3):
+            assert torch.equal(fused.gemm_bias_act(xg, Wt, bg, act, splits=splits), got)
+
+
+def test_gemm_split_k_workspace_serves_a_sequence_of_shapes():
+    """One workspace per stream: its counters are back at zero after every call, so calls of
+    different shapes and split counts can follow each other."""
+    want = {}
+    shapes = [(512, 768, 3072, 4), (64, 256, 1024, 2), (300, 1024, 4096, 3), (512, 768, 3072, 2)]
+    data = {}
+    for (M, N, K, sp) in shapes:
+        x = _rand(M, K, seed=M + sp); W = _rand(K, N, seed=N + sp, scale=0.05); b = _rand(N, seed=7, scale=0.5)
+        data[(M, N, K, sp)] = (x.cuda(), fused.pack_weight(W.cuda()), b.cuda())
+        want[(M, N, K, sp)] = oe.gemm_bias_act(x, W, b, "gelu")
+    for rep in range(3):
+        for key in shapes:
+            _close(fused.gemm_bias_act(*data[key], "gelu", splits=key[3]), want[key], f"sequence {key} pass {rep}")
 
 
 def test_gemm_strided_rows_and_no_bias():
