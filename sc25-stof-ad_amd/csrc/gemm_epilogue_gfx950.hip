@@ -1,6 +1,6 @@
 // Fused encoder GEMMs for gfx950 (MI355X):
-//   stof_gemm_bias_act     C = act(A @ W^T + bias)                       (bias / GELU / ReLU epilogue)
-//   stof_gemm_bias_res_ln  C = LN(A @ W^T + bias + residual) * g + b     (LayerNorm epilogue)
+//   stof_gemm_bias_act, stof_gemm_bias_act_splitk       C = act(A @ W^T + bias)       (bias / GELU / ReLU epilogue)
+//   stof_gemm_bias_res_ln, stof_gemm_bias_res_ln_cluster  C = LN(A @ W^T + bias + residual) * g + b   (LayerNorm epilogue)
 //
 // They replace the reference's Triton templates (src/triton_template/gemm_gemm.py:99-150,
 // src/triton_template/gemm_add_layernorm.py:78-123).  Common design:
@@ -14,10 +14,11 @@
 //    a lane then owns ONE token row (lane & 31) and its registers run along the feature
 //    dimension in groups of four consecutive columns.  Bias, activation, residual and the
 //    LayerNorm statistics become per-lane register loops, and stores are 8-byte vectors;
-//  * the LayerNorm kernel gives one workgroup (8 waves) the full row of N features, each
-//    wave a slice of N/8 columns; mean and variance are reduced in registers, across the
-//    lane pair with v_permlane32_swap and across the 8 waves through 2 KB of LDS, so the
-//    pre-normalisation tensor never leaves the chip.
+//  * the LayerNorm kernels keep the pre-normalisation tensor on chip: either one workgroup
+//    (8 waves) owns the full row of N features, each wave a slice of N/8 columns, with mean
+//    and variance reduced in registers, across the lane pair with v_permlane32_swap and across
+//    the 8 waves through 2 KB of LDS; or the N / 128 workgroups of a block of 128 token rows
+//    each own a 128 x 128 tile and exchange per-row statistics through a small workspace.
 #include "stof_common.h"
 
 namespace {
@@ -222,18 +223,16 @@ __global__ __launch_bounds__(256) void gemm_bias_act_kernel(const GemmParams p) 
 }
 
 // ------------------------------------------------------------------------------------------
-// Ring form of the same GEMM: tile (64 * MI tokens) x 128 (features) x 32 (K), 4 waves as
-// 2 x 2, each (32 * MI) tokens x 64 features = MI x 2 MFMA tiles.  The K loop is a ring of NS
-// stages filled by direct-to-LDS loads and is software pipelined inside the wave.
-//   MI = 1, NS = 4 (small) is the one that is launched: 64-token tiles, four times the workgroups
-//     of the 128 x 128 form and three tiles in flight per workgroup: the form for token counts
-//     that give the 128 x 128 form less than one workgroup per two compute units, where the K
-//     loop of each workgroup runs at the latency of its loads (512 tokens, N 768, K 3072:
-//     36 -> 23 us).
-//   MI = 4, NS = 3 (256-token tiles; 0.75 KB of LDS reads per MFMA instead of 1 KB, 85 FLOP per
-//     byte over the L2 -> LDS path instead of 64) was the form for large grids until the
-//     128 x 128 form got buffer-resource loads and the banded tile order; the kernel still
-//     supports it, the library no longer instantiates it.
+// Ring form of the same GEMM for small token counts: tile 64 (tokens) x 128 (features) x 32 (K),
+// 4 waves as 2 x 2, each 32 tokens x 64 features = 2 MFMA tiles; four times the workgroups of the
+// 128 x 128 form.  The K loop is a ring of NS = 4 stages filled by direct-to-LDS loads (three
+// tiles in flight per workgroup) and is software pipelined inside the wave: the form for token
+// counts that give the 128 x 128 form less than one workgroup per two compute units, where the
+// K loop of each workgroup runs at the latency of its loads (512 tokens, N 768, K 3072:
+// 36 -> 23 us).  With SK the K dimension is split over several workgroups per tile as well.
+// (The same structure with 256-token tiles and three stages - 0.75 KB of LDS reads per MFMA
+// instead of 1 KB - was the form for large grids until the 128 x 128 form got buffer-resource
+// loads and the banded tile order; it is no longer part of the library.)
 // ------------------------------------------------------------------------------------------
 constexpr int kWFeat = 128;
 
@@ -243,14 +242,12 @@ __device__ __forceinline__ int swz4(int row) { return (row >> 2) & 3; }
 // s_waitcnt immediate that waits for the vector-memory counter only (lgkmcnt 15, expcnt 7)
 constexpr int vmcnt_imm(int n) { return (n & 15) | ((n >> 4) << 14) | 0x0F70; }
 
-template <int ACT, int NS, int MI, bool SK = false>
+template <int ACT, int NS, bool SK = false>
 __global__ __launch_bounds__(256, 2) void gemm_bias_act_ring_kernel(const GemmParams p) {
-  static_assert(MI == 1 || MI == 2 || MI == 4, "token tiles per wave");
-  static_assert(!SK || MI == 1, "the split-K epilogue is written for the 64-token form");
   constexpr int kK = 32;
-  constexpr int kTok = 64 * MI;           // tokens per workgroup: two waves of MI 32-token tiles
-  constexpr int kLoads = MI + 2;          // load instructions per wave per tile
-  constexpr int kATile = kTok * kK * 2, kWTile = kWFeat * kK * 2;   // 4 KB * MI, 8 KB
+  constexpr int kTok = 64;                // tokens per workgroup: two waves of 32
+  constexpr int kLoads = 3;               // load instructions per wave per tile
+  constexpr int kATile = kTok * kK * 2, kWTile = kWFeat * kK * 2;   // 4 KB, 8 KB
   // Ring of NS stages: NS tiles are in flight or in use at any time, so a tile has NS - 1 tile
   // times to arrive.  (The fragment reads below are asm, so the compiler does not order them
   // against the direct-to-LDS loads and one array per operand is enough.)
@@ -260,7 +257,7 @@ __global__ __launch_bounds__(256, 2) void gemm_bias_act_ring_kernel(const GemmPa
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int lane = threadIdx.x & 63;
   const int j32 = lane & 31, g = lane >> 5;
-  const int wf = wave >> 1, wt = wave & 1;   // feature half (64), token half (32 * MI)
+  const int wf = wave >> 1, wt = wave & 1;   // feature half (64), token half (32)
 
   // split-K: the grid is `splits` copies of the tile grid, copy z takes the z-th range of k-tiles
   const int tile_grid = (int)(8u * (unsigned)((p.tiles_m + 7) / 8) * (unsigned)p.tiles_n);
@@ -270,112 +267,68 @@ __global__ __launch_bounds__(256, 2) void gemm_bias_act_ring_kernel(const GemmPa
   const int m0 = tm * kTok, n0 = tn * kWFeat;
   const int kt_first = SK ? z * p.nk_split : 0;
 
-  // Loads: one instruction = 16 rows of 64 B.  A tile: 4 * MI instructions (MI per wave), W
-  // tile: 8 (2 per wave).  Rows past the edge re-read the last row.  Addresses are a wave-uniform tile
-  // base (advanced along K in scalar registers) plus a 32-bit per-lane byte offset.
+  // Loads: one instruction = 16 rows of 64 B.  A tile: 4 instructions (one per wave), W tile: 8
+  // (2 per wave).  Rows past the edge re-read the last row.  Plain global addresses: the K loop
+  // runs at the latency of its loads, and the buffer-resource form that the 128 x 128 kernel
+  // gains from measured 10-25 % slower here (512 x 3072 x 768: 11.4 vs 9.1 us).
   const int drow = lane >> 2;
-  uint32_t a_off[MI], w_off[2];
-#pragma unroll
-  for (int i = 0; i < MI; ++i) {
-    const int trow = 16 * (MI * wave + i) + drow;
-    const int chunk = (lane & 3) ^ swz4(trow);
-    a_off[i] = (uint32_t)min(trow, p.M - 1 - m0) * (uint32_t)(p.lda * 2) + 16 * chunk;
+  uint32_t a_off, w_off[2];
+  {
+    const int trow = 16 * wave + drow;
+    a_off = (uint32_t)min(trow, p.M - 1 - m0) * (uint32_t)(p.lda * 2) + 16 * ((lane & 3) ^ swz4(trow));
   }
 #pragma unroll
   for (int i = 0; i < 2; ++i) {
     const int trow = 16 * (2 * wave + i) + drow;
-    const int chunk = (lane & 3) ^ swz4(trow);
-    w_off[i] = (uint32_t)min(trow, p.N - 1 - n0) * (uint32_t)(p.K * 2) + 16 * chunk;
+    w_off[i] = (uint32_t)min(trow, p.N - 1 - n0) * (uint32_t)(p.K * 2) + 16 * ((lane & 3) ^ swz4(trow));
   }
-  // (The small form keeps plain global addresses: its K loop runs at the latency of its loads, and
-  // the buffer form measured 10-25 % slower there - 512 x 3072 x 768: 11.4 vs 9.1 us - while the wide
-  // form, which runs at their rate, gains 2-3 % from it.)
-  const half_t* a_first = p.A + (int64_t)m0 * p.lda;
-  const half_t* w_first = p.W + (int64_t)n0 * p.K;
-  const __amdgpu_buffer_rsrc_t a_rs = tile_rsrc(a_first), w_rs = tile_rsrc(w_first);
+  const char* a_first = reinterpret_cast<const char*>(p.A + (int64_t)m0 * p.lda);
+  const char* w_first = reinterpret_cast<const char*>(p.W + (int64_t)n0 * p.K);
   auto issue = [&](int kt, int stage) {
     const uint32_t koff = (uint32_t)(kt_first + kt) * (kK * 2);
     lds_byte* ad = (lds_byte*)a_lds + stage * kATile;
     lds_byte* wd = (lds_byte*)w_lds + stage * kWTile;
-    if constexpr (MI == 1) {
-      const char* ab = reinterpret_cast<const char*>(a_first) + koff;
-      const char* wb = reinterpret_cast<const char*>(w_first) + koff;
+    __builtin_amdgcn_global_load_lds((gptr_t*)(a_first + koff + a_off), (__attribute__((address_space(3))) void*)(ad + wave * 1024), 16, 0, 0);
 #pragma unroll
-      for (int i = 0; i < MI; ++i)
-        __builtin_amdgcn_global_load_lds((gptr_t*)(ab + a_off[i]), (__attribute__((address_space(3))) void*)(ad + (MI * wave + i) * 1024), 16, 0, 0);
-#pragma unroll
-      for (int i = 0; i < 2; ++i)
-        __builtin_amdgcn_global_load_lds((gptr_t*)(wb + w_off[i]), (__attribute__((address_space(3))) void*)(wd + (2 * wave + i) * 1024), 16, 0, 0);
-    } else {
-#pragma unroll
-      for (int i = 0; i < MI; ++i) dma16b(a_rs, a_off[i], koff, ad + (MI * wave + i) * 1024);
-#pragma unroll
-      for (int i = 0; i < 2; ++i) dma16b(w_rs, w_off[i], koff, wd + (2 * wave + i) * 1024);
-    }
+    for (int i = 0; i < 2; ++i)
+      __builtin_amdgcn_global_load_lds((gptr_t*)(w_first + koff + w_off[i]), (__attribute__((address_space(3))) void*)(wd + (2 * wave + i) * 1024), 16, 0, 0);
   };
   // fragment read: row (32*t + j32), chunk 2*ks + g of 4, row pitch 64 B
   int rd[2];
 #pragma unroll
   for (int ks = 0; ks < 2; ++ks) rd[ks] = j32 * 64 + (((2 * ks + g) ^ swz4(j32)) << 4);
 
-  floatx16 acc[2][MI];   // [feature tile ni][token tile mi]
+  floatx16 acc[2][1];   // [feature tile ni][token tile]
 #pragma unroll
   for (int i = 0; i < 2; ++i)
 #pragma unroll
-    for (int j = 0; j < MI; ++j)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+    for (int r = 0; r < 16; ++r) acc[i][0][r] = 0.f;
 
   // Fragment reads are written as asm: the compiler orders LDS reads it can see after every
   // direct-to-LDS load it cannot prove disjoint, which drains the ring.  The ring's own
   // counter waits cover that dependency; the LDS counter is waited on by hand (lds_wait).
-  auto frags = [&](uint32_t wa, uint32_t aa, half8_t (&wbk)[2], half8_t (&xak)[MI]) {
-    if constexpr (MI == 4) {
-      asm volatile(
-          "ds_read_b128 %0, %6\n\tds_read_b128 %1, %6 offset:2048\n\t"
-          "ds_read_b128 %2, %7\n\tds_read_b128 %3, %7 offset:2048\n\t"
-          "ds_read_b128 %4, %7 offset:4096\n\tds_read_b128 %5, %7 offset:6144"
-          : "=&v"(wbk[0]), "=&v"(wbk[1]), "=&v"(xak[0]), "=&v"(xak[1]), "=&v"(xak[2]), "=&v"(xak[3])
-          : "v"(wa), "v"(aa));
-    } else if constexpr (MI == 2) {
-      asm volatile(
-          "ds_read_b128 %0, %4\n\tds_read_b128 %1, %4 offset:2048\n\t"
-          "ds_read_b128 %2, %5\n\tds_read_b128 %3, %5 offset:2048"
-          : "=&v"(wbk[0]), "=&v"(wbk[1]), "=&v"(xak[0]), "=&v"(xak[1])
-          : "v"(wa), "v"(aa));
-    } else {
-      asm volatile(
-          "ds_read_b128 %0, %3\n\tds_read_b128 %1, %3 offset:2048\n\t"
-          "ds_read_b128 %2, %4"
-          : "=&v"(wbk[0]), "=&v"(wbk[1]), "=&v"(xak[0])
-          : "v"(wa), "v"(aa));
-    }
+  auto frags = [&](uint32_t wa, uint32_t aa, half8_t (&wbk)[2], half8_t& xak) {
+    asm volatile(
+        "ds_read_b128 %0, %3\n\tds_read_b128 %1, %3 offset:2048\n\t"
+        "ds_read_b128 %2, %4"
+        : "=&v"(wbk[0]), "=&v"(wbk[1]), "=&v"(xak)
+        : "v"(wa), "v"(aa));
   };
   // Wait for the fragment reads of one set: all reads (newer_in_flight false) or all but the
-  // MI + 2 reads of the set requested last.  The wait is an asm statement that names the
+  // 3 reads of the set requested last.  The wait is an asm statement that names the
   // fragments it covers as read-write operands, so every use of them depends on it and neither
   // the scheduler nor the register allocator can move a use (or a copy) above the wait.  The LDS
   // counter is shared with scalar loads, which return out of order: an outstanding one can only
   // make this wait longer, never shorter, because LDS reads return in order among themselves.
-  auto lds_wait = [&](bool newer_in_flight, half8_t (&wbk)[2], half8_t (&xak)[MI]) {
+  auto lds_wait = [&](bool newer_in_flight, half8_t (&wbk)[2], half8_t& xak) {
     __builtin_amdgcn_sched_barrier(0);   // (keeps the software pipeline in the order written)
-    if constexpr (MI == 4) {
-      if (newer_in_flight) asm volatile("s_waitcnt lgkmcnt(6)" : "+v"(wbk[0]), "+v"(wbk[1]), "+v"(xak[0]), "+v"(xak[1]), "+v"(xak[2]), "+v"(xak[3]));
-      else asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(wbk[0]), "+v"(wbk[1]), "+v"(xak[0]), "+v"(xak[1]), "+v"(xak[2]), "+v"(xak[3]));
-    } else if constexpr (MI == 2) {
-      if (newer_in_flight) asm volatile("s_waitcnt lgkmcnt(4)" : "+v"(wbk[0]), "+v"(wbk[1]), "+v"(xak[0]), "+v"(xak[1]));
-      else asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(wbk[0]), "+v"(wbk[1]), "+v"(xak[0]), "+v"(xak[1]));
-    } else {
-      if (newer_in_flight) asm volatile("s_waitcnt lgkmcnt(3)" : "+v"(wbk[0]), "+v"(wbk[1]), "+v"(xak[0]));
-      else asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(wbk[0]), "+v"(wbk[1]), "+v"(xak[0]));
-    }
+    if (newer_in_flight) asm volatile("s_waitcnt lgkmcnt(3)" : "+v"(wbk[0]), "+v"(wbk[1]), "+v"(xak));
+    else asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(wbk[0]), "+v"(wbk[1]), "+v"(xak));
     __builtin_amdgcn_sched_barrier(0);
   };
-  auto mfmas = [&](const half8_t (&wbk)[2], const half8_t (&xak)[MI]) {
+  auto mfmas = [&](const half8_t (&wbk)[2], const half8_t& xak) {
 #pragma unroll
-    for (int mi = 0; mi < MI; ++mi)
-#pragma unroll
-      for (int ni = 0; ni < 2; ++ni) acc[ni][mi] = mfma32(wbk[ni], xak[mi], acc[ni][mi]);
+    for (int ni = 0; ni < 2; ++ni) acc[ni][0] = mfma32(wbk[ni], xak, acc[ni][0]);
   };
   auto wg_barrier = [&]() {
     // bare barrier: the fences of __syncthreads() would drain the loads that must stay in flight
@@ -384,8 +337,8 @@ __global__ __launch_bounds__(256, 2) void gemm_bias_act_ring_kernel(const GemmPa
     __builtin_amdgcn_sched_barrier(0);
   };
   const uint32_t w_rd = (uint32_t)(uintptr_t)(lds_byte*)w_lds + (uint32_t)(64 * wf) * 64;
-  const uint32_t a_rd = (uint32_t)(uintptr_t)(lds_byte*)a_lds + (uint32_t)(32 * MI * wt) * 64;
-  half8_t xa0[MI], wb0[2], xa1[MI], wb1[2];   // fragments of k-step 0 / k-step 1 of a tile
+  const uint32_t a_rd = (uint32_t)(uintptr_t)(lds_byte*)a_lds + (uint32_t)(32 * wt) * 64;
+  half8_t xa0, wb0[2], xa1, wb1[2];   // fragments of k-step 0 / k-step 1 of a tile
 
   const int nk = SK ? min(p.nk_split, p.K / kK - kt_first) : p.K / kK;
 #pragma unroll
@@ -476,7 +429,7 @@ __global__ __launch_bounds__(256, 2) void gemm_bias_act_ring_kernel(const GemmPa
     if (lane == 0) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     store_wave_block<ACT, 1>(p, sum, (lds_byte*)a_lds + wave * 4096, m0 + 32 * wt, n0 + 64 * wf, lane);
   } else {
-    store_wave_block<ACT, MI>(p, acc, (lds_byte*)a_lds + wave * 4096, m0 + 32 * MI * wt, n0 + 64 * wf, lane);
+    store_wave_block<ACT, 1>(p, acc, (lds_byte*)a_lds + wave * 4096, m0 + 32 * wt, n0 + 64 * wf, lane);
   }
 }
 
@@ -990,16 +943,16 @@ static_assert(kClusterStatsOffset % 256 == 0, "statistics start on a 256-byte bo
 constexpr int kSmallStages = 4;
 constexpr int kSmallMaxTiles = 128;
 
-template <int NS, int MI>
+template <int NS>
 int launch_ring(GemmParams& p, int act, hipStream_t st) {
-  p.tiles_m = (p.M + 64 * MI - 1) / (64 * MI);
+  p.tiles_m = (p.M + 63) / 64;
   p.tiles_n = (p.N + kWFeat - 1) / kWFeat;
   const dim3 grid(raster_grid(p.tiles_m, p.tiles_n)), block(256);
   switch (act) {
-    case STOF_ACT_NONE: hipLaunchKernelGGL((gemm_bias_act_ring_kernel<STOF_ACT_NONE, NS, MI>), grid, block, 0, st, p); break;
-    case STOF_ACT_GELU_ERF: hipLaunchKernelGGL((gemm_bias_act_ring_kernel<STOF_ACT_GELU_ERF, NS, MI>), grid, block, 0, st, p); break;
-    case STOF_ACT_GELU_TANH: hipLaunchKernelGGL((gemm_bias_act_ring_kernel<STOF_ACT_GELU_TANH, NS, MI>), grid, block, 0, st, p); break;
-    case STOF_ACT_RELU: hipLaunchKernelGGL((gemm_bias_act_ring_kernel<STOF_ACT_RELU, NS, MI>), grid, block, 0, st, p); break;
+    case STOF_ACT_NONE: hipLaunchKernelGGL((gemm_bias_act_ring_kernel<STOF_ACT_NONE, NS>), grid, block, 0, st, p); break;
+    case STOF_ACT_GELU_ERF: hipLaunchKernelGGL((gemm_bias_act_ring_kernel<STOF_ACT_GELU_ERF, NS>), grid, block, 0, st, p); break;
+    case STOF_ACT_GELU_TANH: hipLaunchKernelGGL((gemm_bias_act_ring_kernel<STOF_ACT_GELU_TANH, NS>), grid, block, 0, st, p); break;
+    case STOF_ACT_RELU: hipLaunchKernelGGL((gemm_bias_act_ring_kernel<STOF_ACT_RELU, NS>), grid, block, 0, st, p); break;
     default: return STOF_ERR_UNSUPPORTED;
   }
   return stof_check_launch();
@@ -1023,7 +976,7 @@ extern "C" int stof_gemm_bias_act(const void* A, const void* Wt, const void* bia
   hipStream_t st = (hipStream_t)stream;
   if (((M + 63) / 64) * ((N + kGT - 1) / kGT) > (1 << 30)) return STOF_ERR_BAD_SHAPE;   // the grid is a 32-bit count
   const int64_t tiles128 = ((M + kGT - 1) / kGT) * ((N + kGT - 1) / kGT);
-  if (tiles128 <= kSmallMaxTiles) return launch_ring<kSmallStages, 1>(p, act, st);
+  if (tiles128 <= kSmallMaxTiles) return launch_ring<kSmallStages>(p, act, st);
   p.tiles_m = (int)((M + kGT - 1) / kGT); p.tiles_n = (int)((N + kGT - 1) / kGT);
   const dim3 grid(raster_grid(p.tiles_m, p.tiles_n)), block(256);
   switch (act) {
@@ -1099,10 +1052,10 @@ extern "C" int stof_gemm_bias_act_splitk(const void* A, const void* Wt, const vo
   const dim3 grid(raster_grid(p.tiles_m, p.tiles_n) * (unsigned)p.splits), block(256);
   hipStream_t st = (hipStream_t)stream;
   switch (act) {
-    case STOF_ACT_NONE: hipLaunchKernelGGL((gemm_bias_act_ring_kernel<STOF_ACT_NONE, kSmallStages, 1, true>), grid, block, 0, st, p); break;
-    case STOF_ACT_GELU_ERF: hipLaunchKernelGGL((gemm_bias_act_ring_kernel<STOF_ACT_GELU_ERF, kSmallStages, 1, true>), grid, block, 0, st, p); break;
-    case STOF_ACT_GELU_TANH: hipLaunchKernelGGL((gemm_bias_act_ring_kernel<STOF_ACT_GELU_TANH, kSmallStages, 1, true>), grid, block, 0, st, p); break;
-    case STOF_ACT_RELU: hipLaunchKernelGGL((gemm_bias_act_ring_kernel<STOF_ACT_RELU, kSmallStages, 1, true>), grid, block, 0, st, p); break;
+    case STOF_ACT_NONE: hipLaunchKernelGGL((gemm_bias_act_ring_kernel<STOF_ACT_NONE, kSmallStages, true>), grid, block, 0, st, p); break;
+    case STOF_ACT_GELU_ERF: hipLaunchKernelGGL((gemm_bias_act_ring_kernel<STOF_ACT_GELU_ERF, kSmallStages, true>), grid, block, 0, st, p); break;
+    case STOF_ACT_GELU_TANH: hipLaunchKernelGGL((gemm_bias_act_ring_kernel<STOF_ACT_GELU_TANH, kSmallStages, true>), grid, block, 0, st, p); break;
+    case STOF_ACT_RELU: hipLaunchKernelGGL((gemm_bias_act_ring_kernel<STOF_ACT_RELU, kSmallStages, true>), grid, block, 0, st, p); break;
     default: return STOF_ERR_UNSUPPORTED;
   }
   return stof_check_launch();
