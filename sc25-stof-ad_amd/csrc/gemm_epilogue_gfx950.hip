@@ -1002,7 +1002,7 @@ constexpr int kSplitMaxSplits = 8;       // what the entry point takes
 // 2048 x 768 x 3072 22.3 | 24.6 27.3 25.3; 512 x 768 x 768 7.7 | 8.6 8.7 8.9; 512 x 2304 x 768 8.3 | 12.4 12.0:
 // it pays while the grid stays within one workgroup per compute unit and a split keeps 24 k-tiles;
 // the hand-over (stores acknowledged, count, reads) costs about 5 us.
-constexpr int kSplitPlanMaxSplits = 4;
+constexpr int kSplitPlanMaxSplits = 3;   // (3 and 4 splits measure alike where 4 fit; 4 is the less steady)
 constexpr int kSplitMinKTiles = 24;      // k-tiles of 32 per split at least
 constexpr int kSplitTargetGroups = 256;  // one workgroup per compute unit
 

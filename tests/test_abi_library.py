@@ -77,7 +77,7 @@ def test_other_entry_points_argument_checks(lib):
     assert lib.stof_gemm_bias_act(P, P, None, P, 64, 64, 64, 64, 64, 9, None) == -3      # activation
     assert lib.stof_gemm_bias_act(P, P + 8, None, P, 64, 64, 64, 64, 64, 0, None) == -4
     # split-K form: A, Wt, bias, C, M, N, K, lda, ldc, act, splits, workspace, bytes, stream
-    assert lib.stof_gemm_bias_act_splitk_plan(512, 768, 3072) == 4       # 48 tiles of 64 x 128, 96 k-tiles
+    assert lib.stof_gemm_bias_act_splitk_plan(512, 768, 3072) == 3       # 48 tiles of 64 x 128, 96 k-tiles
     assert lib.stof_gemm_bias_act_splitk_plan(1024, 768, 3072) == 2      # 96 tiles: two splits stay within 256 workgroups
     assert lib.stof_gemm_bias_act_splitk_plan(512, 768, 768) == 1        # 24 k-tiles: too short to split
     assert lib.stof_gemm_bias_act_splitk_plan(2048, 768, 3072) == 1      # 192 tiles already
