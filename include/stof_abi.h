@@ -250,7 +250,7 @@ int stof_gemm_bias_act(const void* A, const void* Wt, const void* bias, void* C,
  * stof_gemm_bias_act_splitk_plan returns the number of splits this library would use for a shape,
  * 1 where stof_gemm_bias_act is the form to call (its rule: the plain form would run at most 128
  * tiles of 128 x 128, the split grid stays within 256 workgroups and 3 splits, and every split
- * keeps at least 24 k-tiles of 32).
+ * keeps at least 24 k-tiles of 32; or 129 .. 192 tiles of 128 x 128 with K >= 3072: 2 splits).
  */
 int stof_gemm_bias_act_splitk_plan(int64_t M, int64_t N, int64_t K);
 int64_t stof_gemm_bias_act_splitk_workspace_bytes(int64_t M, int64_t N, int splits);

@@ -125,6 +125,79 @@ __device__ __forceinline__ void store_wave_block(const GemmParams& p, const floa
   }
 }
 
+// Split-K hand-over for one wave (launches with p.splits > 1: the grid is `splits` copies of the
+// tile grid, copy z has multiplied the z-th range of k-tiles).  The wave hands its partial sums
+// (acc, 32 * MT floats per lane) to the wave of the same place in the split that finishes last:
+// 8-byte device-scope stores (written through to memory, 512 contiguous bytes per instruction), a
+// wait until they are acknowledged, then one count on the (tile, wave) counter.  The wave that
+// counts last adds the partial sums in the order of z - its own from registers - so the result
+// does not depend on which split came last, puts the counter back to zero for the next launch and
+// returns true with the total in acc; the others return false and are done.
+template <int MT>
+__device__ __forceinline__ bool splitk_handover(const GemmParams& p, floatx16 (&acc)[2][MT], int64_t tile, int z, int wave, int lane) {
+  typedef unsigned long long u64;
+  constexpr int kSlot = 1024 * MT;   // 8-byte words per (tile, split, wave)
+  u64* mine = reinterpret_cast<u64*>(p.partials) + ((tile * p.splits + z) * 4 + wave) * kSlot + lane;
+#pragma unroll
+  for (int ni = 0; ni < 2; ++ni)
+#pragma unroll
+    for (int mi = 0; mi < MT; ++mi)
+#pragma unroll
+      for (int r = 0; r < 16; r += 2) {
+        // (through scalar copies: a bit cast applied directly to a vector element reads element 0)
+        const float lo = acc[ni][mi][r], hi = acc[ni][mi][r + 1];
+        const u64 v = ((u64)__builtin_bit_cast(unsigned, hi) << 32) | __builtin_bit_cast(unsigned, lo);
+        __hip_atomic_store(mine + ((ni * MT + mi) * 8 + (r >> 1)) * 64, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+  // (relaxed atomics to different addresses are not ordered for the compiler: the empty asm
+  // statements keep the stores above the wait, the count below it and the reads below the count)
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0)
+  asm volatile("" ::: "memory");
+  int* counter = p.counters + tile * 4 + wave;
+  int before = 0;
+  if (lane == 0) before = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  before = __builtin_amdgcn_readfirstlane(before);
+  asm volatile("" ::: "memory");
+  if (before != p.splits - 1) return false;
+  floatx16 sum[2][MT];
+#pragma unroll
+  for (int ni = 0; ni < 2; ++ni)
+#pragma unroll
+    for (int mi = 0; mi < MT; ++mi)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) sum[ni][mi][r] = 0.f;
+  const u64* slot0 = reinterpret_cast<const u64*>(p.partials) + ((tile * p.splits) * 4 + wave) * kSlot + lane;
+  for (int zz = 0; zz < p.splits; ++zz) {
+    if (zz == z) {
+#pragma unroll
+      for (int ni = 0; ni < 2; ++ni)
+#pragma unroll
+        for (int mi = 0; mi < MT; ++mi)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) sum[ni][mi][r] += acc[ni][mi][r];
+    } else {
+      const u64* src = slot0 + (int64_t)zz * 4 * kSlot;
+#pragma unroll
+      for (int ni = 0; ni < 2; ++ni)
+#pragma unroll
+        for (int mi = 0; mi < MT; ++mi)
+#pragma unroll
+          for (int r = 0; r < 16; r += 2) {
+            const u64 v = __hip_atomic_load(src + ((ni * MT + mi) * 8 + (r >> 1)) * 64, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            sum[ni][mi][r] += __builtin_bit_cast(float, (unsigned)(v & 0xffffffffull));
+            sum[ni][mi][r + 1] += __builtin_bit_cast(float, (unsigned)(v >> 32));
+          }
+    }
+  }
+  if (lane == 0) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+  for (int ni = 0; ni < 2; ++ni)
+#pragma unroll
+    for (int mi = 0; mi < MT; ++mi) acc[ni][mi] = sum[ni][mi];
+  return true;
+}
+
 // ------------------------------------------------------------------------------------------
 // C[M,N] = act(A[M,K] @ Wt[N,K]^T + bias[N]);  tile 128 (tokens) x 128 (features) x 64 (K),
 // 4 waves as 2 x 2, each 64 tokens x 64 features = 2 x 2 MFMA tiles.
@@ -134,7 +207,7 @@ constexpr int kGT = 128;            // tile edge (tokens and features)
 constexpr int kGK = 64;             // K per tile
 constexpr int kGTile = kGT * kGK * 2;   // bytes per operand tile (16 KB)
 
-template <int ACT>
+template <int ACT, bool SK = false>
 __global__ __launch_bounds__(256) void gemm_bias_act_kernel(const GemmParams p) {
   __shared__ __attribute__((aligned(1024))) unsigned char a_lds0[kGTile];
   __shared__ __attribute__((aligned(1024))) unsigned char a_lds1[kGTile];
@@ -146,9 +219,13 @@ __global__ __launch_bounds__(256) void gemm_bias_act_kernel(const GemmParams p) 
   const int j32 = lane & 31, g = lane >> 5;
   const int wm = wave >> 1, wn = wave & 1;
 
+  // split-K: the grid is `splits` copies of the tile grid, copy z takes the z-th range of k-tiles
+  const int tile_grid = (int)(8u * (unsigned)((p.tiles_m + 7) / 8) * (unsigned)p.tiles_n);
+  const int z = SK ? (int)blockIdx.x / tile_grid : 0;
   int tm, tn;
-  if (!raster_tile(blockIdx.x, p.tiles_m, p.tiles_n, tm, tn)) return;
+  if (!raster_tile((int)blockIdx.x - z * tile_grid, p.tiles_m, p.tiles_n, tm, tn)) return;
   const int m0 = tm * kGT, n0 = tn * kGT;
+  const int kt_first = SK ? z * p.nk_split : 0;
 
   // DMA: 16 instructions of 8 rows per operand tile; wave w issues 4w..4w+3.
   uint32_t a_off[4], w_off[4];
@@ -161,7 +238,7 @@ __global__ __launch_bounds__(256) void gemm_bias_act_kernel(const GemmParams p) 
   }
   const __amdgpu_buffer_rsrc_t a_rs = tile_rsrc(p.A + (int64_t)m0 * p.lda), w_rs = tile_rsrc(p.W + (int64_t)n0 * p.K);
   auto issue = [&](int kt, lds_byte* ad, lds_byte* wd) {
-    const uint32_t koff = (uint32_t)kt * (kGK * 2);
+    const uint32_t koff = (uint32_t)(kt_first + kt) * (kGK * 2);
 #pragma unroll
     for (int i = 0; i < 4; ++i) dma16b(a_rs, a_off[i], koff, ad + (4 * wave + i) * 1024);
 #pragma unroll
@@ -203,7 +280,7 @@ __global__ __launch_bounds__(256) void gemm_bias_act_kernel(const GemmParams p) 
     }
   };
 
-  const int nk = p.K / kGK;
+  const int nk = SK ? min(p.nk_split, p.K / kGK - kt_first) : p.K / kGK;
   issue(0, (lds_byte*)a_lds0, (lds_byte*)w_lds0);
   for (int kt = 0; kt < nk; kt += 2) {
     __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): this wave's share of tile kt landed
@@ -219,6 +296,9 @@ __global__ __launch_bounds__(256) void gemm_bias_act_kernel(const GemmParams p) 
   }
 
   __syncthreads();   // every wave is done with the operand tiles
+  if constexpr (SK) {
+    if (!splitk_handover<2>(p, acc, (int64_t)tm * p.tiles_n + tn, z, wave, lane)) return;
+  }
   store_wave_block<ACT, 2>(p, acc, (lds_byte*)a_lds0 + wave * 4096, m0 + 64 * wm, n0 + 64 * wn, lane);
 }
 
@@ -373,64 +453,9 @@ __global__ __launch_bounds__(256, 2) void gemm_bias_act_ring_kernel(const GemmPa
 
   wg_barrier();   // every wave has read its last fragments (and no load is in flight): the ring is free
   if constexpr (SK) {
-    // Each wave hands its 32 x 64 partial sums (32 floats per lane) to the wave of the same place
-    // in the split that finishes last: 8-byte device-scope stores (written through to memory, 512
-    // contiguous bytes per instruction), a wait until they are acknowledged, then one count on the
-    // (tile, wave) counter.  The wave that counts last adds the partial sums in the order of z -
-    // its own from registers - so the result does not depend on which split came last, applies
-    // the epilogue, and puts the counter back to zero for the next launch.
-    typedef unsigned long long u64;
-    const int64_t tile = (int64_t)tm * p.tiles_n + tn;
-    u64* mine = reinterpret_cast<u64*>(p.partials) + ((tile * p.splits + z) * 4 + wave) * 1024 + lane;
-#pragma unroll
-    for (int ni = 0; ni < 2; ++ni)
-#pragma unroll
-      for (int r = 0; r < 16; r += 2) {
-        // (through scalar copies: a bit cast applied directly to a vector element reads element 0)
-        const float lo = acc[ni][0][r], hi = acc[ni][0][r + 1];
-        const u64 v = ((u64)__builtin_bit_cast(unsigned, hi) << 32) | __builtin_bit_cast(unsigned, lo);
-        __hip_atomic_store(mine + (8 * ni + (r >> 1)) * 64, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      }
-    // (relaxed atomics to different addresses are not ordered for the compiler: the empty asm
-    // statements keep the stores above the wait, the count below it and the reads below the count)
-    asm volatile("" ::: "memory");
-    __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
-    asm volatile("" ::: "memory");
-    int* counter = p.counters + tile * 4 + wave;
-    int before = 0;
-    if (lane == 0) before = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    before = __builtin_amdgcn_readfirstlane(before);
-    asm volatile("" ::: "memory");
-    if (before != p.splits - 1) return;
-    floatx16 sum[2][1];
-#pragma unroll
-    for (int ni = 0; ni < 2; ++ni)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) sum[ni][0][r] = 0.f;
-    const u64* slot0 = reinterpret_cast<const u64*>(p.partials) + ((tile * p.splits) * 4 + wave) * 1024 + lane;
-    for (int zz = 0; zz < p.splits; ++zz) {
-      if (zz == z) {
-#pragma unroll
-        for (int ni = 0; ni < 2; ++ni)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) sum[ni][0][r] += acc[ni][0][r];
-      } else {
-        const u64* src = slot0 + (int64_t)zz * 4 * 1024;
-#pragma unroll
-        for (int ni = 0; ni < 2; ++ni)
-#pragma unroll
-          for (int r = 0; r < 16; r += 2) {
-            const u64 v = __hip_atomic_load(src + (8 * ni + (r >> 1)) * 64, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            sum[ni][0][r] += __builtin_bit_cast(float, (unsigned)(v & 0xffffffffull));
-            sum[ni][0][r + 1] += __builtin_bit_cast(float, (unsigned)(v >> 32));
-          }
-      }
-    }
-    if (lane == 0) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    store_wave_block<ACT, 1>(p, sum, (lds_byte*)a_lds + wave * 4096, m0 + 32 * wt, n0 + 64 * wf, lane);
-  } else {
-    store_wave_block<ACT, 1>(p, acc, (lds_byte*)a_lds + wave * 4096, m0 + 32 * wt, n0 + 64 * wf, lane);
+    if (!splitk_handover<1>(p, acc, (int64_t)tm * p.tiles_n + tn, z, wave, lane)) return;
   }
+  store_wave_block<ACT, 1>(p, acc, (lds_byte*)a_lds + wave * 4096, m0 + 32 * wt, n0 + 64 * wf, lane);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -1002,18 +1027,24 @@ constexpr int kSplitMaxSplits = 8;       // what the entry point takes
 // 2048 x 768 x 3072 22.3 | 24.6 27.3 25.3; 512 x 768 x 768 7.7 | 8.6 8.7 8.9; 512 x 2304 x 768 8.3 | 12.4 12.0:
 // it pays while the grid stays within one workgroup per compute unit and a split keeps 24 k-tiles;
 // the hand-over (stores acknowledged, count, reads) costs about 5 us.
+// Between kSmallMaxTiles and kSplitMidMaxTiles tiles of 128 x 128 (fewer workgroups than compute
+// units) two splits of a long K pay on that form as well, by less, because a workgroup hands over
+// 64 KB: 3072 x 768 x 3072 34.4 -> 28.0, 4096 x 768 x 3072 34.8 -> 29.6, 3072 x 1024 x 4096 40.2 -> 36.1;
+// 5120 x 768 x 3072 (240 tiles) 35.7 -> 33.4, 4096 x 1024 x 4096 (256) 43.2 -> 42.6, K 1536: 17.0 -> 19.7.
+constexpr int kSplitMidMaxTiles = 192;
+constexpr int kSplitMidMinK = 3072;
 constexpr int kSplitPlanMaxSplits = 3;   // (3 and 4 splits measure alike where 4 fit; 4 is the less steady)
 constexpr int kSplitMinKTiles = 24;      // k-tiles of 32 per split at least
 constexpr int kSplitTargetGroups = 256;  // one workgroup per compute unit
 
 // How many ways stof_gemm_bias_act_splitk should split K for this shape; 1 = the plain form is the
-// one to use.  Only where the plain GEMM runs its 64-token form (at most kSmallMaxTiles tiles of
+// one to use.  Mostly where the plain GEMM runs its 64-token form (at most kSmallMaxTiles tiles of
 // 128 x 128): there a workgroup's K loop runs at the latency of its loads and most compute units
 // have no workgroup at all.
 extern "C" int stof_gemm_bias_act_splitk_plan(int64_t M, int64_t N, int64_t K) {
   if (M <= 0 || N <= 0 || K <= 0 || K % kGK != 0) return 1;
   const int64_t tiles128 = ((M + kGT - 1) / kGT) * ((N + kGT - 1) / kGT);
-  if (tiles128 > kSmallMaxTiles) return 1;
+  if (tiles128 > kSmallMaxTiles) return (tiles128 <= kSplitMidMaxTiles && K >= kSplitMidMinK) ? 2 : 1;
   const int64_t tiles64 = ((M + 63) / 64) * ((N + kWFeat - 1) / kWFeat);
   int64_t splits = kSplitTargetGroups / tiles64;
   if (splits > (K / 32) / kSplitMinKTiles) splits = (K / 32) / kSplitMinKTiles;
@@ -1025,7 +1056,27 @@ extern "C" int64_t stof_gemm_bias_act_splitk_workspace_bytes(int64_t M, int64_t 
   if (M <= 0 || N <= 0 || splits < 1 || splits > kSplitMaxSplits) return 0;
   const int64_t tiles64 = ((M + 63) / 64) * ((N + kWFeat - 1) / kWFeat);
   if (tiles64 > kSplitMaxTiles) return 0;
-  return kSplitPartialsOffset + tiles64 * splits * (64 * kWFeat * 4);
+  // (either form: fp32 partial sums of the output padded to whole 128 x 128 tiles, per split)
+  return kSplitPartialsOffset + ((M + kGT - 1) / kGT) * ((N + kGT - 1) / kGT) * splits * (kGT * kGT * 4);
+}
+
+template <bool SMALL>
+int launch_splitk(const GemmParams& p, int act, unsigned groups, hipStream_t st) {
+  const dim3 grid(groups), block(256);
+  switch (act) {
+#define STOF_SPLITK_CASE(A) \
+    case A: \
+      if (SMALL) hipLaunchKernelGGL((gemm_bias_act_ring_kernel<A, kSmallStages, true>), grid, block, 0, st, p); \
+      else hipLaunchKernelGGL((gemm_bias_act_kernel<A, true>), grid, block, 0, st, p); \
+      break;
+    STOF_SPLITK_CASE(STOF_ACT_NONE)
+    STOF_SPLITK_CASE(STOF_ACT_GELU_ERF)
+    STOF_SPLITK_CASE(STOF_ACT_GELU_TANH)
+    STOF_SPLITK_CASE(STOF_ACT_RELU)
+#undef STOF_SPLITK_CASE
+    default: return STOF_ERR_UNSUPPORTED;
+  }
+  return stof_check_launch();
 }
 
 extern "C" int stof_gemm_bias_act_splitk(const void* A, const void* Wt, const void* bias, void* C,
@@ -1043,22 +1094,19 @@ extern "C" int stof_gemm_bias_act_splitk(const void* A, const void* Wt, const vo
   GemmParams p;
   p.A = (const half_t*)A; p.W = (const half_t*)Wt; p.bias = (const half_t*)bias; p.C = (half_t*)C;
   p.M = (int)M; p.N = (int)N; p.K = (int)K; p.lda = (int)lda; p.ldc = (int)ldc;
-  p.tiles_m = (int)((M + 63) / 64); p.tiles_n = (int)((N + kWFeat - 1) / kWFeat);
-  const int nk = (int)(K / 32);
-  p.nk_split = (nk + splits - 1) / splits;
-  p.splits = (nk + p.nk_split - 1) / p.nk_split;   // (every split has at least one k-tile)
   p.counters = reinterpret_cast<int*>(workspace);
   p.partials = reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) + kSplitPartialsOffset);
-  const dim3 grid(raster_grid(p.tiles_m, p.tiles_n) * (unsigned)p.splits), block(256);
+  // The tile form follows the plain GEMM's rule: 64-token tiles (k-tiles of 32) where the
+  // 128 x 128 form (k-tiles of 64) would have at most kSmallMaxTiles workgroups.
+  const bool small = ((M + kGT - 1) / kGT) * ((N + kGT - 1) / kGT) <= kSmallMaxTiles;
+  const int tile_m = small ? 64 : kGT, tile_k = small ? 32 : kGK;
+  p.tiles_m = (int)((M + tile_m - 1) / tile_m); p.tiles_n = (int)((N + kGT - 1) / kGT);
+  const int nk = (int)(K / tile_k);
+  p.nk_split = (nk + splits - 1) / splits;
+  p.splits = (nk + p.nk_split - 1) / p.nk_split;   // (every split has at least one k-tile)
+  const unsigned groups = raster_grid(p.tiles_m, p.tiles_n) * (unsigned)p.splits;
   hipStream_t st = (hipStream_t)stream;
-  switch (act) {
-    case STOF_ACT_NONE: hipLaunchKernelGGL((gemm_bias_act_ring_kernel<STOF_ACT_NONE, kSmallStages, true>), grid, block, 0, st, p); break;
-    case STOF_ACT_GELU_ERF: hipLaunchKernelGGL((gemm_bias_act_ring_kernel<STOF_ACT_GELU_ERF, kSmallStages, true>), grid, block, 0, st, p); break;
-    case STOF_ACT_GELU_TANH: hipLaunchKernelGGL((gemm_bias_act_ring_kernel<STOF_ACT_GELU_TANH, kSmallStages, true>), grid, block, 0, st, p); break;
-    case STOF_ACT_RELU: hipLaunchKernelGGL((gemm_bias_act_ring_kernel<STOF_ACT_RELU, kSmallStages, true>), grid, block, 0, st, p); break;
-    default: return STOF_ERR_UNSUPPORTED;
-  }
-  return stof_check_launch();
+  return small ? launch_splitk<true>(p, act, groups, st) : launch_splitk<false>(p, act, groups, st);
 }
 
 extern "C" int stof_gemm_bias_res_ln(const void* A, const void* Wt, const void* bias, const void* residual,

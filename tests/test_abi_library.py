@@ -82,8 +82,10 @@ def test_other_entry_points_argument_checks(lib):
     assert lib.stof_gemm_bias_act_splitk_plan(512, 768, 768) == 1        # 24 k-tiles: too short to split
     assert lib.stof_gemm_bias_act_splitk_plan(2048, 768, 3072) == 1      # 192 tiles already
     assert lib.stof_gemm_bias_act_splitk_plan(8192, 3072, 768) == 1 and lib.stof_gemm_bias_act_splitk_plan(512, 768, 100) == 1
+    assert lib.stof_gemm_bias_act_splitk_plan(4096, 768, 3072) == 2      # 192 tiles of 128 x 128 on 256 compute units, long K
+    assert lib.stof_gemm_bias_act_splitk_plan(4096, 768, 768) == 1 and lib.stof_gemm_bias_act_splitk_plan(8192, 768, 3072) == 1
     sneed = lib.stof_gemm_bias_act_splitk_workspace_bytes(512, 768, 4)
-    assert sneed == 4096 * 16 + 48 * 4 * 64 * 128 * 4
+    assert sneed == 4096 * 16 + 24 * 4 * 128 * 128 * 4      # counters, then 4 splits of 4 x 6 tiles of 128 x 128 floats
     assert lib.stof_gemm_bias_act_splitk_workspace_bytes(512, 768, 9) == 0 and lib.stof_gemm_bias_act_splitk_workspace_bytes(1 << 20, 768, 2) == 0
     sk = lambda **kw: lib.stof_gemm_bias_act_splitk(kw.get("A", P), P, None, P, kw.get("M", 512), 768, kw.get("K", 3072), 3072, 768,
                                                     kw.get("act", 0), kw.get("splits", 4), kw.get("ws", P), kw.get("wsb", sneed), None)

@@ -50,7 +50,10 @@ def test_gemm_bias_act(M, N, K, act):
 # splits 1 = one workgroup per tile.  (129, 136, 128): 4 k-tiles, so 3 splits become 2 of 2 k-tiles;
 # (1, 8, 64): 2 k-tiles; (512, 768, 3072): the FFN-out product of a 512-token BERT-base layer;
 # (200, 520, 1088): ragged edges, 34 k-tiles over 8 splits (5 + 5 + ... + 4).
-@pytest.mark.parametrize("M,N,K", [(512, 768, 3072), (200, 520, 1088), (129, 136, 128), (1, 8, 64)])
+# (3072, 768, 3072) and (2500, 1032, 704): more than 128 tiles of 128 x 128, so the split runs on that
+# tile form (k-tiles of 64; 11 of them over 3 splits = 4 + 4 + 3, ragged edges).
+@pytest.mark.parametrize("M,N,K", [(512, 768, 3072), (200, 520, 1088), (129, 136, 128), (1, 8, 64),
+                                   (3072, 768, 3072), (2500, 1032, 704)])
 @pytest.mark.parametrize("splits", [1, 2, 3, 8])
 def test_gemm_split_k(M, N, K, splits):
     print(f"gemm split-K M{M} N{N} K{K} splits {splits}", flush=True)
