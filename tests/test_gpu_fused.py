@@ -88,10 +88,10 @@ def test_gemm_strided_rows_and_no_bias():
     W = _rand(128, 72, seed=5, scale=0.1)
     got = fused.gemm_bias_act(xs, fused.pack_weight(W.cuda()), None, "none")
     _close(got, x[:, :128].float() @ W.float(), "strided")
-    big = _rand(49152, 832, seed=15)             # wide form, row pitch 832, K = 768
+    big = _rand(49152, 832, seed=15)             # many bands of the tile order, row pitch 832, K = 768
     Wb = _rand(768, 512, seed=16, scale=0.05)
     _close(fused.gemm_bias_act(big.cuda()[:, :768], fused.pack_weight(Wb.cuda()), None, "none"),
-           big[:, :768].float() @ Wb.float(), "strided, wide form")
+           big[:, :768].float() @ Wb.float(), "strided, 49152 rows")
     ident = torch.eye(64).half()                  # closed form: W = I returns the input
     _close(fused.gemm_bias_act(x.cuda()[:, :64].contiguous(), ident.cuda(), None, "none"), x[:, :64], "identity")
 
