@@ -160,11 +160,13 @@ class CapturedForward:
         return self.y
 
 
-def eager_layer(x, w, mask, n_heads, eps=1e-12):
+def eager_layer(x, w, mask, n_heads, eps=1e-12, gelu="erf"):
     """The same layer in plain PyTorch ops on x's device (matmul, add, softmax, F.gelu,
     F.layer_norm, permute + contiguous exactly as src/benchmk_end2end.py:31-88): the unfused
-    comparator the fused layer is timed against.  ``mask`` [B,S,S] or [1,S,S] of 0/1."""
+    comparator the fused layer is timed against.  ``mask`` [B,S,S] or [1,S,S] of 0/1.
+    ``gelu``: "erf" (BERT, :81), "tanh" (GPT, :25-26,144) or "relu" (T5, :206)."""
     import torch.nn.functional as F
+    act = {"erf": F.gelu, "tanh": lambda t: F.gelu(t, approximate="tanh"), "relu": F.relu}[gelu]
     B, S, D = x.shape
     hd = D // n_heads
     qkv = torch.matmul(x, w["W_qkv"]) + w["b_qkv"]
@@ -179,6 +181,6 @@ def eager_layer(x, w, mask, n_heads, eps=1e-12):
     h = torch.matmul(h, w["W_o"]) + w["b_o"]
     h = F.layer_norm(h + x, (D,), weight=w["g1"], bias=w["be1"], eps=eps)
     r = h
-    h = F.gelu(torch.matmul(h, w["W_1"]) + w["b_1"])
+    h = act(torch.matmul(h, w["W_1"]) + w["b_1"])
     h = torch.matmul(h, w["W_2"]) + w["b_2"]
     return F.layer_norm(h + r, (D,), weight=w["g2"], bias=w["be2"], eps=eps)

@@ -332,3 +332,19 @@ def test_captured_stack_replays_match_eager_launches():
         want0 = oe.bert_layer(want0, w, mask.float(), H, eps=1e-12, round_fp16=mode)
     _close(run(xs[0]), want0, "captured stack vs fp16-storing oracle")
 
+
+
+@pytest.mark.parametrize("model,mask_id,block", [("bert_small", 3, 64), ("gpt", 1, 64), ("t5", 2, 32)])
+def test_end2end_example_runs(model, mask_id, block):
+    """The example with the reference's end-to-end command line: fused stack against plain PyTorch
+    ops (erf GELU, tanh GELU, ReLU feed-forward; 32 x 32 LUT blocks re-tiled for the T5 run)."""
+    import subprocess, sys, os
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    script = os.path.join(root, "sc25-stof-ad_amd", "examples", "end2end.py")
+    r = subprocess.run([sys.executable, script, "--model", model, "--mask_id", str(mask_id), "--block_m", str(block), "--block_n", str(block),
+                        "--batch_size", "2", "--seq_len", "256", "--warmup_iters", "2", "--running_iters", "3"],
+                       capture_output=True, text=True, timeout=110)
+    assert r.returncode == 0, r.stdout + r.stderr
+    assert "STOF            :" in r.stdout and "Torch Native    :" in r.stdout
+    line = [l for l in r.stdout.splitlines() if l.startswith("max abs difference")][0]
+    assert float(line.split(":")[1]) < 5e-2, r.stdout      # 6 / 12 layers of fp16 kernels on both sides; observed 4e-3 .. 1.6e-2
