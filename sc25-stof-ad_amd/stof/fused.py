@@ -211,7 +211,9 @@ def ln_gemm_form(M, N, K):
     the bias+residual+LayerNorm kernel; the pre-normalisation values pass through HBM as fp16), or
     "row" where K is a multiple of 32 but not of 64, which only that kernel takes."""
     tiles = ((M + 127) // 128) * (N // 128)
-    if cluster_supported(N, K) and tiles >= CLUSTER_MIN_TILES:
+    # (where the tiled GEMM would split K - 129 .. 192 tiles and a long K - it overtakes the cluster
+    # form, which cannot: 4096 x 768 x 3072 36.5 us as two launches against 39.9)
+    if cluster_supported(N, K) and tiles >= CLUSTER_MIN_TILES and _lib.lib().stof_gemm_bias_act_splitk_plan(M, N, K) == 1:
         return "cluster"
     return "split" if K % 64 == 0 else "row"
 
