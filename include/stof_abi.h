@@ -242,7 +242,7 @@ int stof_gemm_bias_act(const void* A, const void* Wt, const void* bias, void* C,
  * workgroup leaves fp32 partial sums in `workspace`; the one that finishes last adds them in the
  * order of the splits (so the result does not depend on the order of arrival), applies bias and
  * activation and writes C.  Arguments and rules as stof_gemm_bias_act, plus:
- *   splits      2 .. 8 (fewer are used when K / 32 has fewer than that many k-tiles);
+ *   splits      2 .. 8 (fewer are used when K / 64 has fewer than that many k-tiles);
  *   workspace   at least stof_gemm_bias_act_splitk_workspace_bytes(M, N, splits) bytes, 16-byte
  *               aligned, ZERO at first use; every call leaves its counters zero again, so one
  *               workspace serves any sequence of calls on one stream (calls that overlap in time
@@ -250,7 +250,7 @@ int stof_gemm_bias_act(const void* A, const void* Wt, const void* bias, void* C,
  * stof_gemm_bias_act_splitk_plan returns the number of splits this library would use for a shape,
  * 1 where stof_gemm_bias_act is the form to call (its rule: the plain form would run at most 128
  * tiles of 128 x 128, the split grid stays within 256 workgroups and 3 splits, and every split
- * keeps at least 24 k-tiles of 32; or 129 .. 192 tiles of 128 x 128 with K >= 3072: 2 splits).
+ * keeps K >= 768; or 129 .. 192 tiles of 128 x 128 with K >= 3072: 2 splits).
  */
 int stof_gemm_bias_act_splitk_plan(int64_t M, int64_t N, int64_t K);
 int64_t stof_gemm_bias_act_splitk_workspace_bytes(int64_t M, int64_t N, int splits);

@@ -303,18 +303,23 @@ __global__ __launch_bounds__(256) void gemm_bias_act_kernel(const GemmParams p) 
 }
 
 // ------------------------------------------------------------------------------------------
-// Ring form of the same GEMM for small token counts: tile 64 (tokens) x 128 (features) x 32 (K),
+// Ring form of the same GEMM for small token counts: tile 64 (tokens) x 128 (features) x KT (K),
 // 4 waves as 2 x 2, each 32 tokens x 64 features = 2 MFMA tiles; four times the workgroups of the
-// 128 x 128 form.  The K loop is a ring of NS = 4 stages filled by direct-to-LDS loads (three
-// tiles in flight per workgroup) and is software pipelined inside the wave: the form for token
-// counts that give the 128 x 128 form less than one workgroup per two compute units, where the
-// K loop of each workgroup runs at the latency of its loads (512 tokens, N 768, K 3072:
-// 36 -> 23 us).  With SK the K dimension is split over several workgroups per tile as well.
+// 128 x 128 form.  The K loop is a ring of NS stages filled by direct-to-LDS loads (NS - 1 tiles
+// in flight per workgroup) and is software pipelined inside the wave: the form for token counts
+// that give the 128 x 128 form less than one workgroup per two compute units, where the K loop
+// of each workgroup runs at the latency of its loads.  Launched with KT = 64, NS = 3 (72 KB of
+// LDS, two workgroups per compute unit, 48 KB in flight per workgroup, one barrier per 64 of K);
+// KT = 32, NS = 4 (36 KB in flight, a barrier per 32 of K) was the first version: 512 tokens,
+// N 768, K 3072 22.1 -> 17.9 us, N 1024, K 4096 27.6 -> 22.4, 2048 x 768 x 3072 22.6 -> 18.8;
+// K 768 unchanged (8 us, the pace of the launches).  NS = 4 with KT = 64 measures like NS = 3,
+// NS = 2 is 50 % slower.  With SK the K dimension is split over several workgroups per tile as well.
 // (The same structure with 256-token tiles and three stages - 0.75 KB of LDS reads per MFMA
 // instead of 1 KB - was the form for large grids until the 128 x 128 form got buffer-resource
 // loads and the banded tile order; it is no longer part of the library.)
 // ------------------------------------------------------------------------------------------
 constexpr int kWFeat = 128;
+constexpr int kSmallKT = 64;          // K per tile of the ring form as it is launched
 
 // 64-byte rows: chunk c of row r sits at position c ^ ((r >> 2) & 3); 16 rows fill 1 KB.
 __device__ __forceinline__ int swz4(int row) { return (row >> 2) & 3; }
@@ -322,12 +327,17 @@ __device__ __forceinline__ int swz4(int row) { return (row >> 2) & 3; }
 // s_waitcnt immediate that waits for the vector-memory counter only (lgkmcnt 15, expcnt 7)
 constexpr int vmcnt_imm(int n) { return (n & 15) | ((n >> 4) << 14) | 0x0F70; }
 
-template <int ACT, int NS, bool SK = false>
+template <int ACT, int NS, bool SK = false, int KT = kSmallKT>
 __global__ __launch_bounds__(256, 2) void gemm_bias_act_ring_kernel(const GemmParams p) {
-  constexpr int kK = 32;
+  static_assert(KT == 32 || KT == 64, "K per tile");
+  constexpr int kK = KT;
   constexpr int kTok = 64;                // tokens per workgroup: two waves of 32
-  constexpr int kLoads = 3;               // load instructions per wave per tile
-  constexpr int kATile = kTok * kK * 2, kWTile = kWFeat * kK * 2;   // 4 KB, 8 KB
+  constexpr int kPitch = kK * 2;          // bytes per tile row
+  constexpr int kRowsPI = 1024 / kPitch;  // tile rows per load instruction (1 KB)
+  constexpr int kAI = kTok / kRowsPI / 4, kWI = kWFeat / kRowsPI / 4;   // load instructions per wave: A tile, W tile
+  constexpr int kLoads = kAI + kWI;       // per wave per tile
+  constexpr int kKS = kK / 16;            // k-steps (MFMA depth 16) per tile
+  constexpr int kATile = kTok * kPitch, kWTile = kWFeat * kPitch;   // 4 / 8 KB, 8 / 16 KB
   // Ring of NS stages: NS tiles are in flight or in use at any time, so a tile has NS - 1 tile
   // times to arrive.  (The fragment reads below are asm, so the compiler does not order them
   // against the direct-to-LDS loads and one array per operand is enough.)
@@ -347,36 +357,43 @@ __global__ __launch_bounds__(256, 2) void gemm_bias_act_ring_kernel(const GemmPa
   const int m0 = tm * kTok, n0 = tn * kWFeat;
   const int kt_first = SK ? z * p.nk_split : 0;
 
-  // Loads: one instruction = 16 rows of 64 B.  A tile: 4 instructions (one per wave), W tile: 8
-  // (2 per wave).  Rows past the edge re-read the last row.  Plain global addresses: the K loop
-  // runs at the latency of its loads, and the buffer-resource form that the 128 x 128 kernel
-  // gains from measured 10-25 % slower here (512 x 3072 x 768: 11.4 vs 9.1 us).
-  const int drow = lane >> 2;
-  uint32_t a_off, w_off[2];
-  {
-    const int trow = 16 * wave + drow;
-    a_off = (uint32_t)min(trow, p.M - 1 - m0) * (uint32_t)(p.lda * 2) + 16 * ((lane & 3) ^ swz4(trow));
+  // Loads: one instruction = 1 KB = kRowsPI tile rows.  Rows past the edge re-read the last row.
+  // 16-byte chunk c of tile row r sits at chunk position c ^ sw(r) (sw: 2 bits for 64-byte rows,
+  // 3 bits for 128-byte rows), so the fragment reads of 32 consecutive rows spread over the banks.
+  // Plain global addresses: the K loop runs at the latency of its loads, and the buffer-resource
+  // form that the 128 x 128 kernel gains from measured 10-25 % slower here (512 x 3072 x 768:
+  // 11.4 vs 9.1 us).
+  auto sw = [](int row) { return KT == 32 ? swz4(row) : swz(row); };
+  constexpr int kChunks = kPitch / 16;
+  const int drow = lane / kChunks, dchunk = lane % kChunks;
+  uint32_t a_off[kAI], w_off[kWI];
+#pragma unroll
+  for (int i = 0; i < kAI; ++i) {
+    const int trow = kRowsPI * (kAI * wave + i) + drow;
+    a_off[i] = (uint32_t)min(trow, p.M - 1 - m0) * (uint32_t)(p.lda * 2) + 16 * (dchunk ^ sw(trow));
   }
 #pragma unroll
-  for (int i = 0; i < 2; ++i) {
-    const int trow = 16 * (2 * wave + i) + drow;
-    w_off[i] = (uint32_t)min(trow, p.N - 1 - n0) * (uint32_t)(p.K * 2) + 16 * ((lane & 3) ^ swz4(trow));
+  for (int i = 0; i < kWI; ++i) {
+    const int trow = kRowsPI * (kWI * wave + i) + drow;
+    w_off[i] = (uint32_t)min(trow, p.N - 1 - n0) * (uint32_t)(p.K * 2) + 16 * (dchunk ^ sw(trow));
   }
   const char* a_first = reinterpret_cast<const char*>(p.A + (int64_t)m0 * p.lda);
   const char* w_first = reinterpret_cast<const char*>(p.W + (int64_t)n0 * p.K);
   auto issue = [&](int kt, int stage) {
-    const uint32_t koff = (uint32_t)(kt_first + kt) * (kK * 2);
+    const uint32_t koff = (uint32_t)(kt_first + kt) * kPitch;
     lds_byte* ad = (lds_byte*)a_lds + stage * kATile;
     lds_byte* wd = (lds_byte*)w_lds + stage * kWTile;
-    __builtin_amdgcn_global_load_lds((gptr_t*)(a_first + koff + a_off), (__attribute__((address_space(3))) void*)(ad + wave * 1024), 16, 0, 0);
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
-      __builtin_amdgcn_global_load_lds((gptr_t*)(w_first + koff + w_off[i]), (__attribute__((address_space(3))) void*)(wd + (2 * wave + i) * 1024), 16, 0, 0);
+    for (int i = 0; i < kAI; ++i)
+      __builtin_amdgcn_global_load_lds((gptr_t*)(a_first + koff + a_off[i]), (__attribute__((address_space(3))) void*)(ad + (kAI * wave + i) * 1024), 16, 0, 0);
+#pragma unroll
+    for (int i = 0; i < kWI; ++i)
+      __builtin_amdgcn_global_load_lds((gptr_t*)(w_first + koff + w_off[i]), (__attribute__((address_space(3))) void*)(wd + (kWI * wave + i) * 1024), 16, 0, 0);
   };
-  // fragment read: row (32*t + j32), chunk 2*ks + g of 4, row pitch 64 B
-  int rd[2];
+  // fragment read: row (32*t + j32), chunk 2*ks + g
+  int rd[kKS];
 #pragma unroll
-  for (int ks = 0; ks < 2; ++ks) rd[ks] = j32 * 64 + (((2 * ks + g) ^ swz4(j32)) << 4);
+  for (int ks = 0; ks < kKS; ++ks) rd[ks] = j32 * kPitch + (((2 * ks + g) ^ sw(j32)) << 4);
 
   floatx16 acc[2][1];   // [feature tile ni][token tile]
 #pragma unroll
@@ -389,10 +406,10 @@ __global__ __launch_bounds__(256, 2) void gemm_bias_act_ring_kernel(const GemmPa
   // counter waits cover that dependency; the LDS counter is waited on by hand (lds_wait).
   auto frags = [&](uint32_t wa, uint32_t aa, half8_t (&wbk)[2], half8_t& xak) {
     asm volatile(
-        "ds_read_b128 %0, %3\n\tds_read_b128 %1, %3 offset:2048\n\t"
+        "ds_read_b128 %0, %3\n\tds_read_b128 %1, %3 offset:%5\n\t"
         "ds_read_b128 %2, %4"
         : "=&v"(wbk[0]), "=&v"(wbk[1]), "=&v"(xak)
-        : "v"(wa), "v"(aa));
+        : "v"(wa), "v"(aa), "n"(32 * kPitch));
   };
   // Wait for the fragment reads of one set: all reads (newer_in_flight false) or all but the
   // 3 reads of the set requested last.  The wait is an asm statement that names the
@@ -416,9 +433,9 @@ __global__ __launch_bounds__(256, 2) void gemm_bias_act_ring_kernel(const GemmPa
     __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_sched_barrier(0);
   };
-  const uint32_t w_rd = (uint32_t)(uintptr_t)(lds_byte*)w_lds + (uint32_t)(64 * wf) * 64;
-  const uint32_t a_rd = (uint32_t)(uintptr_t)(lds_byte*)a_lds + (uint32_t)(32 * wt) * 64;
-  half8_t xa0, wb0[2], xa1, wb1[2];   // fragments of k-step 0 / k-step 1 of a tile
+  const uint32_t w_rd = (uint32_t)(uintptr_t)(lds_byte*)w_lds + (uint32_t)(64 * wf) * kPitch;
+  const uint32_t a_rd = (uint32_t)(uintptr_t)(lds_byte*)a_lds + (uint32_t)(32 * wt) * kPitch;
+  half8_t xa[2], wb[2][2];   // two sets of fragments: k-step ks uses set ks & 1
 
   const int nk = SK ? min(p.nk_split, p.K / kK - kt_first) : p.K / kK;
 #pragma unroll
@@ -427,27 +444,30 @@ __global__ __launch_bounds__(256, 2) void gemm_bias_act_ring_kernel(const GemmPa
   if (nk >= NS) __builtin_amdgcn_s_waitcnt(vmcnt_imm(kLoads * (NS - 1)));   // tile 0 landed
   else __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
   wg_barrier();
-  frags(w_rd + rd[0], a_rd + rd[0], wb0, xa0);
-  // Tile t: the reads of its second k-step go out before the MFMAs of its first; then tile
-  // t+1 is awaited, the barrier lets tile t's stage be refilled with tile t+NS, and the first
-  // fragments of tile t+1 are read while the MFMAs of tile t's second k-step execute.
+  frags(w_rd + rd[0], a_rd + rd[0], wb[0], xa[0]);
+  // Tile t: the reads of k-step ks + 1 go out before the MFMAs of k-step ks; during the last
+  // k-step tile t+1 is awaited, the barrier lets tile t's stage be refilled with tile t+NS, and
+  // the first fragments of tile t+1 are read while the MFMAs of that last k-step execute.
   int cs = 0;   // stage of tile t
   for (int t = 0; t < nk; ++t) {
     const int ns = (cs + 1 == NS) ? 0 : cs + 1;
-    frags(w_rd + cs * kWTile + rd[1], a_rd + cs * kATile + rd[1], wb1, xa1);
-    lds_wait(true, wb0, xa0);
-    mfmas(wb0, xa0);
-    lds_wait(false, wb1, xa1);
+#pragma unroll
+    for (int ks = 0; ks + 1 < kKS; ++ks) {
+      frags(w_rd + cs * kWTile + rd[ks + 1], a_rd + cs * kATile + rd[ks + 1], wb[(ks + 1) & 1], xa[(ks + 1) & 1]);
+      lds_wait(true, wb[ks & 1], xa[ks & 1]);
+      mfmas(wb[ks & 1], xa[ks & 1]);
+    }
+    lds_wait(false, wb[1], xa[1]);   // (kKS is even: the last k-step uses set 1, the next tile starts in set 0)
     if (t + 1 < nk) {
       // tiles t+1 .. t+NS-1 are outstanding; all but the first may stay in flight
       if (t + NS - 1 < nk) __builtin_amdgcn_s_waitcnt(vmcnt_imm(kLoads * (NS - 2)));
       else __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
       wg_barrier();
       if (t + NS < nk) issue(t + NS, cs);
-      frags(w_rd + ns * kWTile + rd[0], a_rd + ns * kATile + rd[0], wb0, xa0);
+      frags(w_rd + ns * kWTile + rd[0], a_rd + ns * kATile + rd[0], wb[0], xa[0]);
     }
     __builtin_amdgcn_sched_barrier(0);
-    mfmas(wb1, xa1);
+    mfmas(wb[1], xa[1]);
     cs = ns;
   }
 
@@ -965,7 +985,7 @@ static_assert(kClusterStatsOffset % 256 == 0, "statistics start on a 256-byte bo
 //    kSmallMaxTiles workgroups.  GPU time, N x K of the BERT-base layer: 512 tokens 14.4 -> 8.9,
 //    14.0 -> 8.4, 14.5 -> 10.6, 36.0 -> 22.9 us; 2048 tokens x N 768: 14.2 -> 8.9, 36.9 -> 23.2 us;
 //    from 192 tiles on (4096 tokens x N 768, 2048 x N 2304) the two are within 5 % either way.
-constexpr int kSmallStages = 4;
+constexpr int kSmallStages = 3;
 constexpr int kSmallMaxTiles = 128;
 
 template <int NS>
@@ -1025,7 +1045,7 @@ constexpr int kSplitMaxSplits = 8;       // what the entry point takes
 // epilogue: 512 x 768 x 3072 22.2 | 15.7 13.7 13.9 19.6 17.0; 128 x 768 x 3072 21.3 | 14.8 13.0 12.7 18.1 15.9;
 // 512 x 1024 x 4096 27.7 | 18.6 16.5 17.3 20.3 21.4; 1024 x 768 x 3072 21.8 | 15.9 22.8 17.7 22.0 20.9;
 // 2048 x 768 x 3072 22.3 | 24.6 27.3 25.3; 512 x 768 x 768 7.7 | 8.6 8.7 8.9; 512 x 2304 x 768 8.3 | 12.4 12.0:
-// it pays while the grid stays within one workgroup per compute unit and a split keeps 24 k-tiles;
+// (taken with 32-wide k-tiles) it pays while the grid stays within one workgroup per compute unit and a split keeps K >= 768;
 // the hand-over (stores acknowledged, count, reads) costs about 5 us.
 // Between kSmallMaxTiles and kSplitMidMaxTiles tiles of 128 x 128 (fewer workgroups than compute
 // units) two splits of a long K pay on that form as well, by less, because a workgroup hands over
@@ -1034,7 +1054,7 @@ constexpr int kSplitMaxSplits = 8;       // what the entry point takes
 constexpr int kSplitMidMaxTiles = 192;
 constexpr int kSplitMidMinK = 3072;
 constexpr int kSplitPlanMaxSplits = 3;   // (3 and 4 splits measure alike where 4 fit; 4 is the less steady)
-constexpr int kSplitMinKTiles = 24;      // k-tiles of 32 per split at least
+constexpr int kSplitMinK = 768;          // K per split at least
 constexpr int kSplitTargetGroups = 256;  // one workgroup per compute unit
 
 // How many ways stof_gemm_bias_act_splitk should split K for this shape; 1 = the plain form is the
@@ -1047,7 +1067,7 @@ extern "C" int stof_gemm_bias_act_splitk_plan(int64_t M, int64_t N, int64_t K) {
   if (tiles128 > kSmallMaxTiles) return (tiles128 <= kSplitMidMaxTiles && K >= kSplitMidMinK) ? 2 : 1;
   const int64_t tiles64 = ((M + 63) / 64) * ((N + kWFeat - 1) / kWFeat);
   int64_t splits = kSplitTargetGroups / tiles64;
-  if (splits > (K / 32) / kSplitMinKTiles) splits = (K / 32) / kSplitMinKTiles;
+  if (splits > K / kSplitMinK) splits = K / kSplitMinK;
   if (splits > kSplitPlanMaxSplits) splits = kSplitPlanMaxSplits;
   return splits < 2 ? 1 : (int)splits;
 }
@@ -1099,7 +1119,7 @@ extern "C" int stof_gemm_bias_act_splitk(const void* A, const void* Wt, const vo
   // The tile form follows the plain GEMM's rule: 64-token tiles (k-tiles of 32) where the
   // 128 x 128 form (k-tiles of 64) would have at most kSmallMaxTiles workgroups.
   const bool small = ((M + kGT - 1) / kGT) * ((N + kGT - 1) / kGT) <= kSmallMaxTiles;
-  const int tile_m = small ? 64 : kGT, tile_k = small ? 32 : kGK;
+  const int tile_m = small ? 64 : kGT, tile_k = small ? kSmallKT : kGK;
   p.tiles_m = (int)((M + tile_m - 1) / tile_m); p.tiles_n = (int)((N + kGT - 1) / kGT);
   const int nk = (int)(K / tile_k);
   p.nk_split = (nk + splits - 1) / splits;

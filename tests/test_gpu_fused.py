@@ -33,8 +33,8 @@ def _rand(*shape, seed=0, scale=1.0):
 #    encoder's shapes, (8155, 3080, 1024) and (2100, 2312, 192) ragged token / feature edges,
 #    (8292, 3072, 1088) an odd number of K tiles; (49152, 512, 768) and (49155, 520, 832): more token
 #    tiles than resident workgroups (several bands of the tile order, padded last band);
-#  small ring (at most 128 tiles of 128 x 128): (64, 2304, 768), (1, 8, 64) fewer K tiles than ring
-#    stages, (129, 136, 128) ragged edges;
+#  small ring (at most 128 tiles of 128 x 128; k-tiles of 64, three stages): (64, 2304, 768), (1, 8, 64)
+#    and (129, 136, 128) fewer k-tiles than ring stages, the latter with ragged edges;
 #  split-K on the small ring (few tiles, long K; the library's rule picks it): (300, 768, 3072).
 @pytest.mark.parametrize("M,N,K", [(8192, 3072, 1024), (8155, 3080, 1024), (8292, 3072, 1088), (8192, 3072, 768),
                                    (49152, 512, 768), (49155, 520, 832),
@@ -47,9 +47,9 @@ def test_gemm_bias_act(M, N, K, act):
     _close(got, oe.gemm_bias_act(x, W, b, act), f"gemm {act}")
 
 
-# splits 1 = one workgroup per tile.  (129, 136, 128): 4 k-tiles, so 3 splits become 2 of 2 k-tiles;
-# (1, 8, 64): 2 k-tiles; (512, 768, 3072): the FFN-out product of a 512-token BERT-base layer;
-# (200, 520, 1088): ragged edges, 34 k-tiles over 8 splits (5 + 5 + ... + 4).
+# splits 1 = one workgroup per tile.  (129, 136, 128): 2 k-tiles of 64, so 3 or 8 splits become 2 of one k-tile;
+# (1, 8, 64): a single k-tile, every split count collapses to one; (512, 768, 3072): the FFN-out product
+# of a 512-token BERT-base layer; (200, 520, 1088): ragged edges, 17 k-tiles over 8 splits (3 + 3 + ... + 2).
 # (3072, 768, 3072) and (2500, 1032, 704): more than 128 tiles of 128 x 128, so the split runs on that
 # tile form (k-tiles of 64; 11 of them over 3 splits = 4 + 4 + 3, ragged edges).
 @pytest.mark.parametrize("M,N,K", [(512, 768, 3072), (200, 520, 1088), (129, 136, 128), (1, 8, 64),
