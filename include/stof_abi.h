@@ -301,6 +301,11 @@ int stof_gemm_bias_res_ln(const void* A, const void* Wt, const void* bias, const
  * time (calls sharing a workspace on different streams race).  The first 4 bytes are an error
  * word: a workgroup whose bounded wait for its partners ran out sets it to 1 (the output is
  * then invalid); it is never set in normal operation and stays set until the caller clears it.
+ * The launch is at most two workgroups per compute unit, which all run at once when the device
+ * is otherwise free; each takes its tiles one after another.  A kernel of another stream that
+ * keeps compute units occupied for longer than the wait lasts (about 0.1 s) can keep part of the
+ * grid from starting and make the waits of the rest run out: check the error word where such
+ * kernels share the device.
  */
 int64_t stof_gemm_bias_res_ln_cluster_workspace_bytes(int64_t M, int64_t N);
 /* Number of polls after which a wave of the cluster kernel stops waiting for its partners and sets the
