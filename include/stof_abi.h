@@ -292,7 +292,7 @@ int stof_gemm_bias_res_ln(const void* A, const void* Wt, const void* bias, const
  * `workspace`, so the pre-normalisation values still never reach HBM while the grid is N / 128
  * times larger.  The form for token counts at which one workgroup per 64 rows leaves compute
  * units idle (8192 tokens at hidden 768 / 1024).
- * N in {256, 512, 768, 1024}; K % 64 == 0; M <= 2^21; A rows at pitch lda, residual rows at pitch
+ * N a multiple of 128 from 256 to 1024; K % 64 == 0; M <= 2^21; A rows at pitch lda, residual rows at pitch
  * ldr, C rows at pitch ldc (elements, multiples of 8); A, Wt, residual, C 16-byte aligned.
  * bias / residual / gamma / beta may be NULL.
  * workspace: stof_gemm_bias_res_ln_cluster_workspace_bytes(M, N) bytes (0 = shape not supported)

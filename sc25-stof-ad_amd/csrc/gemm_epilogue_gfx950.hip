@@ -1185,7 +1185,7 @@ extern "C" int stof_gemm_bias_res_ln_cluster(const void* A, const void* Wt, cons
   if (!A || !Wt || !C || !workspace) return STOF_ERR_NULL_POINTER;
   if (M <= 0 || K <= 0 || K % kGK != 0 || M > kClusterMaxRows || K > (1 << 30) || lda < K || ldc < N || (residual && ldr < N))
     return STOF_ERR_BAD_SHAPE;
-  if (N != 256 && N != 512 && N != 768 && N != 1024) return STOF_ERR_UNSUPPORTED;
+  if (N % kGT != 0 || N < 2 * kGT || N > 8 * kGT) return STOF_ERR_UNSUPPORTED;   // 256, 384, ..., 1024
   if (!stof_aligned16(A) || !stof_aligned16(Wt) || !stof_aligned16(C) || ((uintptr_t)bias & 7) ||
       !stof_aligned16(residual) || ((uintptr_t)gamma & 7) || ((uintptr_t)beta & 7) || ((uintptr_t)workspace & 15) ||
       lda % 8 != 0 || ldc % 8 != 0 || ldr % 8 != 0)
@@ -1211,8 +1211,11 @@ extern "C" int stof_gemm_bias_res_ln_cluster(const void* A, const void* Wt, cons
   hipStream_t st = (hipStream_t)stream;
   switch (p.tiles_n) {
     case 2: hipLaunchKernelGGL(gemm_bias_res_ln_cluster_kernel<2>, grid, block, 0, st, p); break;
+    case 3: hipLaunchKernelGGL(gemm_bias_res_ln_cluster_kernel<3>, grid, block, 0, st, p); break;
     case 4: hipLaunchKernelGGL(gemm_bias_res_ln_cluster_kernel<4>, grid, block, 0, st, p); break;
+    case 5: hipLaunchKernelGGL(gemm_bias_res_ln_cluster_kernel<5>, grid, block, 0, st, p); break;
     case 6: hipLaunchKernelGGL(gemm_bias_res_ln_cluster_kernel<6>, grid, block, 0, st, p); break;
+    case 7: hipLaunchKernelGGL(gemm_bias_res_ln_cluster_kernel<7>, grid, block, 0, st, p); break;
     default: hipLaunchKernelGGL(gemm_bias_res_ln_cluster_kernel<8>, grid, block, 0, st, p); break;
   }
   return stof_check_launch();

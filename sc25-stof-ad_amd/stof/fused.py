@@ -162,7 +162,7 @@ _cluster_ws = {}          # (device index, stream handle) -> zeroed workspace te
 
 def cluster_supported(N, K):
     """Shapes the row-block-cluster form of the LayerNorm GEMM takes."""
-    return N in (256, 512, 768, 1024) and K % 64 == 0
+    return N % 128 == 0 and 256 <= N <= 1024 and K % 64 == 0
 
 
 def _cluster_workspace(dev, stream, nbytes):

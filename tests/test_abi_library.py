@@ -119,7 +119,7 @@ def test_other_entry_points_argument_checks(lib):
     assert cl(ws=None) == -1
     assert cl(K=96) == -2 and cl(lda=512) == -2 and cl(M=(1 << 21) + 1) == -2
     assert cl(wsb=cneed - 1) == -2          # workspace too small
-    assert cl(N=384) == -3 and cl(N=2048, ldc=2048) == -3
+    assert cl(N=320) == -3 and cl(N=128) == -3 and cl(N=2048, ldc=2048) == -3      # multiples of 128 from 256 to 1024
     assert cl(A=P + 8) == -4 and cl(res=P + 8) == -4 and cl(res=P, ldr=772) == -4
     assert lib.stof_rowwise_attn_fwd(P, P, P, P, 7, 0, 0, None, 1, 128, 12, 64, 0, -1, None) == -3
     assert lib.stof_rowwise_attn_fwd(P, P, P, P, 2, 0, 0, None, 1, 128, 12, 64, 0, -1, None) == -1            # mask kind, no bits

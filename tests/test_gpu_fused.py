@@ -161,7 +161,7 @@ def test_fused_op_errors():
     with pytest.raises(StofError):
         fused.gemm_bias_residual_layernorm(_rand(64, 128).cuda(), _rand(384, 128).cuda(), None, None, None, None, form="row")  # N = 384
     with pytest.raises(StofError):
-        fused.gemm_bias_residual_layernorm(_rand(64, 128).cuda(), _rand(384, 128).cuda(), None, None, None, None, form="cluster")
+        fused.gemm_bias_residual_layernorm(_rand(64, 128).cuda(), _rand(320, 128).cuda(), None, None, None, None, form="cluster")
     x2 = _rand(64, 128, seed=22); W2 = _rand(128, 384, seed=23, scale=0.05)     # "auto" takes the two-launch form there
     ones, zeros = torch.ones(384).half(), torch.zeros(384).half()
     _close(fused.gemm_bias_residual_layernorm(x2.cuda(), fused.pack_weight(W2.cuda()), None, None, None, None),

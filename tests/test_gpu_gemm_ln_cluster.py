@@ -26,8 +26,9 @@ def _rand(*shape, seed=0, scale=1.0):
 # (1000, 1024, 1024): ragged last row block; (7, 256, 64): a single partly filled cluster;
 # (40000, 512, 128): more tiles than workgroups (each workgroup walks over several tiles);
 # eps 1e-12 with a row offset of 30: statistics that a one-pass variance would lose
+# (3000, 384, 192) / (5000, 640, 128) / (2050, 896, 64): the odd cluster sizes (3, 5, 7 workgroups per row block)
 @pytest.mark.parametrize("M,N,K", [(8192, 768, 768), (8192, 768, 3072), (8192, 1024, 4096), (1000, 1024, 1024),
-                                   (7, 256, 64), (40000, 512, 128)])
+                                   (7, 256, 64), (40000, 512, 128), (3000, 384, 192), (5000, 640, 128), (2050, 896, 64)])
 @pytest.mark.parametrize("eps", [1e-5, 1e-12])
 def test_gemm_ln_cluster_matches_oracle(M, N, K, eps):
     print(f"gemm_ln cluster M{M} N{N} K{K} eps{eps}", flush=True)
@@ -72,7 +73,7 @@ def test_gemm_ln_cluster_optional_operands_and_errors():
     with pytest.raises(fused.StofError):
         fused.gemm_bias_residual_layernorm(x.cuda()[:, :96].contiguous(), fused.pack_weight(W.cuda()[:96]), None, None, None, None,
                                            1e-5, form="cluster")   # K % 64 != 0
-    Wbad = _rand(128, 384, seed=3)
+    Wbad = _rand(128, 320, seed=3)
     with pytest.raises(fused.StofError):
         fused.gemm_bias_residual_layernorm(x.cuda(), fused.pack_weight(Wbad.cuda()), None, None, None, None, 1e-5, form="cluster")
 
