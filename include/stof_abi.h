@@ -35,6 +35,7 @@
  *                                                           src/triton_template/gemm_add_layernorm.py:78-144
  *                              and matmul + bias + residual + F.layer_norm, src/benchmk_end2end.py:73-76
  *   stof_gemm_bias_res_ln_cluster  the same interfaces (a second launch form of the operator)
+ *   stof_*_dt                  the entry points above with the element format as an argument (fp16 or bfloat16)
  */
 #ifndef STOF_ABI_H
 #define STOF_ABI_H
@@ -316,6 +317,30 @@ int stof_gemm_bias_res_ln_cluster(const void* A, const void* Wt, const void* bia
                                   const void* gamma, const void* beta, void* C,
                                   int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldr, int64_t ldc,
                                   float eps, void* workspace, int64_t workspace_bytes, void* stream);
+
+/*
+ * The four entry points above for tensors in either 16-bit format: the same arguments plus
+ * dtype = STOF_DTYPE_F16 (what the functions without the suffix pass) or STOF_DTYPE_BF16, before
+ * `stream`.  With bfloat16 every activation, weight, bias, gamma / beta and output tensor is
+ * bfloat16, the products run on v_mfma_f32_32x32x16_bf16 and accumulation, statistics and
+ * workspaces stay fp32.  (The reference computes in fp16 only; bfloat16 is an addition behind
+ * the same operators.  stof_gemm_bias_res_ln and stof_gemm_act_gemm take fp16 only.)
+ */
+int stof_bias_res_ln_dt(const void* x, const void* bias, const void* residual,
+                        const void* gamma, const void* beta, void* y,
+                        float* mean, float* rstd,
+                        int64_t M, int64_t N, float eps, int dtype, void* stream);
+int stof_gemm_bias_act_dt(const void* A, const void* Wt, const void* bias, void* C,
+                          int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldc,
+                          int act, int dtype, void* stream);
+int stof_gemm_bias_act_splitk_dt(const void* A, const void* Wt, const void* bias, void* C,
+                                 int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldc,
+                                 int act, int splits, void* workspace, int64_t workspace_bytes,
+                                 int dtype, void* stream);
+int stof_gemm_bias_res_ln_cluster_dt(const void* A, const void* Wt, const void* bias, const void* residual,
+                                     const void* gamma, const void* beta, void* C,
+                                     int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldr, int64_t ldc,
+                                     float eps, void* workspace, int64_t workspace_bytes, int dtype, void* stream);
 
 #ifdef __cplusplus
 }

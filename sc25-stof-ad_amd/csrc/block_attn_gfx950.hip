@@ -66,24 +66,7 @@ struct AttnParams {
 
 enum { kKindLut = 0, kKindPred = 1, kKindBits = 2 };
 
-// BF: the tensors are bfloat16 instead of fp16.  Operand fragments are carried as 16-bit
-// patterns in half8_t either way (loads, LDS and the transposing read do not look at the
-// format); only the MFMA opcode, the conversion of the probabilities and the final store differ.
-typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef unsigned short ushort8_t __attribute__((ext_vector_type(8)));
-template <bool BF>
-__device__ __forceinline__ floatx16 mfma32(half8_t a, half8_t b, floatx16 c) {
-  if constexpr (BF)
-    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
-  else
-    return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
-}
-// fp32 -> the tensors' 16-bit format (round to nearest even), as a 16-bit pattern in half_t
-template <bool BF>
-__device__ __forceinline__ half_t to_elem(float x) {
-  if constexpr (BF) return __builtin_bit_cast(half_t, (__bf16)x);
-  else return (half_t)x;
-}
 
 // max / sum of a value with its partner lane (lane ^ 32).  v_permlane32_swap(x, x) leaves
 // {own, partner} in some order in its two results for either half of the wave.

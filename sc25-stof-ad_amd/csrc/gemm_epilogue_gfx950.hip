@@ -26,9 +26,6 @@ namespace {
 typedef __attribute__((address_space(3))) unsigned char lds_byte;
 typedef __attribute__((address_space(1))) const void gptr_t;
 
-__device__ __forceinline__ floatx16 mfma32(half8_t a, half8_t b, floatx16 c) {
-  return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
-}
 __device__ __forceinline__ float pair_sum(float x) {
   const unsigned u = __builtin_bit_cast(unsigned, x);
   const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
@@ -91,7 +88,7 @@ inline unsigned raster_grid(int tiles_m, int tiles_n) { return 8u * (unsigned)((
 // features therefore goes through 4 KB of LDS of the wave's own (the operand tiles are free
 // after the last k-step; rows of 128 B with the 16-byte chunk index XOR-ed by the row, so the
 // row-wise reads are conflict-free) and leaves as 4 stores of 8 full 128-byte lines each.
-template <int ACT, int MT>
+template <int ACT, int MT, bool BF = false>
 __device__ __forceinline__ void store_wave_block(const GemmParams& p, const floatx16 (&acc)[2][MT], lds_byte* stage,
                                                  int m_base, int n_base, int lane) {
   const int j32 = lane & 31, g = lane >> 5;
@@ -112,7 +109,10 @@ __device__ __forceinline__ void store_wave_block(const GemmParams& p, const floa
       for (int q4 = 0; q4 < 4; ++q4) {
         half4_t o;
 #pragma unroll
-        for (int e = 0; e < 4; ++e) o[e] = (half_t)activate<ACT>(acc[ni][mi][4 * q4 + e] + (float)bv[ni][q4][e]);
+        for (int e = 0; e < 4; ++e) {
+          const half_t be = bv[ni][q4][e];
+          o[e] = to_elem<BF>(activate<ACT>(acc[ni][mi][4 * q4 + e] + from_elem<BF>(be)));
+        }
         *reinterpret_cast<__attribute__((address_space(3))) half4_t*>(stage + j32 * 128 + (((4 * ni + q4) ^ (j32 & 7)) << 4) + 8 * g) = o;
       }
 #pragma unroll
@@ -207,7 +207,7 @@ constexpr int kGT = 128;            // tile edge (tokens and features)
 constexpr int kGK = 64;             // K per tile
 constexpr int kGTile = kGT * kGK * 2;   // bytes per operand tile (16 KB)
 
-template <int ACT, bool SK = false>
+template <int ACT, bool SK = false, bool BF = false>
 __global__ __launch_bounds__(256) void gemm_bias_act_kernel(const GemmParams p) {
   __shared__ __attribute__((aligned(1024))) unsigned char a_lds0[kGTile];
   __shared__ __attribute__((aligned(1024))) unsigned char a_lds1[kGTile];
@@ -275,7 +275,7 @@ __global__ __launch_bounds__(256) void gemm_bias_act_kernel(const GemmParams p) 
 #pragma unroll
       for (int ni = 0; ni < 2; ++ni)
 #pragma unroll
-        for (int mi = 0; mi < 2; ++mi) acc[ni][mi] = mfma32(wb[ks & 1][ni], xa[ks & 1][mi], acc[ni][mi]);
+        for (int mi = 0; mi < 2; ++mi) acc[ni][mi] = mfma32<BF>(wb[ks & 1][ni], xa[ks & 1][mi], acc[ni][mi]);
       __builtin_amdgcn_sched_barrier(0);
     }
   };
@@ -299,7 +299,7 @@ __global__ __launch_bounds__(256) void gemm_bias_act_kernel(const GemmParams p) 
   if constexpr (SK) {
     if (!splitk_handover<2>(p, acc, (int64_t)tm * p.tiles_n + tn, z, wave, lane)) return;
   }
-  store_wave_block<ACT, 2>(p, acc, (lds_byte*)a_lds0 + wave * 4096, m0 + 64 * wm, n0 + 64 * wn, lane);
+  store_wave_block<ACT, 2, BF>(p, acc, (lds_byte*)a_lds0 + wave * 4096, m0 + 64 * wm, n0 + 64 * wn, lane);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -327,7 +327,7 @@ __device__ __forceinline__ int swz4(int row) { return (row >> 2) & 3; }
 // s_waitcnt immediate that waits for the vector-memory counter only (lgkmcnt 15, expcnt 7)
 constexpr int vmcnt_imm(int n) { return (n & 15) | ((n >> 4) << 14) | 0x0F70; }
 
-template <int ACT, int NS, bool SK = false, int KT = kSmallKT>
+template <int ACT, int NS, bool SK = false, int KT = kSmallKT, bool BF = false>
 __global__ __launch_bounds__(256, 2) void gemm_bias_act_ring_kernel(const GemmParams p) {
   static_assert(KT == 32 || KT == 64, "K per tile");
   constexpr int kK = KT;
@@ -425,7 +425,7 @@ __global__ __launch_bounds__(256, 2) void gemm_bias_act_ring_kernel(const GemmPa
   };
   auto mfmas = [&](const half8_t (&wbk)[2], const half8_t& xak) {
 #pragma unroll
-    for (int ni = 0; ni < 2; ++ni) acc[ni][0] = mfma32(wbk[ni], xak, acc[ni][0]);
+    for (int ni = 0; ni < 2; ++ni) acc[ni][0] = mfma32<BF>(wbk[ni], xak, acc[ni][0]);
   };
   auto wg_barrier = [&]() {
     // bare barrier: the fences of __syncthreads() would drain the loads that must stay in flight
@@ -475,7 +475,7 @@ __global__ __launch_bounds__(256, 2) void gemm_bias_act_ring_kernel(const GemmPa
   if constexpr (SK) {
     if (!splitk_handover<1>(p, acc, (int64_t)tm * p.tiles_n + tn, z, wave, lane)) return;
   }
-  store_wave_block<ACT, 1>(p, acc, (lds_byte*)a_lds + wave * 4096, m0 + 32 * wt, n0 + 64 * wf, lane);
+  store_wave_block<ACT, 1, BF>(p, acc, (lds_byte*)a_lds + wave * 4096, m0 + 32 * wt, n0 + 64 * wf, lane);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -554,7 +554,7 @@ __global__ __launch_bounds__(512) void gemm_bias_res_ln_kernel(const LnGemmParam
       for (int ni = 0; ni < NC; ++ni) {
         const half8_t wb = lds_frag(wt, (32 * NC * wave + 32 * ni) * 64 + rd[ks]);
 #pragma unroll
-        for (int mi = 0; mi < 2; ++mi) acc[ni][mi] = mfma32(wb, xa[mi], acc[ni][mi]);
+        for (int mi = 0; mi < 2; ++mi) acc[ni][mi] = mfma32<false>(wb, xa[mi], acc[ni][mi]);
       }
     }
   };
@@ -697,7 +697,7 @@ constexpr int kClusterSpinLimit = 1 << 18;   // default number of polls before a
 int g_cluster_spin_limit = kClusterSpinLimit;
 constexpr unsigned long long kStatsValid = 1ull << 63;
 
-template <int NT>   // NT = N / 128 workgroups per row block
+template <int NT, bool BF = false>   // NT = N / 128 workgroups per row block
 __global__ __launch_bounds__(256) void gemm_bias_res_ln_cluster_kernel(const LnClusterParams p) {
   __shared__ __attribute__((aligned(1024))) unsigned char a_lds0[kGTile];
   __shared__ __attribute__((aligned(1024))) unsigned char a_lds1[kGTile];
@@ -802,7 +802,7 @@ __global__ __launch_bounds__(256) void gemm_bias_res_ln_cluster_kernel(const LnC
 #pragma unroll
       for (int ni = 0; ni < 2; ++ni)
 #pragma unroll
-        for (int mi = 0; mi < 2; ++mi) acc[ni][mi] = mfma32(wb[ks & 1][ni], xa[ks & 1][mi], acc[ni][mi]);
+        for (int mi = 0; mi < 2; ++mi) acc[ni][mi] = mfma32<BF>(wb[ks & 1][ni], xa[ks & 1][mi], acc[ni][mi]);
       __builtin_amdgcn_sched_barrier(0);
     }
   };
@@ -853,7 +853,8 @@ __global__ __launch_bounds__(256) void gemm_bias_res_ln_cluster_kernel(const LnC
       for (int q4 = 0; q4 < 4; ++q4)
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-          const float v = acc[ni][mi][4 * q4 + e] + (float)bv[ni][q4][e] + (float)rv[ni][q4][e];
+          const half_t be = bv[ni][q4][e], re = rv[ni][q4][e];
+          const float v = acc[ni][mi][4 * q4 + e] + from_elem<BF>(be) + from_elem<BF>(re);
           acc[ni][mi][4 * q4 + e] = v;
           s += v;
         }
@@ -881,7 +882,7 @@ __global__ __launch_bounds__(256) void gemm_bias_res_ln_cluster_kernel(const LnC
 #pragma unroll
     for (int q4 = 0; q4 < 4; ++q4) {
       const int n = nb + 32 * ni + 8 * q4 + 4 * g;
-      gv[ni][q4] = half4_t{(half_t)1.f, (half_t)1.f, (half_t)1.f, (half_t)1.f};
+      gv[ni][q4] = half4_t{to_elem<BF>(1.f), to_elem<BF>(1.f), to_elem<BF>(1.f), to_elem<BF>(1.f)};
       tv[ni][q4] = half4_t{(half_t)0.f, (half_t)0.f, (half_t)0.f, (half_t)0.f};
       if (p.gamma) gv[ni][q4] = *reinterpret_cast<const half4_t*>(p.gamma + n);
       if (p.beta) tv[ni][q4] = *reinterpret_cast<const half4_t*>(p.beta + n);
@@ -936,8 +937,10 @@ __global__ __launch_bounds__(256) void gemm_bias_res_ln_cluster_kernel(const LnC
       for (int q4 = 0; q4 < 4; ++q4) {
         half4_t o;
 #pragma unroll
-        for (int e = 0; e < 4; ++e)
-          o[e] = (half_t)((acc[ni][mi][4 * q4 + e] - mean[mi]) * rstd[mi] * (float)gv[ni][q4][e] + (float)tv[ni][q4][e]);
+        for (int e = 0; e < 4; ++e) {
+          const half_t ge = gv[ni][q4][e], te = tv[ni][q4][e];
+          o[e] = to_elem<BF>((acc[ni][mi][4 * q4 + e] - mean[mi]) * rstd[mi] * from_elem<BF>(ge) + from_elem<BF>(te));
+        }
         *reinterpret_cast<__attribute__((address_space(3))) half4_t*>(stage + j32 * 128 + (((4 * ni + q4) ^ (j32 & 7)) << 4) + 8 * g) = o;
       }
 #pragma unroll
@@ -988,29 +991,43 @@ static_assert(kClusterStatsOffset % 256 == 0, "statistics start on a 256-byte bo
 constexpr int kSmallStages = 3;
 constexpr int kSmallMaxTiles = 128;
 
-template <int NS>
-int launch_ring(GemmParams& p, int act, hipStream_t st) {
-  p.tiles_m = (p.M + 63) / 64;
-  p.tiles_n = (p.N + kWFeat - 1) / kWFeat;
-  const dim3 grid(raster_grid(p.tiles_m, p.tiles_n)), block(256);
+// One launch of a bias / activation GEMM: tile form (64-token ring or 128 x 128), K split over
+// workgroups or not, element format.
+template <bool SMALL, bool SK, bool BF>
+int launch_gemm(const GemmParams& p, int act, unsigned groups, hipStream_t st) {
+  const dim3 grid(groups), block(256);
   switch (act) {
-    case STOF_ACT_NONE: hipLaunchKernelGGL((gemm_bias_act_ring_kernel<STOF_ACT_NONE, NS>), grid, block, 0, st, p); break;
-    case STOF_ACT_GELU_ERF: hipLaunchKernelGGL((gemm_bias_act_ring_kernel<STOF_ACT_GELU_ERF, NS>), grid, block, 0, st, p); break;
-    case STOF_ACT_GELU_TANH: hipLaunchKernelGGL((gemm_bias_act_ring_kernel<STOF_ACT_GELU_TANH, NS>), grid, block, 0, st, p); break;
-    case STOF_ACT_RELU: hipLaunchKernelGGL((gemm_bias_act_ring_kernel<STOF_ACT_RELU, NS>), grid, block, 0, st, p); break;
+#define STOF_GEMM_CASE(A) \
+    case A: \
+      if constexpr (SMALL) hipLaunchKernelGGL((gemm_bias_act_ring_kernel<A, kSmallStages, SK, kSmallKT, BF>), grid, block, 0, st, p); \
+      else hipLaunchKernelGGL((gemm_bias_act_kernel<A, SK, BF>), grid, block, 0, st, p); \
+      break;
+    STOF_GEMM_CASE(STOF_ACT_NONE)
+    STOF_GEMM_CASE(STOF_ACT_GELU_ERF)
+    STOF_GEMM_CASE(STOF_ACT_GELU_TANH)
+    STOF_GEMM_CASE(STOF_ACT_RELU)
+#undef STOF_GEMM_CASE
     default: return STOF_ERR_UNSUPPORTED;
   }
   return stof_check_launch();
 }
+template <bool SK>
+int launch_gemm(const GemmParams& p, bool small, int dtype, int act, hipStream_t st) {
+  const unsigned groups = raster_grid(p.tiles_m, p.tiles_n) * (unsigned)(SK ? p.splits : 1);
+  if (dtype == STOF_DTYPE_BF16)
+    return small ? launch_gemm<true, SK, true>(p, act, groups, st) : launch_gemm<false, SK, true>(p, act, groups, st);
+  return small ? launch_gemm<true, SK, false>(p, act, groups, st) : launch_gemm<false, SK, false>(p, act, groups, st);
+}
 
 }  // namespace
 
-extern "C" int stof_gemm_bias_act(const void* A, const void* Wt, const void* bias, void* C,
-                                  int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldc,
-                                  int act, void* stream) {
+extern "C" int stof_gemm_bias_act_dt(const void* A, const void* Wt, const void* bias, void* C,
+                                     int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldc,
+                                     int act, int dtype, void* stream) {
   if (!A || !Wt || !C) return STOF_ERR_NULL_POINTER;
   if (M <= 0 || N <= 0 || K <= 0 || K % kGK != 0 || N % 8 != 0 || lda < K || ldc < N) return STOF_ERR_BAD_SHAPE;
   if (M > (1 << 30) || N > (1 << 30) || K > (1 << 30)) return STOF_ERR_BAD_SHAPE;
+  if (dtype != STOF_DTYPE_F16 && dtype != STOF_DTYPE_BF16) return STOF_ERR_UNSUPPORTED;
   if (!stof_aligned16(A) || !stof_aligned16(Wt) || !stof_aligned16(C) || (bias && ((uintptr_t)bias & 7)) ||
       lda % 8 != 0 || ldc % 8 != 0)
     return STOF_ERR_MISALIGNED;
@@ -1018,20 +1035,17 @@ extern "C" int stof_gemm_bias_act(const void* A, const void* Wt, const void* bia
   p.A = (const half_t*)A; p.W = (const half_t*)Wt; p.bias = (const half_t*)bias; p.C = (half_t*)C;
   p.M = (int)M; p.N = (int)N; p.K = (int)K; p.lda = (int)lda; p.ldc = (int)ldc;
   p.partials = nullptr; p.counters = nullptr; p.splits = 1; p.nk_split = 0;
-  hipStream_t st = (hipStream_t)stream;
   if (((M + 63) / 64) * ((N + kGT - 1) / kGT) > (1 << 30)) return STOF_ERR_BAD_SHAPE;   // the grid is a 32-bit count
-  const int64_t tiles128 = ((M + kGT - 1) / kGT) * ((N + kGT - 1) / kGT);
-  if (tiles128 <= kSmallMaxTiles) return launch_ring<kSmallStages>(p, act, st);
-  p.tiles_m = (int)((M + kGT - 1) / kGT); p.tiles_n = (int)((N + kGT - 1) / kGT);
-  const dim3 grid(raster_grid(p.tiles_m, p.tiles_n)), block(256);
-  switch (act) {
-    case STOF_ACT_NONE: hipLaunchKernelGGL(gemm_bias_act_kernel<STOF_ACT_NONE>, grid, block, 0, st, p); break;
-    case STOF_ACT_GELU_ERF: hipLaunchKernelGGL(gemm_bias_act_kernel<STOF_ACT_GELU_ERF>, grid, block, 0, st, p); break;
-    case STOF_ACT_GELU_TANH: hipLaunchKernelGGL(gemm_bias_act_kernel<STOF_ACT_GELU_TANH>, grid, block, 0, st, p); break;
-    case STOF_ACT_RELU: hipLaunchKernelGGL(gemm_bias_act_kernel<STOF_ACT_RELU>, grid, block, 0, st, p); break;
-    default: return STOF_ERR_UNSUPPORTED;
-  }
-  return stof_check_launch();
+  const bool small = ((M + kGT - 1) / kGT) * ((N + kGT - 1) / kGT) <= kSmallMaxTiles;
+  const int tile_m = small ? 64 : kGT;
+  p.tiles_m = (int)((M + tile_m - 1) / tile_m); p.tiles_n = (int)((N + kGT - 1) / kGT);
+  return launch_gemm<false>(p, small, dtype, act, (hipStream_t)stream);
+}
+
+extern "C" int stof_gemm_bias_act(const void* A, const void* Wt, const void* bias, void* C,
+                                  int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldc,
+                                  int act, void* stream) {
+  return stof_gemm_bias_act_dt(A, Wt, bias, C, M, N, K, lda, ldc, act, STOF_DTYPE_F16, stream);
 }
 
 // ---- split-K form of the 64-token ring GEMM, for few output tiles and a long K ----------------
@@ -1080,31 +1094,14 @@ extern "C" int64_t stof_gemm_bias_act_splitk_workspace_bytes(int64_t M, int64_t 
   return kSplitPartialsOffset + ((M + kGT - 1) / kGT) * ((N + kGT - 1) / kGT) * splits * (kGT * kGT * 4);
 }
 
-template <bool SMALL>
-int launch_splitk(const GemmParams& p, int act, unsigned groups, hipStream_t st) {
-  const dim3 grid(groups), block(256);
-  switch (act) {
-#define STOF_SPLITK_CASE(A) \
-    case A: \
-      if (SMALL) hipLaunchKernelGGL((gemm_bias_act_ring_kernel<A, kSmallStages, true>), grid, block, 0, st, p); \
-      else hipLaunchKernelGGL((gemm_bias_act_kernel<A, true>), grid, block, 0, st, p); \
-      break;
-    STOF_SPLITK_CASE(STOF_ACT_NONE)
-    STOF_SPLITK_CASE(STOF_ACT_GELU_ERF)
-    STOF_SPLITK_CASE(STOF_ACT_GELU_TANH)
-    STOF_SPLITK_CASE(STOF_ACT_RELU)
-#undef STOF_SPLITK_CASE
-    default: return STOF_ERR_UNSUPPORTED;
-  }
-  return stof_check_launch();
-}
-
-extern "C" int stof_gemm_bias_act_splitk(const void* A, const void* Wt, const void* bias, void* C,
-                                         int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldc,
-                                         int act, int splits, void* workspace, int64_t workspace_bytes, void* stream) {
+extern "C" int stof_gemm_bias_act_splitk_dt(const void* A, const void* Wt, const void* bias, void* C,
+                                            int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldc,
+                                            int act, int splits, void* workspace, int64_t workspace_bytes,
+                                            int dtype, void* stream) {
   if (!A || !Wt || !C || !workspace) return STOF_ERR_NULL_POINTER;
   if (M <= 0 || N <= 0 || K <= 0 || K % kGK != 0 || N % 8 != 0 || lda < K || ldc < N) return STOF_ERR_BAD_SHAPE;
   if (K > (1 << 30) || splits < 2 || splits > kSplitMaxSplits) return STOF_ERR_BAD_SHAPE;
+  if (dtype != STOF_DTYPE_F16 && dtype != STOF_DTYPE_BF16) return STOF_ERR_UNSUPPORTED;
   const int64_t tiles64 = ((M + 63) / 64) * ((N + kWFeat - 1) / kWFeat);
   if (tiles64 > kSplitMaxTiles) return STOF_ERR_UNSUPPORTED;
   if (!stof_aligned16(A) || !stof_aligned16(Wt) || !stof_aligned16(C) || (bias && ((uintptr_t)bias & 7)) ||
@@ -1116,17 +1113,21 @@ extern "C" int stof_gemm_bias_act_splitk(const void* A, const void* Wt, const vo
   p.M = (int)M; p.N = (int)N; p.K = (int)K; p.lda = (int)lda; p.ldc = (int)ldc;
   p.counters = reinterpret_cast<int*>(workspace);
   p.partials = reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) + kSplitPartialsOffset);
-  // The tile form follows the plain GEMM's rule: 64-token tiles (k-tiles of 32) where the
-  // 128 x 128 form (k-tiles of 64) would have at most kSmallMaxTiles workgroups.
+  // The tile form follows the plain GEMM's rule: 64-token tiles where the 128 x 128 form would
+  // have at most kSmallMaxTiles workgroups.
   const bool small = ((M + kGT - 1) / kGT) * ((N + kGT - 1) / kGT) <= kSmallMaxTiles;
   const int tile_m = small ? 64 : kGT, tile_k = small ? kSmallKT : kGK;
   p.tiles_m = (int)((M + tile_m - 1) / tile_m); p.tiles_n = (int)((N + kGT - 1) / kGT);
   const int nk = (int)(K / tile_k);
   p.nk_split = (nk + splits - 1) / splits;
   p.splits = (nk + p.nk_split - 1) / p.nk_split;   // (every split has at least one k-tile)
-  const unsigned groups = raster_grid(p.tiles_m, p.tiles_n) * (unsigned)p.splits;
-  hipStream_t st = (hipStream_t)stream;
-  return small ? launch_splitk<true>(p, act, groups, st) : launch_splitk<false>(p, act, groups, st);
+  return launch_gemm<true>(p, small, dtype, act, (hipStream_t)stream);
+}
+
+extern "C" int stof_gemm_bias_act_splitk(const void* A, const void* Wt, const void* bias, void* C,
+                                         int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldc,
+                                         int act, int splits, void* workspace, int64_t workspace_bytes, void* stream) {
+  return stof_gemm_bias_act_splitk_dt(A, Wt, bias, C, M, N, K, lda, ldc, act, splits, workspace, workspace_bytes, STOF_DTYPE_F16, stream);
 }
 
 extern "C" int stof_gemm_bias_res_ln(const void* A, const void* Wt, const void* bias, const void* residual,
@@ -1178,11 +1179,12 @@ extern "C" int stof_gemm_bias_res_ln_cluster_set_spin_limit(int polls) {
   return STOF_OK;
 }
 
-extern "C" int stof_gemm_bias_res_ln_cluster(const void* A, const void* Wt, const void* bias, const void* residual,
-                                             const void* gamma, const void* beta, void* C,
-                                             int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldr, int64_t ldc,
-                                             float eps, void* workspace, int64_t workspace_bytes, void* stream) {
+extern "C" int stof_gemm_bias_res_ln_cluster_dt(const void* A, const void* Wt, const void* bias, const void* residual,
+                                                const void* gamma, const void* beta, void* C,
+                                                int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldr, int64_t ldc,
+                                                float eps, void* workspace, int64_t workspace_bytes, int dtype, void* stream) {
   if (!A || !Wt || !C || !workspace) return STOF_ERR_NULL_POINTER;
+  if (dtype != STOF_DTYPE_F16 && dtype != STOF_DTYPE_BF16) return STOF_ERR_UNSUPPORTED;
   if (M <= 0 || K <= 0 || K % kGK != 0 || M > kClusterMaxRows || K > (1 << 30) || lda < K || ldc < N || (residual && ldr < N))
     return STOF_ERR_BAD_SHAPE;
   if (N % kGT != 0 || N < 2 * kGT || N > 8 * kGT) return STOF_ERR_UNSUPPORTED;   // 256, 384, ..., 1024
@@ -1209,14 +1211,25 @@ extern "C" int stof_gemm_bias_res_ln_cluster(const void* A, const void* Wt, cons
   if (resident < 8 * p.tiles_n) return STOF_ERR_UNSUPPORTED;   // a device too small to hold one cluster per XCD
   const dim3 grid((unsigned)(groups < resident ? groups : resident)), block(256);
   hipStream_t st = (hipStream_t)stream;
+  const bool bf = dtype == STOF_DTYPE_BF16;
   switch (p.tiles_n) {
-    case 2: hipLaunchKernelGGL(gemm_bias_res_ln_cluster_kernel<2>, grid, block, 0, st, p); break;
-    case 3: hipLaunchKernelGGL(gemm_bias_res_ln_cluster_kernel<3>, grid, block, 0, st, p); break;
-    case 4: hipLaunchKernelGGL(gemm_bias_res_ln_cluster_kernel<4>, grid, block, 0, st, p); break;
-    case 5: hipLaunchKernelGGL(gemm_bias_res_ln_cluster_kernel<5>, grid, block, 0, st, p); break;
-    case 6: hipLaunchKernelGGL(gemm_bias_res_ln_cluster_kernel<6>, grid, block, 0, st, p); break;
-    case 7: hipLaunchKernelGGL(gemm_bias_res_ln_cluster_kernel<7>, grid, block, 0, st, p); break;
-    default: hipLaunchKernelGGL(gemm_bias_res_ln_cluster_kernel<8>, grid, block, 0, st, p); break;
+#define STOF_CLUSTER_CASE(NT) \
+    case NT: \
+      if (bf) hipLaunchKernelGGL((gemm_bias_res_ln_cluster_kernel<NT, true>), grid, block, 0, st, p); \
+      else hipLaunchKernelGGL((gemm_bias_res_ln_cluster_kernel<NT, false>), grid, block, 0, st, p); \
+      break;
+    STOF_CLUSTER_CASE(2) STOF_CLUSTER_CASE(3) STOF_CLUSTER_CASE(4) STOF_CLUSTER_CASE(5)
+    STOF_CLUSTER_CASE(6) STOF_CLUSTER_CASE(7) STOF_CLUSTER_CASE(8)
+#undef STOF_CLUSTER_CASE
+    default: return STOF_ERR_UNSUPPORTED;
   }
   return stof_check_launch();
+}
+
+extern "C" int stof_gemm_bias_res_ln_cluster(const void* A, const void* Wt, const void* bias, const void* residual,
+                                             const void* gamma, const void* beta, void* C,
+                                             int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldr, int64_t ldc,
+                                             float eps, void* workspace, int64_t workspace_bytes, void* stream) {
+  return stof_gemm_bias_res_ln_cluster_dt(A, Wt, bias, residual, gamma, beta, C, M, N, K, lda, ldr, ldc, eps,
+                                          workspace, workspace_bytes, STOF_DTYPE_F16, stream);
 }

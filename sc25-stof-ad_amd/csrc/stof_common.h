@@ -13,6 +13,30 @@ typedef float floatx16 __attribute__((ext_vector_type(16)));
 
 #define STOF_WAVE 64
 
+// BF: the tensors are bfloat16 instead of fp16.  Operand fragments are carried as 16-bit
+// patterns in half_t / half8_t either way (loads, LDS and the transposing read do not look at
+// the format); only the MFMA opcode and the conversions from and to fp32 differ.
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+template <bool BF>
+__device__ __forceinline__ floatx16 mfma32(half8_t a, half8_t b, floatx16 c) {
+  if constexpr (BF)
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
+  else
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+}
+// fp32 -> the tensors' 16-bit format (round to nearest even), as a 16-bit pattern in half_t
+template <bool BF>
+__device__ __forceinline__ half_t to_elem(float x) {
+  if constexpr (BF) return __builtin_bit_cast(half_t, (__bf16)x);
+  else return (half_t)x;
+}
+// the tensors' 16-bit format -> fp32 (bfloat16: the pattern is the upper half of the fp32 pattern)
+template <bool BF>
+__device__ __forceinline__ float from_elem(half_t e) {
+  if constexpr (BF) return __builtin_bit_cast(float, (uint32_t)__builtin_bit_cast(unsigned short, e) << 16);
+  else return (float)e;
+}
+
 // One wavefront spans two halves of 32 lanes; exchange a value with the partner lane
 // (lane ^ 32).  Used by the 32x32 MFMA layouts where a column lives in lanes l and l^32.
 __device__ __forceinline__ float xchg32(float x) {

@@ -43,6 +43,12 @@ _SIGNATURES = {
     "stof_gemm_bias_act_splitk": (c_int, [_P, _P, _P, _P, c_int64, c_int64, c_int64, c_int64, c_int64, c_int, c_int,
                                           _P, c_int64, _P]),
     "stof_gemm_bias_res_ln": (c_int, [_P, _P, _P, _P, _P, _P, _P, c_int64, c_int64, c_int64, c_float, _P]),
+    "stof_bias_res_ln_dt": (c_int, [_P, _P, _P, _P, _P, _P, _P, _P, c_int64, c_int64, c_float, c_int, _P]),
+    "stof_gemm_bias_act_dt": (c_int, [_P, _P, _P, _P, c_int64, c_int64, c_int64, c_int64, c_int64, c_int, c_int, _P]),
+    "stof_gemm_bias_act_splitk_dt": (c_int, [_P, _P, _P, _P, c_int64, c_int64, c_int64, c_int64, c_int64, c_int, c_int,
+                                             _P, c_int64, c_int, _P]),
+    "stof_gemm_bias_res_ln_cluster_dt": (c_int, [_P, _P, _P, _P, _P, _P, _P, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64,
+                                                 c_float, _P, c_int64, c_int, _P]),
     "stof_gemm_bias_res_ln_cluster_workspace_bytes": (c_int64, [c_int64, c_int64]),
     "stof_gemm_bias_res_ln_cluster_set_spin_limit": (c_int, [c_int]),
     "stof_gemm_bias_res_ln_cluster": (c_int, [_P, _P, _P, _P, _P, _P, _P, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64,

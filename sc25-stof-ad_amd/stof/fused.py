@@ -42,12 +42,23 @@ def _require(cond, msg):
         raise StofError(msg)
 
 
-def _f16c(name, t, allow_none=False):
+_DTYPES = {torch.float16: 0, torch.bfloat16: 1}   # STOF_DTYPE_*
+
+
+def _f16c(name, t, allow_none=False, like=None):
+    """``t`` contiguous; a CUDA float16 tensor, or of ``like``'s 16-bit format if that is given."""
     if t is None:
         _require(allow_none, f"{name} is required")
         return None
-    _require(t.is_cuda and t.dtype == torch.float16, f"{name} must be a CUDA float16 tensor")
+    want = torch.float16 if like is None else like.dtype
+    _require(t.is_cuda and t.dtype == want, f"{name} must be a CUDA {str(want).replace('torch.', '')} tensor")
     return t.contiguous()
+
+
+def _elem16(name, t):
+    """``t`` must be a CUDA tensor in one of the two 16-bit formats; its STOF_DTYPE_* code."""
+    _require(t.is_cuda and t.dtype in _DTYPES, f"{name} must be a CUDA float16 or bfloat16 tensor")
+    return _DTYPES[t.dtype]
 
 
 def _p(t):
@@ -69,12 +80,14 @@ def pack_weight(W):
 
 
 def bias_residual_layernorm(x, bias, residual, gamma, beta, eps=1e-5, return_stats=False, out=None):
-    """LN(x + bias + residual) * gamma + beta over the last dim; any operand but x may be None."""
-    x = _f16c("x", x)
+    """LN(x + bias + residual) * gamma + beta over the last dim; any operand but x may be None.
+    float16 or, all operands alike, bfloat16."""
+    dt = _elem16("x", x)
+    x = x.contiguous()
     N = x.shape[-1]
     M = x.numel() // N
-    bias = _f16c("bias", bias, True); residual = _f16c("residual", residual, True)
-    gamma = _f16c("gamma", gamma, True); beta = _f16c("beta", beta, True)
+    bias = _f16c("bias", bias, True, x); residual = _f16c("residual", residual, True, x)
+    gamma = _f16c("gamma", gamma, True, x); beta = _f16c("beta", beta, True, x)
     for name, t in (("bias", bias), ("gamma", gamma), ("beta", beta)):
         _require(t is None or t.numel() == N, f"{name} must have {N} elements")
     _require(residual is None or residual.shape == x.shape, "residual must have x's shape")
@@ -84,8 +97,8 @@ def bias_residual_layernorm(x, bias, residual, gamma, beta, eps=1e-5, return_sta
     if return_stats:
         mean = torch.empty(M, dtype=torch.float32, device=x.device)
         rstd = torch.empty(M, dtype=torch.float32, device=x.device)
-    check(_lib.lib().stof_bias_res_ln(x.data_ptr(), _p(bias), _p(residual), _p(gamma), _p(beta),
-                                      y.data_ptr(), _p(mean), _p(rstd), M, N, float(eps), _stream(y)),
+    check(_lib.lib().stof_bias_res_ln_dt(x.data_ptr(), _p(bias), _p(residual), _p(gamma), _p(beta),
+                                         y.data_ptr(), _p(mean), _p(rstd), M, N, float(eps), dt, _stream(y)),
           "stof_bias_res_ln")
     return (y, mean, rstd) if return_stats else y
 
@@ -110,15 +123,16 @@ def _splitk_workspace(dev, stream, nbytes):
 
 
 def gemm_bias_act(x, Wt, bias=None, act="none", out=None, splits=None):
-    """act(x @ Wt^T + bias): x [..., K] (rows may be strided), Wt [N, K], bias [N].
+    """act(x @ Wt^T + bias): x [..., K] (rows may be strided), Wt [N, K], bias [N]; float16 or,
+    all operands alike, bfloat16.
 
     ``splits``: None = the library's rule (stof_gemm_bias_act_splitk_plan: K split over several
     workgroups per tile where the output has few tiles and K is long), 1 = one workgroup per tile
     (stof_gemm_bias_act), 2 .. 8 = that many splits (stof_gemm_bias_act_splitk)."""
     _require(act in ACT, f"unknown activation {act!r}")
     _require(splits is None or 1 <= int(splits) <= 8, "splits must be None or 1 .. 8")
-    _require(x.is_cuda and x.dtype == torch.float16, "x must be a CUDA float16 tensor")
-    Wt = _f16c("Wt", Wt); bias = _f16c("bias", bias, True)
+    dt = _elem16("x", x)
+    Wt = _f16c("Wt", Wt, like=x); bias = _f16c("bias", bias, True, x)
     K = x.shape[-1]
     N = Wt.shape[0]
     _require(Wt.dim() == 2 and Wt.shape[1] == K, f"Wt must be [N, {K}]")
@@ -128,7 +142,8 @@ def gemm_bias_act(x, Wt, bias=None, act="none", out=None, splits=None):
         x2 = x2.contiguous()
     M = x2.shape[0]
     if out is None:
-        out = torch.empty(x.shape[:-1] + (N,), dtype=torch.float16, device=x.device)
+        out = torch.empty(x.shape[:-1] + (N,), dtype=x.dtype, device=x.device)
+    _require(out.dtype == x.dtype, "out must have x's element format")
     o2 = out.view(-1, N)
     _require(o2.shape[0] == M and o2.stride(1) == 1, "out must be [..., N] with contiguous rows")
     lib = _lib.lib()
@@ -139,13 +154,13 @@ def gemm_bias_act(x, Wt, bias=None, act="none", out=None, splits=None):
         nbytes = lib.stof_gemm_bias_act_splitk_workspace_bytes(M, N, splits)
         _require(nbytes > 0, f"shape not supported by the split-K form: M {M}, N {N}")
         ws = _splitk_workspace(x.device, st, nbytes)
-        check(lib.stof_gemm_bias_act_splitk(x2.data_ptr(), Wt.data_ptr(), _p(bias), o2.data_ptr(),
-                                            M, N, K, x2.stride(0), o2.stride(0), ACT[act], int(splits),
-                                            ws.data_ptr(), ws.numel(), st),
+        check(lib.stof_gemm_bias_act_splitk_dt(x2.data_ptr(), Wt.data_ptr(), _p(bias), o2.data_ptr(),
+                                               M, N, K, x2.stride(0), o2.stride(0), ACT[act], int(splits),
+                                               ws.data_ptr(), ws.numel(), dt, st),
               "stof_gemm_bias_act_splitk")
         return out
-    check(lib.stof_gemm_bias_act(x2.data_ptr(), Wt.data_ptr(), _p(bias), o2.data_ptr(),
-                                 M, N, K, x2.stride(0), o2.stride(0), ACT[act], st),
+    check(lib.stof_gemm_bias_act_dt(x2.data_ptr(), Wt.data_ptr(), _p(bias), o2.data_ptr(),
+                                    M, N, K, x2.stride(0), o2.stride(0), ACT[act], dt, st),
           "stof_gemm_bias_act")
     return out
 
@@ -233,9 +248,11 @@ def gemm_bias_residual_layernorm(x, Wt, bias, residual, gamma, beta, eps=1e-5, o
     if form == "split":
         y = gemm_bias_act(x, Wt, None, "none")
         return bias_residual_layernorm(y, bias, None if residual is None else residual.reshape(y.shape), gamma, beta, eps, out=out)
-    x = _f16c("x", x); Wt = _f16c("Wt", Wt)
-    bias = _f16c("bias", bias, True); residual = _f16c("residual", residual, True)
-    gamma = _f16c("gamma", gamma, True); beta = _f16c("beta", beta, True)
+    dt = _elem16("x", x)
+    _require(dt == 0 or form == "cluster", "the row form takes float16 only")
+    x = x.contiguous(); Wt = _f16c("Wt", Wt, like=x)
+    bias = _f16c("bias", bias, True, x); residual = _f16c("residual", residual, True, x)
+    gamma = _f16c("gamma", gamma, True, x); beta = _f16c("beta", beta, True, x)
     K = x.shape[-1]
     N = Wt.shape[0]
     M = x.numel() // K
@@ -244,16 +261,17 @@ def gemm_bias_residual_layernorm(x, Wt, bias, residual, gamma, beta, eps=1e-5, o
     for name, t in (("bias", bias), ("gamma", gamma), ("beta", beta)):
         _require(t is None or t.numel() == N, f"{name} must have {N} elements")
     if out is None:
-        out = torch.empty(x.shape[:-1] + (N,), dtype=torch.float16, device=x.device)
+        out = torch.empty(x.shape[:-1] + (N,), dtype=x.dtype, device=x.device)
+    _require(out.dtype == x.dtype, "out must have x's element format")
     lib = _lib.lib()
     st = _stream(out)
     if form == "cluster":
         _require(cluster_supported(N, K), f"unsupported shape for the cluster form: N {N}, K {K}")
         nbytes = lib.stof_gemm_bias_res_ln_cluster_workspace_bytes(M, N)
         ws = _cluster_workspace(x.device, st, nbytes)
-        check(lib.stof_gemm_bias_res_ln_cluster(x.data_ptr(), Wt.data_ptr(), _p(bias), _p(residual), _p(gamma), _p(beta),
-                                                out.data_ptr(), M, N, K, K, N, N, float(eps),
-                                                ws.data_ptr(), ws.numel(), st),
+        check(lib.stof_gemm_bias_res_ln_cluster_dt(x.data_ptr(), Wt.data_ptr(), _p(bias), _p(residual), _p(gamma), _p(beta),
+                                                   out.data_ptr(), M, N, K, K, N, N, float(eps),
+                                                   ws.data_ptr(), ws.numel(), dt, st),
               "stof_gemm_bias_res_ln_cluster")
         return out
     check(lib.stof_gemm_bias_res_ln(x.data_ptr(), Wt.data_ptr(), _p(bias), _p(residual),
