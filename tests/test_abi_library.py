@@ -94,6 +94,12 @@ def test_other_entry_points_argument_checks(lib):
     assert sk(wsb=sneed - 1) == -2         # workspace too small
     assert sk(act=9) == -3 and sk(M=1 << 20, wsb=1 << 40) == -3      # more tiles than the counter area holds
     assert sk(A=P + 8) == -4 and sk(ws=P + 8) == -4
+    # the entry points that take the element format: 0 fp16, 1 bfloat16, anything else unsupported
+    assert lib.stof_gemm_bias_act_dt(P, P, None, P, 64, 64, 64, 64, 64, 0, 2, None) == -3
+    assert lib.stof_gemm_bias_act_dt(P, P, None, P, 64, 64, 96, 96, 64, 0, 1, None) == -2      # K % 64, as without the suffix
+    assert lib.stof_bias_res_ln_dt(P, None, None, None, None, P, None, None, 10, 64, 1e-5, 7, None) == -3
+    assert lib.stof_gemm_bias_act_splitk_dt(P, P, None, P, 512, 768, 3072, 3072, 768, 0, 4, P, sneed, 2, None) == -3
+    assert lib.stof_gemm_bias_res_ln_cluster_dt(P, P, None, None, None, None, P, 8192, 768, 768, 768, 768, 768, 1e-5, P, 1 << 30, 5, None) == -3
     # chained GEMM + activation + GEMM: X, W1t, b1, W2t, b2, Y, M, K, F, H, ldx, ldy, act, workspace, bytes, stream
     need = lib.stof_gemm_act_gemm_workspace_bytes(64, 128)
     assert need >= 64 * 128 * 4 + 4 and lib.stof_gemm_act_gemm_workspace_bytes(0, 128) == 0
