@@ -168,6 +168,10 @@ def bench_layer_c3(steps, warmup):
         y_eager = eager_layer(x, w, maskg, cfg.heads, cfg.eps)
         out["eager_ms"], _ = time_region(lambda: eager_layer(x, w, maskg, cfg.heads, cfg.eps), max(steps // 4, 5), 5)
     out["output_check"] = output_check(y_auto, y_eager, valid=(torch.arange(cfg.seq)[None, :] < L[:, None]).cuda())
+    # the same layer on bfloat16 tensors (an addition: the reference is fp16 only)
+    layer_bf = EncoderLayer({k: v.to(torch.bfloat16) for k, v in w.items()}, cfg.heads, eps=cfg.eps)
+    x_bf = x.to(torch.bfloat16)
+    out["bf16_ms"], _ = time_region(lambda: layer_bf(x_bf, lut), steps, warmup)
     layer = EncoderLayer(w, cfg.heads, eps=cfg.eps, ln_fusion="auto")
     out["stages_ms"] = {name: time_region(fn, steps, warmup)[1] for name, fn in layer.stages(x, lut)}
     out["layer_ms_without_qkv_gemm"] = sum(v for k, v in out["stages_ms"].items() if k != "qkv_gemm")
