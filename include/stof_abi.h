@@ -46,7 +46,7 @@
 extern "C" {
 #endif
 
-#define STOF_ABI_VERSION 2
+#define STOF_ABI_VERSION 3   /* 3: split-K and element-format entry points added (nothing removed or changed) */
 
 enum {
   STOF_OK = 0,

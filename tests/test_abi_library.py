@@ -37,7 +37,7 @@ def test_every_declared_symbol_is_exported_and_bound(lib):
 
 
 def test_version_and_status_strings(lib):
-    assert lib.stof_abi_version() == 2
+    assert lib.stof_abi_version() == 3
     for code in (0, -1, -2, -3, -4, -5, -6, -7, -99):
         assert len(lib.stof_status_string(code)) > 0
 
