@@ -1048,10 +1048,10 @@ extern "C" int stof_gemm_bias_act(const void* A, const void* Wt, const void* bia
   return stof_gemm_bias_act_dt(A, Wt, bias, C, M, N, K, lda, ldc, act, STOF_DTYPE_F16, stream);
 }
 
-// ---- split-K form of the 64-token ring GEMM, for few output tiles and a long K ----------------
+// ---- K split over workgroups (either tile form), for few output tiles and a long K --------------
 // Workspace: one counter per (tile, wave) for up to kSplitMaxTiles tiles (a fixed area, so that a
-// workspace that served one shape can serve another; zero between calls), then the partial sums,
-// 32 KB per (tile, split).
+// workspace that served one shape can serve another; zero between calls), then the fp32 partial
+// sums: 32 KB per (64 x 128 tile, split) or 64 KB per (128 x 128 tile, split).
 constexpr int64_t kSplitMaxTiles = 4096;
 constexpr int64_t kSplitPartialsOffset = kSplitMaxTiles * 4 * 4;
 constexpr int kSplitMaxSplits = 8;       // what the entry point takes
