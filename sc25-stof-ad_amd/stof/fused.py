@@ -18,6 +18,8 @@ Weights are consumed in the ``[N, K]`` (nn.Linear) orientation, K contiguous, wh
 the MFMA B operand wants; ``pack_weight`` converts a reference-style ``[K, N]`` matrix once.
 Nothing here falls back to PyTorch math: a missing library or unsupported shape raises.
 """
+import functools
+
 import torch
 
 from . import _lib
@@ -51,7 +53,8 @@ def _f16c(name, t, allow_none=False, like=None):
         _require(allow_none, f"{name} is required")
         return None
     want = torch.float16 if like is None else like.dtype
-    _require(t.is_cuda and t.dtype == want, f"{name} must be a CUDA {str(want).replace('torch.', '')} tensor")
+    if not (t.is_cuda and t.dtype == want):
+        raise StofError(f"{name} must be a CUDA {str(want).replace('torch.', '')} tensor")
     return t.contiguous()
 
 
@@ -149,7 +152,7 @@ def gemm_bias_act(x, Wt, bias=None, act="none", out=None, splits=None):
     lib = _lib.lib()
     st = _stream(o2)
     if splits is None:
-        splits = lib.stof_gemm_bias_act_splitk_plan(M, N, K)
+        splits = _splitk_plan(M, N, K)
     if splits > 1:
         nbytes = lib.stof_gemm_bias_act_splitk_workspace_bytes(M, N, splits)
         _require(nbytes > 0, f"shape not supported by the split-K form: M {M}, N {N}")
@@ -221,6 +224,13 @@ def clear_cluster_exchange_error(dev=None):
 CLUSTER_MIN_TILES = 192
 
 
+@functools.lru_cache(maxsize=4096)
+def _splitk_plan(M, N, K):
+    """stof_gemm_bias_act_splitk_plan, remembered per shape (a pure function of the three sizes)."""
+    return _lib.lib().stof_gemm_bias_act_splitk_plan(M, N, K)
+
+
+@functools.lru_cache(maxsize=4096)
 def ln_gemm_form(M, N, K):
     """How ``form="auto"`` runs a LayerNorm GEMM of M rows: "cluster", or "split" (tiled GEMM, then
     the bias+residual+LayerNorm kernel; the pre-normalisation values pass through HBM as fp16), or
@@ -228,7 +238,7 @@ def ln_gemm_form(M, N, K):
     tiles = ((M + 127) // 128) * (N // 128)
     # (where the tiled GEMM would split K - 129 .. 192 tiles and a long K - it overtakes the cluster
     # form, which cannot: 4096 x 768 x 3072 36.5 us as two launches against 39.9)
-    if cluster_supported(N, K) and tiles >= CLUSTER_MIN_TILES and _lib.lib().stof_gemm_bias_act_splitk_plan(M, N, K) == 1:
+    if cluster_supported(N, K) and tiles >= CLUSTER_MIN_TILES and _splitk_plan(M, N, K) == 1:
         return "cluster"
     return "split" if K % 64 == 0 else "row"
 
