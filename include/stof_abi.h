@@ -17,6 +17,8 @@
  * Reference interfaces replaced (paths relative to the reference tree):
  *   stof_block_attn_fwd        launch_block_attn_mask      src/ops/src/block_attn_mask.cpp:8-15,
  *                                                           src/ops/src/block_attn_mask_cuda.cu:6026-6322
+ *   stof_attn_plan_*,
+ *   stof_block_attn_fwd_planned  the LUT reads of the same kernels, block_attn_mask_cuda.cu:3590-3700
  *   stof_pack_mask_bits        (the fp16 additive blocks built at src/util/masks.py:159-166,
  *                               consumed at block_attn_mask_cuda.cu:3680-3698, and the fp16
  *                               row_mask of launcher_rowwise_attn_mask, rowwise_attn_mask_cuda.cu:89-101)
@@ -46,7 +48,7 @@
 extern "C" {
 #endif
 
-#define STOF_ABI_VERSION 3   /* 3: split-K and element-format entry points added (nothing removed or changed) */
+#define STOF_ABI_VERSION 4   /* 4: attention plan entry points added; 3: split-K and element-format entry points (nothing removed or changed) */
 
 enum {
   STOF_OK = 0,
@@ -124,6 +126,49 @@ int stof_block_attn_fwd(
     const int64_t v_strides[3], const int64_t out_strides[3],
     int batch_size, int seq_len, int head_num, int head_size, int dtype,
     int64_t lut_batch_stride, int launch_form, void* stream);
+
+/*
+ * The walk of a LUT laid out ahead of time ("plan"), and stof_block_attn_fwd reading it.
+ *
+ * The reference's kernels read the LUT as it is: row pointers, then the row's column list, then
+ * per key block a search of the PART list (block_attn_mask_cuda.cu:3590-3700).  Here a workgroup
+ * owns one or two query blocks and visits the union of their key blocks; without a plan it reads
+ * the row pointers of its whole head (to find its place in the order by row length), then the
+ * column lists, and merges them - several dependent trips through memory before its first K/V
+ * tile.  A plan holds, per LUT (per sample for per-sample LUTs) and per group in that order, the
+ * finished walk: the workgroup's first load is its walk.  A LUT is usually built once and used for
+ * every layer and step, so the plan is built once per LUT (one small launch) and kept beside it.
+ *
+ *   stof_attn_plan_rows   query blocks per workgroup (1 or 2) of the launch form that
+ *                         stof_block_attn_fwd would use for this problem and launch_form - the
+ *                         rows_per_group to build the plan with; 0 if that form reads no plan.
+ *   stof_attn_plan_bytes  size of the plan in bytes; 0 = no plan for this shape (seq_len > 65536).
+ *   stof_attn_plan_build  writes the plan for the LOAD / PART lists of a LUT (arguments as in
+ *                         stof_block_attn_fwd; lut_batches = 1 for a shared LUT, else the batch
+ *                         size with row pointers lut_batch_stride apart).  plan: device memory,
+ *                         8-byte aligned, plan_bytes >= stof_attn_plan_bytes(...).
+ *   stof_block_attn_fwd_planned  stof_block_attn_fwd plus the plan.  plan == NULL, or a plan whose
+ *                         plan_rows is not what the launch form takes, runs exactly as
+ *                         stof_block_attn_fwd does.  The plan must have been built from the same
+ *                         LOAD / PART lists; results are bit-identical with and without it.
+ */
+int stof_attn_plan_rows(int batch_size, int head_num, int seq_len, int launch_form);
+int64_t stof_attn_plan_bytes(int seq_len, int rows_per_group, int lut_batches);
+int stof_attn_plan_build(const int32_t* part_row_ptr, const int32_t* part_col_idx,
+                         const int32_t* load_row_ptr, const int32_t* load_col_idx,
+                         int seq_len, int64_t lut_batch_stride, int lut_batches, int rows_per_group,
+                         void* plan, int64_t plan_bytes, void* stream);
+int stof_block_attn_fwd_planned(
+    const void* q, const void* k, const void* v, void* out,
+    const int32_t* full_row_ptr, const int32_t* full_col_idx,
+    const int32_t* part_row_ptr, const int32_t* part_col_idx, const uint64_t* part_bitmask,
+    const int32_t* load_row_ptr, const int32_t* load_col_idx,
+    int block_m, int block_n, float softmax_scale,
+    const int64_t q_strides[3], const int64_t k_strides[3],
+    const int64_t v_strides[3], const int64_t out_strides[3],
+    int batch_size, int seq_len, int head_num, int head_size, int dtype,
+    int64_t lut_batch_stride, int launch_form,
+    const void* plan, int64_t plan_bytes, int plan_rows, void* stream);
 
 /*
  * Process-wide default launch form, used by calls that pass STOF_FORM_DEFAULT: -1 automatic

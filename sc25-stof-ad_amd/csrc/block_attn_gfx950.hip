@@ -62,6 +62,8 @@ struct AttnParams {
   float c;  // softmax_scale * log2(e)
   // row-wise front-ends (KIND != 0): key blocks come from index arithmetic, not from a LUT
   const uint64_t* row_bits; int words; int causal; int band;
+  // precomputed walk (see attn_plan_kernel): one block of plan_stride 8-byte words per (LUT sample, group slot)
+  const uint64_t* plan; int plan_stride;
 };
 
 enum { kKindLut = 0, kKindPred = 1, kKindBits = 2 };
@@ -107,13 +109,28 @@ template <int ROWS> struct RowPtrs {
 // merged through LDS at the end).  The second form halves the work of a wave per key block,
 // so the chain of key blocks of a long LUT row finishes in half the time; it is used for
 // small grids, where that chain and not throughput sets the run time.
-template <int KIND, int ROWS, int KS, bool PIPE, bool BF>
-__device__ __forceinline__ void attn_group(const AttnParams& p, const int bh, const int pair, const RowPtrs<ROWS>& pre,
+template <int KIND, int ROWS, int KS, bool PIPE, bool BF, bool PLAN = false>
+__device__ __forceinline__ void attn_group(const AttnParams& p, const int bh, const int pair_or_slot, const RowPtrs<ROWS>& pre,
                                            unsigned char* k_lds0, unsigned char* k_lds1,
                                            unsigned char* v_lds0, unsigned char* v_lds1,
                                            unsigned char* k_lds2 = nullptr, unsigned char* v_lds2 = nullptr) {
   static_assert(KS == 1 || ROWS == 1, "the key split serves a single query block");
   static_assert(!PIPE || KS == 1, "the software-pipelined loop keeps all 64 keys of a tile in one wave");
+  static_assert(!PLAN || (KIND == kKindLut && !PIPE), "a precomputed walk exists for LUT-driven launches of the plain loop");
+  // PLAN: the group's walk was laid out ahead of time.  Lane l takes word l of the group's plan
+  // block; this one load, issued first of all, replaces the row pointers, the column lists and the
+  // merge of the rows - two dependent round trips through memory and some hundred scalar
+  // instructions between the start of the workgroup and its first K/V tile.
+  int pair = pair_or_slot;
+  uint32_t plan_lo = 0, plan_hi = 0;     // the current window of 64 plan words, one per lane
+  const uint64_t* plan_blk = nullptr;
+  if constexpr (PLAN) {
+    const int sample = p.lut_bs ? bh / p.H : 0;
+    plan_blk = p.plan + ((int64_t)sample * p.nP + pair_or_slot) * p.plan_stride;
+    const int l = threadIdx.x & 63;
+    const uint64_t w = l < p.plan_stride ? plan_blk[l] : 0ull;
+    plan_lo = (uint32_t)w; plan_hi = (uint32_t)(w >> 32);
+  }
   constexpr int kDma = 4 / (ROWS * KS);   // direct-to-LDS instructions per wave and operand tile (8 per tile)
   constexpr int kMT = 2 / KS;             // 32-key sub-tiles of a key block handled by one wave
 
@@ -129,6 +146,13 @@ __device__ __forceinline__ void attn_group(const AttnParams& p, const int bh, co
   __shared__ __attribute__((aligned(256))) float mask_tab[64];
   if (wave == 0) mask_tab[lane] = ((lane >> 2) >> (lane & 3)) & 1 ? -INFINITY : 0.f;
 
+  int plan_n = 0, plan_p0 = 0, plan_i = 0;   // PLAN: steps of the group, first PART slot of this wave's row, next step
+  if constexpr (PLAN) {
+    const uint32_t h0 = __builtin_amdgcn_readlane(plan_lo, 0);
+    pair = h0 & 0xffff;
+    plan_n = h0 >> 16;
+    plan_p0 = rsel == 0 ? __builtin_amdgcn_readlane(plan_lo, 1) : __builtin_amdgcn_readlane(plan_hi, 1);
+  }
   const int b = bh / p.H;
   const int h = bh - b * p.H;
   const int qi = ROWS * pair + rsel;               // this wave's query block
@@ -149,7 +173,9 @@ __device__ __forceinline__ void attn_group(const AttnParams& p, const int bh, co
     row[r].t0 = row[r].n = row[r].p0 = row[r].np = row[r].ptr = row[r].pptr = 0;
     row[r].lo = 0; row[r].hi = -1;
     if (qr < p.nQ) {
-      if (KIND == kKindLut) {
+      if (PLAN) {
+        row[r].n = plan_n;
+      } else if (KIND == kKindLut) {
         if (pre.valid) {   // the placement code has read the row pointers already
           row[r].t0 = pre.t0[r]; row[r].n = pre.n[r]; row[r].p0 = pre.p0[r]; row[r].np = pre.np[r];
         } else {
@@ -175,6 +201,7 @@ __device__ __forceinline__ void attn_group(const AttnParams& p, const int bh, co
   // for Q (HBM), whose latency then overlaps the walk set-up and the first K/V loads.
   int win_e[ROWS], win_pe = 0x7fffffff;
   auto fetch_window = [&]() {
+    if (PLAN) return;
     win_pe = 0x7fffffff;
 #pragma unroll
     for (int r = 0; r < ROWS; ++r) {
@@ -304,9 +331,30 @@ __device__ __forceinline__ void attn_group(const AttnParams& p, const int bh, co
       if (r == rsel) set_mine = m;
     }
   };
-  consume_window(0);
+  if (!PLAN) consume_window(0);
+  uint32_t plan_nlo = 0, plan_nhi = 0;   // PLAN: the window after the current one, requested 16 steps before it is needed
   auto next_step = [&]() -> Step {
     Step s; s.col = 0; s.mine = 0; s.slot = -1; s.valid = false;
+    if constexpr (PLAN) {
+      // word 2 + i of the block is step i: key block (16 bits), listed by row 0 / row 1, partial in
+      // row 0 / row 1 (bits 16-19), and in the upper half the PART slots relative to the rows' first
+      if (plan_i >= plan_n) return s;
+      const int word = plan_i + 2;
+      if ((word & 63) == 0) { plan_lo = plan_nlo; plan_hi = plan_nhi; }
+      const uint32_t lo = __builtin_amdgcn_readlane(plan_lo, word & 63);
+      const uint32_t hi = __builtin_amdgcn_readlane(plan_hi, word & 63);
+      if ((word & 63) == 48 && (word | 63) + 1 < plan_n + 2) {
+        const int at = (word | 63) + 1 + lane;
+        const uint64_t w = at < p.plan_stride ? plan_blk[at] : 0ull;
+        plan_nlo = (uint32_t)w; plan_nhi = (uint32_t)(w >> 32);
+      }
+      ++plan_i;
+      s.valid = true;
+      s.col = lo & 0xffff;
+      s.mine = (lo >> (16 + rsel)) & 1;
+      if (s.mine && ((lo >> (18 + rsel)) & 1)) s.slot = plan_p0 + ((hi >> (16 * rsel)) & 0xffff);
+      return s;
+    }
     while (set_union == 0) {
       if (++win >= n_win) return s;
       fetch_window();
@@ -878,7 +926,7 @@ __device__ __forceinline__ void attn_group(const AttnParams& p, const int bh, co
   for (int i = 0; i < 4; ++i) {
     const int t = 8 * i + (lane >> 3), c = lane & 7;
     const half8_t o = *reinterpret_cast<const __attribute__((address_space(3))) half8_t*>(stage + t * 128 + ((c ^ (t & 7)) << 4));
-    *reinterpret_cast<half8_t*>(ob + (int64_t)t * p.os[2] + 8 * c) = o;
+    __builtin_nontemporal_store(o, reinterpret_cast<half8_t*>(ob + (int64_t)t * p.os[2] + 8 * c));
   }
 }
 
@@ -976,21 +1024,127 @@ __device__ __forceinline__ void balanced_group(const AttnParams& p, int& bh, int
   }
 }
 
-template <int KIND, int ROWS, int KS, bool BF>
+// The placement arithmetic of balanced_group alone: which (batch, head) and which position of
+// the head's length order this workgroup takes.  With a precomputed walk the groups of a LUT
+// are stored in that order already, so nothing has to be read or ranked here.
+__device__ __forceinline__ void balanced_slot(const AttnParams& p, int& bh, int& slot) {
+  const int x = blockIdx.x & 7, i = blockIdx.x >> 3;
+  const int ncu = p.cus_per_xcd;
+  const int hx = p.chunk / p.nP;
+  const int hs = min(hx, max(1, (4 * ncu + p.nP - 1) / p.nP));
+  const int per_set = hs * p.nP;
+  const int s = i / per_set;
+  const int h0 = s * hs;
+  const int hn = min(hs, hx - h0);
+  const int il = i - s * per_set;
+  const int pass = il / ncu, pos = il - pass * ncu;
+  const int plen = min(ncu, hn * p.nP - pass * ncu);
+  const int j = pass * ncu + ((pass & 1) ? plen - 1 - pos : pos);
+  slot = j / hn;
+  bh = x * hx + h0 + (j - slot * hn);
+}
+
+template <int KIND, int ROWS, int KS, bool BF, bool PLAN>
 __global__ __launch_bounds__(128 * ROWS * KS, 4) void block_attn_fwd_kernel(const AttnParams p) {
   STOF_ATTN_LDS_TILES;
   int bh, pair;
   RowPtrs<ROWS> pre;
   pre.valid = false;
   if (p.balance) {
-    balanced_group<KIND, ROWS>(p, bh, pair, pre);
+    if constexpr (PLAN) balanced_slot(p, bh, pair);
+    else balanced_group<KIND, ROWS>(p, bh, pair, pre);
   } else {
     const int vid = xcd_contiguous_id(p);
     if (vid >= p.total) return;
     bh = vid / p.nP;
-    pair = zigzag(vid - bh * p.nP, bh, p.nP);
+    pair = zigzag(vid - bh * p.nP, bh, p.nP);   // (PLAN: a position of the length order - any bijection serves)
   }
-  attn_group<KIND, ROWS, KS, false, BF>(p, bh, pair, pre, k_lds0, k_lds1, v_lds0, v_lds1);
+  attn_group<KIND, ROWS, KS, false, BF, PLAN>(p, bh, pair, pre, k_lds0, k_lds1, v_lds0, v_lds1);
+}
+
+// ---- the walk of every group of a LUT, laid out once per LUT -----------------------------------
+// One block of `stride` 8-byte words per (LUT sample, slot), slot = the group's place when the
+// sample's groups are ordered by descending number of steps (ties: lower group first; more than
+// 64 groups per sample: slot = group).  Word 0: group index (bits 0-15), number of steps (16-31).
+// Word 1: first PART slot of the group's row 0 (low half) and row 1 (high half).  Word 2 + i, step
+// i of the merged ascending walk over the rows' LOAD lists: key block (bits 0-15), listed by row
+// 0 / row 1 (bits 16, 17), partial in row 0 / row 1 (bits 18, 19), PART slot relative to the
+// row's first, row 0 in bits 32-47 and row 1 in bits 48-63.
+constexpr int kPlanMaxKeyBlocks = 1024;   // seq_len <= 65536
+__host__ __device__ inline int plan_stride_words(int nK) { return (nK + 2 + 7) & ~7; }
+
+template <int ROWS>
+__global__ __launch_bounds__(64) void attn_plan_kernel(const int32_t* __restrict__ lrp, const int32_t* __restrict__ lci,
+                                                       const int32_t* __restrict__ prp, const int32_t* __restrict__ pci,
+                                                       int64_t lut_bs, int nQ, int nK, int nP, int stride,
+                                                       uint64_t* __restrict__ plan) {
+  __shared__ unsigned char listed[ROWS][kPlanMaxKeyBlocks];
+  __shared__ unsigned char partial[ROWS][kPlanMaxKeyBlocks];
+  __shared__ unsigned short pslot[ROWS][kPlanMaxKeyBlocks];
+  const int lane = threadIdx.x;
+  const int sample = blockIdx.x / nP, g = blockIdx.x - sample * nP;
+  const int64_t lo = (int64_t)sample * lut_bs;
+  auto clampn = [&](int n) { return n < 0 ? 0 : (n > nK ? nK : n); };
+
+  // the slot: rank of this group among the sample's groups by merged walk length
+  int slot = g;
+  if (nP <= 64) {
+    int len = 0;
+    if (lane < nP) {
+      const int qa = ROWS * lane, qb = qa + 1;
+      const int ta = lrp[lo + qa], na = clampn(lrp[lo + qa + 1] - ta);
+      if (ROWS == 2 && qb < nQ) {
+        const int tb = lrp[lo + qb], nb = clampn(lrp[lo + qb + 1] - tb);
+        int i = 0, j = 0;
+        while (i < na || j < nb) {   // two ascending lists: size of the union
+          const int a = i < na ? lci[ta + i] : 0x7fffffff, b = j < nb ? lci[tb + j] : 0x7fffffff;
+          i += a <= b; j += b <= a; ++len;
+        }
+      } else {
+        len = na;
+      }
+    }
+    const int key = lane < nP ? (len << 6) | (63 - lane) : -1;
+    const int mine = __shfl(key, g, 64);
+    slot = __builtin_popcountll(__ballot(key > mine));
+  }
+
+  for (int r = 0; r < ROWS; ++r)
+    for (int c = lane; c < nK; c += 64) { listed[r][c] = 0; partial[r][c] = 0; }
+  __syncthreads();
+  int p0[2] = {0, 0};
+  for (int r = 0; r < ROWS; ++r) {
+    const int qr = ROWS * g + r;
+    if (qr >= nQ) continue;
+    const int t0 = lrp[lo + qr], n = clampn(lrp[lo + qr + 1] - t0);
+    for (int e = lane; e < n; e += 64) { const int c = lci[t0 + e]; if ((unsigned)c < (unsigned)nK) listed[r][c] = 1; }
+    p0[r] = prp[lo + qr];
+    const int np = clampn(prp[lo + qr + 1] - p0[r]);
+    for (int e = lane; e < np; e += 64) { const int c = pci[p0[r] + e]; if ((unsigned)c < (unsigned)nK) { partial[r][c] = 1; pslot[r][c] = (unsigned short)e; } }
+  }
+  __syncthreads();
+
+  uint64_t* blk = plan + ((int64_t)sample * nP + slot) * stride;
+  int base = 0;
+  for (int w = 0; w * 64 < nK; ++w) {
+    const int c = 64 * w + lane;
+    const bool in0 = c < nK && listed[0][c];
+    const bool in1 = ROWS == 2 && c < nK && listed[ROWS - 1][c];
+    const uint64_t any = __ballot(in0 || in1);
+    if (in0 || in1) {
+      const int pos = base + __builtin_popcountll(any & ((1ull << lane) - 1));
+      const bool pa0 = in0 && partial[0][c], pa1 = in1 && partial[ROWS - 1][c];
+      uint64_t word = (uint64_t)c | ((uint64_t)in0 << 16) | ((uint64_t)in1 << 17) | ((uint64_t)pa0 << 18) | ((uint64_t)pa1 << 19);
+      if (pa0) word |= (uint64_t)pslot[0][c] << 32;
+      if (pa1) word |= (uint64_t)pslot[ROWS - 1][c] << 48;
+      blk[2 + pos] = word;
+    }
+    base += __builtin_popcountll(any);
+  }
+  if (lane == 0) {
+    blk[0] = (uint64_t)g | ((uint64_t)base << 16);
+    blk[1] = (uint64_t)(uint32_t)p0[0] | ((uint64_t)(uint32_t)p0[1] << 32);
+  }
 }
 
 // Two query blocks per workgroup with the software-pipelined main loop (rings of three K and
@@ -1124,8 +1278,10 @@ void set_balance(AttnParams& p, int max_groups) {
   p.balance = (p.total % 8 == 0 && p.chunk % p.nP == 0 && p.nP <= max_groups && p.nP > 1 && cus % 8 == 0 && cus >= 8) ? 1 : 0;
 }
 
+// plan_rows: query blocks per group of the plan in p.plan (0: none).  A plan laid out for the
+// other group size is ignored (the kernel then walks the LUT itself).
 template <int KIND, bool BF>
-void launch_attn_as(AttnParams& p, int nQ, int64_t bh, int requested_form, hipStream_t stream) {
+void launch_attn_as(AttnParams& p, int nQ, int64_t bh, int requested_form, int plan_rows, hipStream_t stream) {
   const int64_t two_row_groups = (int64_t)((nQ + kRowsPerGroup - 1) / kRowsPerGroup) * bh;
   const int form = pick_form(requested_form, two_row_groups, nQ);
   if (form == kFormKeySplit) {
@@ -1133,23 +1289,36 @@ void launch_attn_as(AttnParams& p, int nQ, int64_t bh, int requested_form, hipSt
     p.total = (int)(nQ * bh);
     p.chunk = (p.total + 7) / 8;
     set_balance(p, kBalanceMaxGroupsKeySplit);
-    hipLaunchKernelGGL((block_attn_fwd_kernel<KIND, 1, 2, BF>), dim3(p.chunk * 8), dim3(256), 0, stream, p);
+    if constexpr (KIND == kKindLut) {
+      if (p.plan && plan_rows == 1) {
+        hipLaunchKernelGGL((block_attn_fwd_kernel<KIND, 1, 2, BF, true>), dim3(p.chunk * 8), dim3(256), 0, stream, p);
+        return;
+      }
+    }
+    hipLaunchKernelGGL((block_attn_fwd_kernel<KIND, 1, 2, BF, false>), dim3(p.chunk * 8), dim3(256), 0, stream, p);
   } else {
     p.nP = (nQ + kRowsPerGroup - 1) / kRowsPerGroup;
     p.total = (int)two_row_groups;
     p.chunk = (p.total + 7) / 8;
     set_balance(p, kBalanceMaxGroupsTwoRows);
-    if (form == kFormPipelined)
+    if (form == kFormPipelined) {
       hipLaunchKernelGGL((block_attn_pipe_kernel<KIND, BF>), dim3(p.chunk * 8), dim3(256), 0, stream, p);
-    else
-      hipLaunchKernelGGL((block_attn_fwd_kernel<KIND, kRowsPerGroup, 1, BF>), dim3(p.chunk * 8), dim3(128 * kRowsPerGroup), 0, stream, p);
+      return;
+    }
+    if constexpr (KIND == kKindLut) {
+      if (p.plan && plan_rows == kRowsPerGroup) {
+        hipLaunchKernelGGL((block_attn_fwd_kernel<KIND, kRowsPerGroup, 1, BF, true>), dim3(p.chunk * 8), dim3(128 * kRowsPerGroup), 0, stream, p);
+        return;
+      }
+    }
+    hipLaunchKernelGGL((block_attn_fwd_kernel<KIND, kRowsPerGroup, 1, BF, false>), dim3(p.chunk * 8), dim3(128 * kRowsPerGroup), 0, stream, p);
   }
 }
 
 template <int KIND>
-void launch_attn(AttnParams& p, int nQ, int64_t bh, int requested_form, int dtype, hipStream_t stream) {
-  if (dtype == STOF_DTYPE_BF16) launch_attn_as<KIND, true>(p, nQ, bh, requested_form, stream);
-  else launch_attn_as<KIND, false>(p, nQ, bh, requested_form, stream);
+void launch_attn(AttnParams& p, int nQ, int64_t bh, int requested_form, int dtype, int plan_rows, hipStream_t stream) {
+  if (dtype == STOF_DTYPE_BF16) launch_attn_as<KIND, true>(p, nQ, bh, requested_form, plan_rows, stream);
+  else launch_attn_as<KIND, false>(p, nQ, bh, requested_form, plan_rows, stream);
 }
 
 bool strides_ok(const int64_t s[3]) {
@@ -1168,6 +1337,48 @@ extern "C" int stof_attn_set_launch_form(int form) {
   return STOF_OK;
 }
 
+extern "C" int stof_attn_plan_rows(int batch_size, int head_num, int seq_len, int launch_form) {
+  if (batch_size <= 0 || head_num <= 0 || seq_len <= 0 || seq_len % kBM != 0) return STOF_ERR_BAD_SHAPE;
+  if (launch_form < kFormAuto || launch_form > kFormPipelined) return STOF_ERR_UNSUPPORTED;
+  const int nQ = seq_len / kBM;
+  const int64_t bh = (int64_t)batch_size * head_num;
+  const int form = pick_form(launch_form, (int64_t)((nQ + kRowsPerGroup - 1) / kRowsPerGroup) * bh, nQ);
+  if (form == kFormPipelined) return 0;
+  return form == kFormKeySplit ? 1 : kRowsPerGroup;
+}
+
+extern "C" int64_t stof_attn_plan_bytes(int seq_len, int rows_per_group, int lut_batches) {
+  if (seq_len <= 0 || seq_len % kBM != 0 || lut_batches <= 0 || (rows_per_group != 1 && rows_per_group != kRowsPerGroup)) return 0;
+  const int nK = seq_len / kBN, nQ = seq_len / kBM;
+  if (nK > kPlanMaxKeyBlocks) return 0;
+  const int nP = (nQ + rows_per_group - 1) / rows_per_group;
+  return (int64_t)lut_batches * nP * plan_stride_words(nK) * 8;
+}
+
+extern "C" int stof_attn_plan_build(const int32_t* part_row_ptr, const int32_t* part_col_idx,
+                                    const int32_t* load_row_ptr, const int32_t* load_col_idx,
+                                    int seq_len, int64_t lut_batch_stride, int lut_batches, int rows_per_group,
+                                    void* plan, int64_t plan_bytes, void* stream) {
+  if (!part_row_ptr || !load_row_ptr || !plan) return STOF_ERR_NULL_POINTER;
+  const int64_t need = stof_attn_plan_bytes(seq_len, rows_per_group, lut_batches);
+  if (need == 0) return STOF_ERR_UNSUPPORTED;
+  if (plan_bytes < need) return STOF_ERR_BAD_SHAPE;
+  if ((reinterpret_cast<uintptr_t>(plan) & 7) != 0) return STOF_ERR_MISALIGNED;
+  const int nK = seq_len / kBN, nQ = seq_len / kBM;
+  if (lut_batches > 1 && lut_batch_stride < nQ + 1) return STOF_ERR_BAD_LUT;
+  const int nP = (nQ + rows_per_group - 1) / rows_per_group;
+  if ((int64_t)lut_batches * nP > (int64_t)1 << 30) return STOF_ERR_BAD_SHAPE;
+  const dim3 grid((unsigned)(lut_batches * nP));
+  const int64_t bs = lut_batches > 1 ? lut_batch_stride : 0;
+  if (rows_per_group == 1)
+    hipLaunchKernelGGL((attn_plan_kernel<1>), grid, dim3(64), 0, (hipStream_t)stream, load_row_ptr, load_col_idx,
+                       part_row_ptr, part_col_idx, bs, nQ, nK, nP, plan_stride_words(nK), (uint64_t*)plan);
+  else
+    hipLaunchKernelGGL((attn_plan_kernel<kRowsPerGroup>), grid, dim3(64), 0, (hipStream_t)stream, load_row_ptr, load_col_idx,
+                       part_row_ptr, part_col_idx, bs, nQ, nK, nP, plan_stride_words(nK), (uint64_t*)plan);
+  return stof_check_launch();
+}
+
 extern "C" int stof_block_attn_fwd(
     const void* q, const void* k, const void* v, void* out,
     const int32_t* full_row_ptr, const int32_t* full_col_idx,
@@ -1178,6 +1389,23 @@ extern "C" int stof_block_attn_fwd(
     const int64_t v_strides[3], const int64_t out_strides[3],
     int batch_size, int seq_len, int head_num, int head_size, int dtype,
     int64_t lut_batch_stride, int launch_form, void* stream) {
+  return stof_block_attn_fwd_planned(q, k, v, out, full_row_ptr, full_col_idx, part_row_ptr, part_col_idx, part_bitmask,
+                                     load_row_ptr, load_col_idx, block_m, block_n, softmax_scale, q_strides, k_strides,
+                                     v_strides, out_strides, batch_size, seq_len, head_num, head_size, dtype,
+                                     lut_batch_stride, launch_form, nullptr, 0, 0, stream);
+}
+
+extern "C" int stof_block_attn_fwd_planned(
+    const void* q, const void* k, const void* v, void* out,
+    const int32_t* full_row_ptr, const int32_t* full_col_idx,
+    const int32_t* part_row_ptr, const int32_t* part_col_idx, const uint64_t* part_bitmask,
+    const int32_t* load_row_ptr, const int32_t* load_col_idx,
+    int block_m, int block_n, float softmax_scale,
+    const int64_t q_strides[3], const int64_t k_strides[3],
+    const int64_t v_strides[3], const int64_t out_strides[3],
+    int batch_size, int seq_len, int head_num, int head_size, int dtype,
+    int64_t lut_batch_stride, int launch_form,
+    const void* plan, int64_t plan_bytes, int plan_rows, void* stream) {
   if (launch_form < kFormAuto || launch_form > kFormPipelined) return STOF_ERR_UNSUPPORTED;
   if (dtype != STOF_DTYPE_F16 && dtype != STOF_DTYPE_BF16) return STOF_ERR_UNSUPPORTED;
   if (!q || !k || !v || !out || !full_row_ptr || !part_row_ptr || !load_row_ptr ||
@@ -1206,7 +1434,15 @@ extern "C" int stof_block_attn_fwd(
   p.B = batch_size; p.S = seq_len; p.H = head_num; p.nQ = nQ;
   p.c = softmax_scale * 1.4426950408889634f;
   p.row_bits = nullptr; p.words = 0; p.causal = 0; p.band = 0;
-  launch_attn<kKindLut>(p, nQ, (int64_t)batch_size * head_num, launch_form, dtype, (hipStream_t)stream);
+  p.plan = nullptr; p.plan_stride = 0;
+  if (plan) {
+    const int64_t need = stof_attn_plan_bytes(seq_len, plan_rows, lut_batch_stride ? batch_size : 1);
+    if (need == 0 || plan_bytes < need) return STOF_ERR_BAD_SHAPE;
+    if ((reinterpret_cast<uintptr_t>(plan) & 7) != 0) return STOF_ERR_MISALIGNED;
+    p.plan = (const uint64_t*)plan;
+    p.plan_stride = plan_stride_words(seq_len / kBN);
+  }
+  launch_attn<kKindLut>(p, nQ, (int64_t)batch_size * head_num, launch_form, dtype, plan ? plan_rows : 0, (hipStream_t)stream);
   return stof_check_launch();
 }
 
@@ -1237,8 +1473,9 @@ extern "C" int stof_rowwise_attn_fwd(
   p.c = (1.0f / sqrtf((float)head_size)) * 1.4426950408889634f;
   p.row_bits = mask_bits; p.words = seq_len / 64; p.causal = is_causal ? 1 : 0;
   p.band = kind == STOF_ROW_SLIDING ? bandwidth : 0;
-  if (kind == STOF_ROW_MASK) launch_attn<kKindBits>(p, nQ, (int64_t)batch_size * head_num, launch_form, dtype, (hipStream_t)stream);
-  else launch_attn<kKindPred>(p, nQ, (int64_t)batch_size * head_num, launch_form, dtype, (hipStream_t)stream);
+  p.plan = nullptr; p.plan_stride = 0;
+  if (kind == STOF_ROW_MASK) launch_attn<kKindBits>(p, nQ, (int64_t)batch_size * head_num, launch_form, dtype, 0, (hipStream_t)stream);
+  else launch_attn<kKindPred>(p, nQ, (int64_t)batch_size * head_num, launch_form, dtype, 0, (hipStream_t)stream);
   return stof_check_launch();
 }
 

@@ -22,6 +22,13 @@ _SIGNATURES = {
                                     c_int, c_int, c_float,
                                     POINTER(c_int64), POINTER(c_int64), POINTER(c_int64), POINTER(c_int64),
                                     c_int, c_int, c_int, c_int, c_int, c_int64, c_int, _P]),
+    "stof_block_attn_fwd_planned": (c_int, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P,
+                                            c_int, c_int, c_float,
+                                            POINTER(c_int64), POINTER(c_int64), POINTER(c_int64), POINTER(c_int64),
+                                            c_int, c_int, c_int, c_int, c_int, c_int64, c_int, _P, c_int64, c_int, _P]),
+    "stof_attn_plan_rows": (c_int, [c_int, c_int, c_int, c_int]),
+    "stof_attn_plan_bytes": (c_int64, [c_int, c_int, c_int]),
+    "stof_attn_plan_build": (c_int, [_P, _P, _P, _P, c_int, c_int64, c_int, c_int, _P, c_int64, _P]),
     "stof_attn_set_launch_form": (c_int, [c_int]),
     "stof_pack_mask_bits": (c_int, [_P, _P, c_int64, c_int64, c_int64, c_int, _P]),
     "stof_rowwise_attn_fwd": (c_int, [_P, _P, _P, _P, c_int, c_int, c_int, _P,

@@ -181,7 +181,7 @@ def _prepared_lut(lut, B, S, block_m, block_n, dev):
     key = (B, S, block_m, block_n, dev) + tuple((id(t),) + _content_key(t) for t in lut)
     cached = getattr(lci, _LUT_READY_ATTR, None)
     if cached is not None and cached[0] == key:
-        return cached[1], cached[2]
+        return cached[1], cached[2], cached[5]
     frp, fci, prp, pci, pbm, lrp, lci = lut
     frp = _check_i32("full_row_ptr", frp, dev); fci = _check_i32("full_col_idx", fci, dev)
     prp = _check_i32("part_row_ptr", prp, dev); pci = _check_i32("part_col_idx", pci, dev)
@@ -204,11 +204,36 @@ def _prepared_lut(lut, B, S, block_m, block_n, dev):
     bits = _packed_partial_bits(pbm)
     keep = (frp, fci, prp, pci, bits, lrp, lci_c)
     ptrs = tuple(_ptr(t) for t in keep)
+    plans = {}   # rows per workgroup -> plan tensor (see _plan), filled on first use
     try:
-        setattr(lci, _LUT_READY_ATTR, (key, ptrs, lut_bs, keep, tuple(lut)))   # holds what the key and the pointers refer to
+        setattr(lci, _LUT_READY_ATTR, (key, ptrs, lut_bs, keep, tuple(lut), plans))   # holds what the key and the pointers refer to
     except AttributeError:
         pass
-    return ptrs, lut_bs
+    return ptrs, lut_bs, plans
+
+
+def _plan(plans, lut_ptrs, lut_bs, B, H, S, form, dev):
+    """The precomputed walk of this LUT for the launch form the library will take (built by one
+    small launch the first time a LUT meets that form, then kept with the LUT's other prepared
+    data).  Returns (pointer, bytes, rows per workgroup) or (None, 0, 0) where no plan applies."""
+    lib = _lib.lib()
+    rows = lib.stof_attn_plan_rows(B, H, S, form)
+    if rows <= 0:
+        return None, 0, 0
+    plan = plans.get(rows)
+    if plan is None:
+        batches = B if lut_bs else 1
+        nbytes = lib.stof_attn_plan_bytes(S, rows, batches)
+        if nbytes <= 0:
+            plans[rows] = False
+            return None, 0, 0
+        plan = torch.empty(nbytes // 8, dtype=torch.int64, device=dev)
+        check(lib.stof_attn_plan_build(lut_ptrs[2], lut_ptrs[3], lut_ptrs[5], lut_ptrs[6], S, lut_bs, batches, rows,
+                                       plan.data_ptr(), nbytes, _stream(dev)), "stof_attn_plan_build")
+        plans[rows] = plan
+    if plan is False:
+        return None, 0, 0
+    return plan.data_ptr(), plan.numel() * 8, rows
 
 
 def _check_i32(name, t, device):
@@ -218,7 +243,7 @@ def _check_i32(name, t, device):
 
 
 def block_attn(q, k, v, lut, block_m=64, block_n=64, out=None, out_layout="bhsd", softmax_scale=None,
-               launch_form=None, revalidate=False):
+               launch_form=None, revalidate=False, use_plan=True):
     """Block-masked attention.  q, k, v: fp16 (or, all three, bfloat16) views ``[B,H,S,D]`` with
     unit stride in D (any other strides).  ``lut`` = (full_row_ptr, full_col_idx, part_row_ptr, part_col_idx,
     part_block_mask, load_row_ptr, load_col_idx) as returned by ``get_sparse_storage`` (the
@@ -228,7 +253,9 @@ def block_attn(q, k, v, lut, block_m=64, block_n=64, out=None, out_layout="bhsd"
 
     ``launch_form``: ``None`` / ``"default"`` (the process default, automatic by grid size
     unless ``set_attention_launch_form`` changed it), ``"two_rows"`` or ``"key_split"`` - the
-    per-call counterpart of the reference's ``num_warps``.  ``revalidate=True`` discards what
+    per-call counterpart of the reference's ``num_warps``.  ``use_plan=False`` makes the kernel
+    read the LUT itself instead of the walk laid out once per LUT (same result bit for bit; the
+    plan saves the dependent LUT reads at the start of every workgroup).  ``revalidate=True`` discards what
     is cached for this LUT (validation, packed bit rows, re-tiling) and prepares it again: for
     LUT buffers rewritten behind PyTorch's back, which the caches cannot see.
     """
@@ -244,7 +271,7 @@ def block_attn(q, k, v, lut, block_m=64, block_n=64, out=None, out_layout="bhsd"
     form = _form(launch_form)
     if revalidate:
         _drop_caches(lut)
-    lut_ptrs, lut_bs = _prepared_lut(lut, B, S, block_m, block_n, dev)
+    lut_ptrs, lut_bs, plans = _prepared_lut(lut, B, S, block_m, block_n, dev)
     if out is None:
         if out_layout == "bhsd":
             out = torch.empty((B, H, S, D), dtype=q.dtype, device=dev)
@@ -260,11 +287,12 @@ def block_attn(q, k, v, lut, block_m=64, block_n=64, out=None, out_layout="bhsd"
         raise StofError(f"unknown out_layout {out_layout!r}")
     _require(out.dtype == q.dtype and out.device == dev, "out must have q's dtype and device")
     scale = softmax_scale if softmax_scale is not None else 1.0 / math.sqrt(D)
-    check(_lib.lib().stof_block_attn_fwd(
+    plan_ptr, plan_bytes, plan_rows = _plan(plans, lut_ptrs, lut_bs, B, H, S, form, dev) if use_plan else (None, 0, 0)
+    check(_lib.lib().stof_block_attn_fwd_planned(
         q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(),
         *lut_ptrs, 64, 64, scale,
         strides3(q), strides3(k), strides3(v), ostr,
-        B, S, H, D, _DTYPES[q.dtype], lut_bs, form, _stream(dev)), "stof_block_attn_fwd")
+        B, S, H, D, _DTYPES[q.dtype], lut_bs, form, plan_ptr, plan_bytes, plan_rows, _stream(dev)), "stof_block_attn_fwd")
     return out
 
 

@@ -37,7 +37,7 @@ def test_every_declared_symbol_is_exported_and_bound(lib):
 
 
 def test_version_and_status_strings(lib):
-    assert lib.stof_abi_version() == 3
+    assert lib.stof_abi_version() == 4
     for code in (0, -1, -2, -3, -4, -5, -6, -7, -99):
         assert len(lib.stof_status_string(code)) > 0
 
@@ -62,6 +62,27 @@ def test_block_attn_argument_checks(lib):
     assert call(lbs=2) == -6             # per-sample LUT stride too small
     assert call(form=3) == -3            # launch form
     assert call(dtype=2) == -3           # element format
+
+
+def test_attention_plan_argument_checks(lib):
+    P = 4096
+    # bytes: (query-block groups) x (key blocks + 2 header words, rounded up to 8) x 8 per LUT sample
+    assert lib.stof_attn_plan_bytes(4096, 2, 1) == 32 * 72 * 8
+    assert lib.stof_attn_plan_bytes(4096, 1, 3) == 3 * 64 * 72 * 8
+    assert lib.stof_attn_plan_bytes(192, 2, 1) == 2 * 8 * 8
+    assert lib.stof_attn_plan_bytes(65536 + 64, 2, 1) == 0      # beyond the plan's key-block range
+    assert lib.stof_attn_plan_bytes(4096, 3, 1) == 0
+    assert lib.stof_attn_plan_bytes(100, 2, 1) == 0
+    assert lib.stof_attn_plan_build(None, P, P, P, 512, 0, 1, 2, P, 1 << 20, None) == -1
+    assert lib.stof_attn_plan_build(P, P, P, P, 512, 0, 1, 2, P, 8, None) == -2          # buffer too small
+    assert lib.stof_attn_plan_build(P, P, P, P, 512, 0, 1, 2, P + 4, 1 << 20, None) == -4
+    assert lib.stof_attn_plan_build(P, P, P, P, 512, 4, 2, 2, P, 1 << 20, None) == -6     # row-pointer stride too small
+    assert lib.stof_attn_plan_build(P, P, P, P, 1 << 20, 0, 1, 2, P, 1 << 30, None) == -3
+    assert lib.stof_attn_plan_rows(1, 12, 100, -1) == -2
+    assert lib.stof_attn_plan_rows(1, 12, 512, 5) == -3
+    assert lib.stof_attn_plan_rows(8, 12, 1024, 0) == 2
+    assert lib.stof_attn_plan_rows(8, 12, 1024, 1) == 1
+    assert lib.stof_attn_plan_rows(8, 12, 1024, 2) == 0
 
 
 def test_other_entry_points_argument_checks(lib):
