@@ -120,7 +120,10 @@ __device__ __forceinline__ void store_wave_block(const GemmParams& p, const floa
       const int t = 8 * i + (lane >> 3), c = lane & 7;
       const half8_t o = *reinterpret_cast<const __attribute__((address_space(3))) half8_t*>(stage + t * 128 + ((c ^ (t & 7)) << 4));
       const int m = m_base + 32 * mi + t, n = n_base + 8 * c;
-      if (m < p.M && n < p.N) *reinterpret_cast<half8_t*>(p.C + (int64_t)m * p.ldc + n) = o;
+      // (written through the XCD's cache, so the tile is on its way to memory while the kernel runs and
+      // not part of the end-of-kernel write-back the next launch waits for: a BERT-large layer of five
+      // launches at 8192 tokens 282 -> 269 us, BERT-base 185 -> 184)
+      if (m < p.M && n < p.N) stof_store16_through(p.C + (int64_t)m * p.ldc + n, o);
     }
   }
 }
@@ -948,7 +951,7 @@ __global__ __launch_bounds__(256) void gemm_bias_res_ln_cluster_kernel(const LnC
       const int t = 8 * ii + (lane >> 3), c = lane & 7;
       const half8_t o = *reinterpret_cast<const __attribute__((address_space(3))) half8_t*>(stage + t * 128 + ((c ^ (t & 7)) << 4));
       const int m = m0 + 64 * wm + 32 * mi + t;
-      if (m < p.M) *reinterpret_cast<half8_t*>(p.C + (int64_t)m * p.ldc + nb + 8 * c) = o;
+      if (m < p.M) stof_store16_through(p.C + (int64_t)m * p.ldc + nb + 8 * c, o);
     }
   }
 

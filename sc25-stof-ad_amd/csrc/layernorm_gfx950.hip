@@ -92,7 +92,7 @@ __global__ __launch_bounds__(256) void bias_res_ln_kernel(const LnParams p) {
         if (p.beta) t += bt[i];
         o[i] = to_elem<BF>(t);
       }
-      *reinterpret_cast<half8_t*>(yr + 8 * ch) = o;
+      stof_store16_through(yr + 8 * ch, o);
     }
   }
 }

@@ -80,6 +80,12 @@ template <int ACT> __device__ __forceinline__ float activate(float x) {
   return x;
 }
 
+// 16-byte store written through the XCD's L2 at device scope (sc1): for output rows nobody in
+// this launch reads again.
+__device__ __forceinline__ void stof_store16_through(half_t* dst, half8_t v) {
+  asm volatile("global_store_dwordx4 %0, %1, off sc1" :: "v"(dst), "v"(v) : "memory");
+}
+
 static inline int stof_check_launch() {
   return hipGetLastError() == hipSuccess ? STOF_OK : STOF_ERR_LAUNCH;
 }
