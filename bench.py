@@ -175,6 +175,8 @@ def bench_layer_c3(steps, warmup):
     layer = EncoderLayer(w, cfg.heads, eps=cfg.eps, ln_fusion="auto")
     out["stages_ms"] = {name: time_region(fn, steps, warmup)[1] for name, fn in layer.stages(x, lut)}
     out["layer_ms_without_qkv_gemm"] = sum(v for k, v in out["stages_ms"].items() if k != "qkv_gemm")
+    from stof import fused
+    fused.check_cluster_exchange()             # a cluster-form LayerNorm GEMM that gave up a wait above would have timed garbage
     best = out["auto_ms"]                      # what ln_fusion="auto", the default, runs
     out["layer_ms"] = best
     out["speedup_vs_eager"] = out["eager_ms"] / best
@@ -252,6 +254,8 @@ def bench_stack_c5(steps, warmup):
         for w in ws:
             h = eager_layer(h, w, maskg, cfg.heads, cfg.eps)
         return h
+    from stof import fused
+    fused.check_cluster_exchange()
     with torch.no_grad():
         check = output_check(y, eager(), bound=1e-1)     # 24 chained fp16 layers on both sides
         eager_ms, _ = time_region(eager, max(steps // 2, 3), 2)

@@ -48,7 +48,7 @@
 extern "C" {
 #endif
 
-#define STOF_ABI_VERSION 4   /* 4: attention plan entry points added; 3: split-K and element-format entry points (nothing removed or changed) */
+#define STOF_ABI_VERSION 4   /* 4: attention plan entry points and the cluster form with a wait limit added, the two process-wide setters (attention launch form, cluster spin limit) removed - both are per-call arguments, the library keeps no mutable state; 3: split-K and element-format entry points (nothing removed or changed) */
 
 enum {
   STOF_OK = 0,
@@ -107,8 +107,7 @@ const char* stof_status_string(int status);
  *
  * launch_form is the per-call counterpart of the reference launcher's num_warps (its kernel
  * selection by (num_warps, BLOCK_M, BLOCK_N), block_attn_mask_cuda.cu:6064-6322):
- *   STOF_FORM_DEFAULT (-1) the process default (automatic by grid size unless
- *                          stof_attn_set_launch_form changed it);
+ *   STOF_FORM_DEFAULT (-1) chosen by the library from the grid size;
  *   STOF_FORM_TWO_ROWS (0) two query blocks per workgroup, K/V tiles shared by four wavefronts
  *                          (large grids);
  *   STOF_FORM_KEY_SPLIT (1) one query block per workgroup, the 64 keys of every tile split over
@@ -169,14 +168,6 @@ int stof_block_attn_fwd_planned(
     int batch_size, int seq_len, int head_num, int head_size, int dtype,
     int64_t lut_batch_stride, int launch_form,
     const void* plan, int64_t plan_bytes, int plan_rows, void* stream);
-
-/*
- * Process-wide default launch form, used by calls that pass STOF_FORM_DEFAULT: -1 automatic
- * (the initial state), 0 / 1 as above.  A convenience for harnesses that sweep the forms
- * without touching their call sites; calls that name a form are not affected by it.
- * Returns STOF_ERR_UNSUPPORTED for another value.
- */
-int stof_attn_set_launch_form(int form);
 
 /*
  * Pack fp16 mask rows into bit rows: dst[r*(cols/64) + w] bit t = pred(src[r*ld + 64*w + t]).
@@ -347,17 +338,25 @@ int stof_gemm_bias_res_ln(const void* A, const void* Wt, const void* bias, const
  * time (calls sharing a workspace on different streams race).  The first 4 bytes are an error
  * word: a workgroup whose bounded wait for its partners ran out sets it to 1 (the output is
  * then invalid); it is never set in normal operation and stays set until the caller clears it.
- * The launch is at most two workgroups per compute unit, which all run at once when the device
- * is otherwise free; each takes its tiles one after another.  A kernel of another stream that
+ * The launch is at most as many workgroups as run at once (two per compute unit; the runtime's
+ * occupancy figure for the kernel is asked, and a device that holds less than one row block's
+ * workgroups per XCD returns STOF_ERR_UNSUPPORTED); each takes its tiles one after another.  They
+ * all run at once when the device is otherwise free.  A kernel of another stream or process that
  * keeps compute units occupied for longer than the wait lasts (about 0.1 s) can keep part of the
- * grid from starting and make the waits of the rest run out: check the error word where such
- * kernels share the device.
+ * grid from starting and make the waits of the rest run out: where such kernels share the
+ * device, read the error word after the work that used this form (any later point will do: the
+ * word stays set), or use stof_gemm_bias_act + stof_bias_res_ln instead.
  */
 int64_t stof_gemm_bias_res_ln_cluster_workspace_bytes(int64_t M, int64_t N);
-/* Number of polls after which a wave of the cluster kernel stops waiting for its partners and sets the
- * error word (process-wide; 0 restores the default of 2^18, about a tenth of a second).  Meant for
- * tests of that path: with a limit of 1 a launch ends normally with the error word set. */
-int stof_gemm_bias_res_ln_cluster_set_spin_limit(int polls);
+/* stof_gemm_bias_res_ln_cluster_dt with the length of the bounded wait as an argument: spin_limit polls
+ * (0 = the default of 2^18, about a tenth of a second) before a wave gives up and sets the error
+ * word.  With a limit of 1 a launch ends normally with the error word set: the way to test a
+ * caller's handling of that word without disturbing the device. */
+int stof_gemm_bias_res_ln_cluster_bounded(const void* A, const void* Wt, const void* bias, const void* residual,
+                                          const void* gamma, const void* beta, void* C,
+                                          int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldr, int64_t ldc,
+                                          float eps, void* workspace, int64_t workspace_bytes, int dtype,
+                                          int spin_limit, void* stream);
 int stof_gemm_bias_res_ln_cluster(const void* A, const void* Wt, const void* bias, const void* residual,
                                   const void* gamma, const void* beta, void* C,
                                   int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldr, int64_t ldc,

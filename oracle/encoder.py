@@ -111,7 +111,8 @@ def bert_layer(x, p, mask, n_heads, eps=1e-5, gelu="erf", dtype=torch.float32, r
     result, the first LayerNorm's output, the FFN activation, the layer output) to fp16, as
     the reference's fp16 eager layer does at the same points; all arithmetic inside an
     operator stays in ``dtype``.  ``round_fp16="split"`` additionally rounds the two products
-    that feed a LayerNorm (the eager layer's fp16 matmul outputs, :73 and :83).  ``gelu``: "erf" (:81), "tanh" (new_gelu, :25-26) or "relu" (:206).
+    that feed a LayerNorm (the eager layer's fp16 matmul outputs, :73 and :83); a pair of flags
+    ``(attention-output product, FFN-output product)`` rounds only the ones named.  ``gelu``: "erf" (:81), "tanh" (new_gelu, :25-26) or "relu" (:206).
 
     ``p`` is a dict of weights in the reference's [in, out] orientation:
     W_qkv [D,3D] (or None: then p['qkv_act'] [B,S,3D] plays the reference's
@@ -126,6 +127,10 @@ def bert_layer(x, p, mask, n_heads, eps=1e-5, gelu="erf", dtype=torch.float32, r
         qkv = torch.matmul(x, p["W_qkv"].to(dtype)) + p["b_qkv"].to(dtype)
     else:
         qkv = p["qkv_act"].to(dtype) + p["b_qkv"].to(dtype)
+    rp_o = rp_2 = round_fp16 == "split"
+    if isinstance(round_fp16, tuple):
+        rp_o, rp_2 = bool(round_fp16[0]), bool(round_fp16[1])
+        round_fp16 = True
     qkv = _r16(qkv, round_fp16)
     q, k, v = qkv.chunk(3, dim=-1)
     q = transpose_for_scores(q, n_heads, hd)
@@ -133,9 +138,8 @@ def bert_layer(x, p, mask, n_heads, eps=1e-5, gelu="erf", dtype=torch.float32, r
     v = transpose_for_scores(v, n_heads, hd)
     h = dense_masked_attention(q, k, v, mask, dtype)
     h = _r16(h.permute(0, 2, 1, 3).contiguous().view(x.shape), round_fp16)
-    rp = round_fp16 == "split"
-    h = _r16(gemm_bias_residual_layernorm(h, p["W_o"], p["b_o"], x, p["g1"], p["be1"], eps, dtype, rp), round_fp16)
+    h = _r16(gemm_bias_residual_layernorm(h, p["W_o"], p["b_o"], x, p["g1"], p["be1"], eps, dtype, rp_o), round_fp16)
     r = h
     act = {"erf": "gelu", "tanh": "gelu_tanh", "relu": "relu"}[gelu]
     h = _r16(gemm_bias_act(h, p["W_1"], p["b_1"], act, dtype), round_fp16)
-    return _r16(gemm_bias_residual_layernorm(h, p["W_2"], p["b_2"], r, p["g2"], p["be2"], eps, dtype, rp), round_fp16)
+    return _r16(gemm_bias_residual_layernorm(h, p["W_2"], p["b_2"], r, p["g2"], p["be2"], eps, dtype, rp_2), round_fp16)

@@ -922,6 +922,7 @@ __device__ __forceinline__ void attn_group(const AttnParams& p, const int bh, co
       for (int e = 0; e < 4; ++e) o4[e] = to_elem<BF>(oacc[dt][4 * q4 + e] * inv);
       *reinterpret_cast<__attribute__((address_space(3))) half4_t*>(stage + j32 * 128 + (((4 * dt + q4) ^ (j32 & 7)) << 4) + 8 * g) = o4;
     }
+  const __amdgpu_buffer_rsrc_t o_rsrc = stof_wave_rsrc(ob);   // this wave's 32 output rows (their span is below 2^31 bytes: see strides_ok)
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const int t = 8 * i + (lane >> 3), c = lane & 7;
@@ -931,7 +932,7 @@ __device__ __forceinline__ void attn_group(const AttnParams& p, const int bh, co
     // the next launch waits for: B2 H16 S4096 sparse 40.3 -> 39.4 us per launch, B8 H12 S1024
     // 22.5 -> 21.0, B16 H12 S512 15.6 -> 14.0; inside an encoder layer the following GEMM reads the
     // rows at the same speed (a non-temporal store measured the same alone but slowed that GEMM).
-    stof_store16_through(ob + (int64_t)t * p.os[2] + 8 * c, o);
+    stof_store16_through(o_rsrc, (uint32_t)t * (uint32_t)(p.os[2] * 2) + 16 * c, o);
   }
 }
 
@@ -1236,7 +1237,6 @@ __global__ __launch_bounds__(256) void pack_mask_bits_kernel(const half_t* __res
 // longest chain of key blocks: the chain runs twice as fast.
 constexpr int kRowsPerGroup = 2;
 enum { kFormAuto = -1, kFormTwoRows = 0, kFormKeySplit = 1, kFormPipelined = 2 };
-int g_attn_form = kFormAuto;
 
 // Automatic choice: key split when the sequence has at least kKeySplitMinQueryBlocks query
 // blocks AND the two-row grid gives a compute unit at most kKeySplitMaxGroupsPerCu workgroups.
@@ -1262,7 +1262,6 @@ int compute_units() {
 
 int pick_form(int requested, int64_t two_row_groups, int nQ) {
   if (requested != kFormAuto) return requested;          // the caller's choice for this call
-  if (g_attn_form != kFormAuto) return g_attn_form;      // the process-wide default
   return (nQ >= kKeySplitMinQueryBlocks && two_row_groups <= (int64_t)kKeySplitMaxGroupsPerCu * compute_units()) ? kFormKeySplit : kFormTwoRows;
 }
 
@@ -1335,12 +1334,6 @@ bool strides_ok(const int64_t s[3]) {
 bool span_ok(int64_t seq_len, int64_t row_stride) { return ((seq_len - 1) * row_stride + kD) * 2 < ((int64_t)1 << 31); }
 
 }  // namespace
-
-extern "C" int stof_attn_set_launch_form(int form) {
-  if (form < kFormAuto || form > kFormPipelined) return STOF_ERR_UNSUPPORTED;
-  g_attn_form = form;
-  return STOF_OK;
-}
 
 extern "C" int stof_attn_plan_rows(int batch_size, int head_num, int seq_len, int launch_form) {
   if (batch_size <= 0 || head_num <= 0 || seq_len <= 0 || seq_len % kBM != 0) return STOF_ERR_BAD_SHAPE;

@@ -92,6 +92,8 @@ template <int ACT, int MT, bool BF = false>
 __device__ __forceinline__ void store_wave_block(const GemmParams& p, const floatx16 (&acc)[2][MT], lds_byte* stage,
                                                  int m_base, int n_base, int lane) {
   const int j32 = lane & 31, g = lane >> 5;
+  // the wave's block of C as a buffer: base = its first element, 32-bit byte offsets per lane (ldc < 2^23, host-checked)
+  const __amdgpu_buffer_rsrc_t c_rsrc = stof_wave_rsrc(p.C + (int64_t)m_base * p.ldc + n_base);
   half4_t bv[2][4];
 #pragma unroll
   for (int ni = 0; ni < 2; ++ni)
@@ -123,7 +125,7 @@ __device__ __forceinline__ void store_wave_block(const GemmParams& p, const floa
       // (written through the XCD's cache, so the tile is on its way to memory while the kernel runs and
       // not part of the end-of-kernel write-back the next launch waits for: a BERT-large layer of five
       // launches at 8192 tokens 282 -> 269 us, BERT-base 185 -> 184)
-      if (m < p.M && n < p.N) stof_store16_through(p.C + (int64_t)m * p.ldc + n, o);
+      if (m < p.M && n < p.N) stof_store16_through(c_rsrc, (uint32_t)(32 * mi + t) * (uint32_t)(p.ldc * 2) + 16 * c, o);
     }
   }
 }
@@ -673,7 +675,7 @@ __global__ __launch_bounds__(512) void gemm_bias_res_ln_kernel(const LnGemmParam
 //  * the words travel as relaxed device-scope atomic stores and loads: these are performed beyond
 //    the XCD's cache, so no cache write-back or invalidate is needed (a device-scope fence would
 //    write back the whole L2 of the XCD once per wave);
-//  * the wait is bounded: after a fixed number of polls (2^18; stof_gemm_bias_res_ln_cluster_set_spin_limit) the wave sets the error word of the
+//  * the wait is bounded: after a fixed number of polls (2^18, or the caller's limit) the wave sets the error word of the
 //    workspace and goes on (its output rows are then wrong, the launch still ends).  The cluster's
 //    workgroups are 8 apart in dispatch order - round-robin over the 8 XCDs puts them on one XCD,
 //    where they share the activation rows in L2.  The grid never exceeds two workgroups per
@@ -697,11 +699,16 @@ struct LnClusterParams {
 };
 
 constexpr int kClusterSpinLimit = 1 << 18;   // default number of polls before a wave gives up
-int g_cluster_spin_limit = kClusterSpinLimit;
 constexpr unsigned long long kStatsValid = 1ull << 63;
+// The waits of this kernel need every workgroup of the grid to be running: the grid is sized to
+// kClusterGroupsPerCu workgroups per compute unit, which the launch bounds (registers) and the
+// tile buffers (LDS) must allow; the host also asks the runtime what it allows (see the launch).
+constexpr int kClusterGroupsPerCu = 2;
+constexpr int kLdsPerCu = 160 * 1024;
+static_assert(kClusterGroupsPerCu * 4 * kGTile <= kLdsPerCu, "the cluster kernel's tile buffers must fit a compute unit kClusterGroupsPerCu times");
 
 template <int NT, bool BF = false>   // NT = N / 128 workgroups per row block
-__global__ __launch_bounds__(256) void gemm_bias_res_ln_cluster_kernel(const LnClusterParams p) {
+__global__ __launch_bounds__(256, kClusterGroupsPerCu) void gemm_bias_res_ln_cluster_kernel(const LnClusterParams p) {
   __shared__ __attribute__((aligned(1024))) unsigned char a_lds0[kGTile];
   __shared__ __attribute__((aligned(1024))) unsigned char a_lds1[kGTile];
   __shared__ __attribute__((aligned(1024))) unsigned char w_lds0[kGTile];
@@ -932,6 +939,7 @@ __global__ __launch_bounds__(256) void gemm_bias_res_ln_cluster_kernel(const LnC
 
   // ---- normalise and store: each 32 x 64 block through 4 KB of LDS of the wave's own, out as
   // full 128-byte lines (see store_wave_block)
+  const __amdgpu_buffer_rsrc_t c_rsrc = stof_wave_rsrc(p.C + (int64_t)(m0 + 64 * wm) * p.ldc + nb);
 #pragma unroll
   for (int mi = 0; mi < 2; ++mi) {
 #pragma unroll
@@ -951,7 +959,7 @@ __global__ __launch_bounds__(256) void gemm_bias_res_ln_cluster_kernel(const LnC
       const int t = 8 * ii + (lane >> 3), c = lane & 7;
       const half8_t o = *reinterpret_cast<const __attribute__((address_space(3))) half8_t*>(stage + t * 128 + ((c ^ (t & 7)) << 4));
       const int m = m0 + 64 * wm + 32 * mi + t;
-      if (m < p.M) stof_store16_through(p.C + (int64_t)m * p.ldc + nb + 8 * c, o);
+      if (m < p.M) stof_store16_through(c_rsrc, (uint32_t)(32 * mi + t) * (uint32_t)(p.ldc * 2) + 16 * c, o);
     }
   }
 
@@ -1029,7 +1037,7 @@ extern "C" int stof_gemm_bias_act_dt(const void* A, const void* Wt, const void* 
                                      int act, int dtype, void* stream) {
   if (!A || !Wt || !C) return STOF_ERR_NULL_POINTER;
   if (M <= 0 || N <= 0 || K <= 0 || K % kGK != 0 || N % 8 != 0 || lda < K || ldc < N) return STOF_ERR_BAD_SHAPE;
-  if (M > (1 << 30) || N > (1 << 30) || K > (1 << 30)) return STOF_ERR_BAD_SHAPE;
+  if (M > (1 << 30) || N > (1 << 30) || K > (1 << 30) || ldc >= (1 << 23)) return STOF_ERR_BAD_SHAPE;   // (ldc: 32-bit byte offsets inside a wave's block of C)
   if (dtype != STOF_DTYPE_F16 && dtype != STOF_DTYPE_BF16) return STOF_ERR_UNSUPPORTED;
   if (!stof_aligned16(A) || !stof_aligned16(Wt) || !stof_aligned16(C) || (bias && ((uintptr_t)bias & 7)) ||
       lda % 8 != 0 || ldc % 8 != 0)
@@ -1103,7 +1111,7 @@ extern "C" int stof_gemm_bias_act_splitk_dt(const void* A, const void* Wt, const
                                             int dtype, void* stream) {
   if (!A || !Wt || !C || !workspace) return STOF_ERR_NULL_POINTER;
   if (M <= 0 || N <= 0 || K <= 0 || K % kGK != 0 || N % 8 != 0 || lda < K || ldc < N) return STOF_ERR_BAD_SHAPE;
-  if (K > (1 << 30) || splits < 2 || splits > kSplitMaxSplits) return STOF_ERR_BAD_SHAPE;
+  if (K > (1 << 30) || ldc >= (1 << 23) || splits < 2 || splits > kSplitMaxSplits) return STOF_ERR_BAD_SHAPE;
   if (dtype != STOF_DTYPE_F16 && dtype != STOF_DTYPE_BF16) return STOF_ERR_UNSUPPORTED;
   const int64_t tiles64 = ((M + 63) / 64) * ((N + kWFeat - 1) / kWFeat);
   if (tiles64 > kSplitMaxTiles) return STOF_ERR_UNSUPPORTED;
@@ -1158,16 +1166,24 @@ extern "C" int stof_gemm_bias_res_ln(const void* A, const void* Wt, const void* 
 }
 
 namespace {
-constexpr int kClusterGroupsPerCu = 2;
-int cluster_compute_units() {
-  static int cus = 0;
-  if (cus == 0) {
-    int dev = 0, n = 0;
-    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
-      n = 256;
-    cus = n;
+// Workgroups of one instantiation of the cluster kernel that run at once on the current device:
+// what the runtime reports per compute unit (registers, LDS), capped at the kClusterGroupsPerCu the
+// kernel was written for, times the compute units.  Asked once per device and instantiation.
+constexpr int kMaxDevices = 64;
+template <int NT, bool BF>
+int64_t cluster_resident_groups() {
+  static int cached[kMaxDevices] = {};   // 0 = not asked yet, -1 = the query failed
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return 0;
+  if (cached[dev] == 0) {
+    int cus = 0, per_cu = 0;
+    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0 ||
+        hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, gemm_bias_res_ln_cluster_kernel<NT, BF>, 256, 0) != hipSuccess || per_cu <= 0)
+      cached[dev] = -1;
+    else
+      cached[dev] = (per_cu < kClusterGroupsPerCu ? per_cu : kClusterGroupsPerCu) * cus;
   }
-  return cus;
+  return cached[dev] < 0 ? 0 : cached[dev] / 8 * 8;
 }
 }  // namespace
 
@@ -1176,19 +1192,23 @@ extern "C" int64_t stof_gemm_bias_res_ln_cluster_workspace_bytes(int64_t M, int6
   return kClusterStatsOffset + ((M + kGT - 1) / kGT) * (2 * (N / kGT)) * kGT * 8;
 }
 
-extern "C" int stof_gemm_bias_res_ln_cluster_set_spin_limit(int polls) {
-  if (polls < 0) return STOF_ERR_BAD_SHAPE;
-  g_cluster_spin_limit = polls == 0 ? kClusterSpinLimit : polls;
-  return STOF_OK;
-}
-
 extern "C" int stof_gemm_bias_res_ln_cluster_dt(const void* A, const void* Wt, const void* bias, const void* residual,
                                                 const void* gamma, const void* beta, void* C,
                                                 int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldr, int64_t ldc,
                                                 float eps, void* workspace, int64_t workspace_bytes, int dtype, void* stream) {
+  return stof_gemm_bias_res_ln_cluster_bounded(A, Wt, bias, residual, gamma, beta, C, M, N, K, lda, ldr, ldc, eps,
+                                               workspace, workspace_bytes, dtype, 0, stream);
+}
+
+extern "C" int stof_gemm_bias_res_ln_cluster_bounded(const void* A, const void* Wt, const void* bias, const void* residual,
+                                                     const void* gamma, const void* beta, void* C,
+                                                     int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldr, int64_t ldc,
+                                                     float eps, void* workspace, int64_t workspace_bytes, int dtype,
+                                                     int spin_limit, void* stream) {
   if (!A || !Wt || !C || !workspace) return STOF_ERR_NULL_POINTER;
+  if (spin_limit < 0) return STOF_ERR_BAD_SHAPE;
   if (dtype != STOF_DTYPE_F16 && dtype != STOF_DTYPE_BF16) return STOF_ERR_UNSUPPORTED;
-  if (M <= 0 || K <= 0 || K % kGK != 0 || M > kClusterMaxRows || K > (1 << 30) || lda < K || ldc < N || (residual && ldr < N))
+  if (M <= 0 || K <= 0 || K % kGK != 0 || M > kClusterMaxRows || K > (1 << 30) || lda < K || ldc < N || ldc >= (1 << 23) || (residual && ldr < N))
     return STOF_ERR_BAD_SHAPE;
   if (N % kGT != 0 || N < 2 * kGT || N > 8 * kGT) return STOF_ERR_UNSUPPORTED;   // 256, 384, ..., 1024
   if (!stof_aligned16(A) || !stof_aligned16(Wt) || !stof_aligned16(C) || ((uintptr_t)bias & 7) ||
@@ -1204,23 +1224,23 @@ extern "C" int stof_gemm_bias_res_ln_cluster_dt(const void* A, const void* Wt, c
   p.departed = p.error + 4;
   p.stats = reinterpret_cast<unsigned long long*>(reinterpret_cast<char*>(workspace) + kClusterStatsOffset);
   p.M = (int)M; p.N = (int)N; p.K = (int)K; p.lda = (int)lda; p.ldr = (int)ldr; p.ldc = (int)ldc;
-  p.eps = eps; p.inv_n = 1.0f / (float)N; p.spin_limit = g_cluster_spin_limit;
+  p.eps = eps; p.inv_n = 1.0f / (float)N; p.spin_limit = spin_limit == 0 ? kClusterSpinLimit : spin_limit;
   const int64_t groups = (int64_t)((p.tiles_m + 7) / 8) * 8 * p.tiles_n;
   if (groups > (1 << 30)) return STOF_ERR_BAD_SHAPE;
   p.total_groups = (int)groups;
-  // Two workgroups fit a compute unit (64 KB of LDS each), so a grid of at most that many
-  // (a multiple of 8) is running as a whole from the start.
-  const int64_t resident = ((int64_t)kClusterGroupsPerCu * cluster_compute_units()) / 8 * 8;
-  if (resident < 8 * p.tiles_n) return STOF_ERR_UNSUPPORTED;   // a device too small to hold one cluster per XCD
-  const dim3 grid((unsigned)(groups < resident ? groups : resident)), block(256);
+  // A grid of at most the workgroups that run at once (a multiple of 8) is running as a whole
+  // from the start; fewer than one cluster per XCD, or a runtime that will not say: not this form.
   hipStream_t st = (hipStream_t)stream;
   const bool bf = dtype == STOF_DTYPE_BF16;
   switch (p.tiles_n) {
 #define STOF_CLUSTER_CASE(NT) \
-    case NT: \
+    case NT: { \
+      const int64_t resident = bf ? cluster_resident_groups<NT, true>() : cluster_resident_groups<NT, false>(); \
+      if (resident < 8 * p.tiles_n) return STOF_ERR_UNSUPPORTED; \
+      const dim3 grid((unsigned)(groups < resident ? groups : resident)), block(256); \
       if (bf) hipLaunchKernelGGL((gemm_bias_res_ln_cluster_kernel<NT, true>), grid, block, 0, st, p); \
       else hipLaunchKernelGGL((gemm_bias_res_ln_cluster_kernel<NT, false>), grid, block, 0, st, p); \
-      break;
+      break; }
     STOF_CLUSTER_CASE(2) STOF_CLUSTER_CASE(3) STOF_CLUSTER_CASE(4) STOF_CLUSTER_CASE(5)
     STOF_CLUSTER_CASE(6) STOF_CLUSTER_CASE(7) STOF_CLUSTER_CASE(8)
 #undef STOF_CLUSTER_CASE

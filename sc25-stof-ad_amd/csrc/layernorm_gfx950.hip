@@ -77,6 +77,7 @@ __global__ __launch_bounds__(256) void bias_res_ln_kernel(const LnParams p) {
     if (p.rstd) p.rstd[row] = rstd;
   }
   half_t* yr = p.y + row * p.N;
+  const __amdgpu_buffer_rsrc_t y_rsrc = stof_wave_rsrc(yr);   // this wave's row
 #pragma unroll
   for (int c = 0; c < CH; ++c) {
     const int ch = lane + 64 * c;
@@ -92,7 +93,7 @@ __global__ __launch_bounds__(256) void bias_res_ln_kernel(const LnParams p) {
         if (p.beta) t += bt[i];
         o[i] = to_elem<BF>(t);
       }
-      stof_store16_through(yr + 8 * ch, o);
+      stof_store16_through(y_rsrc, 16 * ch, o);
     }
   }
 }

@@ -80,10 +80,21 @@ template <int ACT> __device__ __forceinline__ float activate(float x) {
   return x;
 }
 
-// 16-byte store written through the XCD's L2 at device scope (sc1): for output rows nobody in
-// this launch reads again.
-__device__ __forceinline__ void stof_store16_through(half_t* dst, half8_t v) {
-  asm volatile("global_store_dwordx4 %0, %1, off sc1" :: "v"(dst), "v"(v) : "memory");
+// Output rows written THROUGH the XCD's L2 at device scope (sc1): for tiles nobody in the launch
+// reads again.  As plain cached stores they sit in L2 until the end-of-kernel write-back, which
+// the next launch waits for.  The store is a raw buffer store (cache policy as an argument of
+// the builtin), addressed as a wave-uniform base plus a 32-bit byte offset per lane.  (Written
+// as inline assembly it loses the compiler's hazard handling: a 16-byte store whose data
+// registers are overwritten within two instructions stores the new values for some lanes.)
+typedef unsigned int uintx4_t __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t stof_wave_rsrc(const void* wave_uniform_base) {
+  const uint64_t a = reinterpret_cast<uint64_t>(wave_uniform_base);
+  const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)a), hi = __builtin_amdgcn_readfirstlane((uint32_t)(a >> 32));
+  return __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<void*>(((uint64_t)hi << 32) | lo), 0, 0x7fffffff, 0x00020000);
+}
+constexpr int kStoreThrough = 16;   // cache-policy bits of the buffer builtins on gfx940+: 1 = sc0, 2 = nt, 16 = sc1
+__device__ __forceinline__ void stof_store16_through(__amdgpu_buffer_rsrc_t rsrc, uint32_t byte_offset, half8_t v) {
+  __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(uintx4_t, v), rsrc, (int)byte_offset, 0, kStoreThrough);
 }
 
 static inline int stof_check_launch() {

@@ -1,4 +1,12 @@
-"""ctypes binding of libstof_hip.so (C ABI declared in include/stof_abi.h).
+"""Binding of libstof_hip.so (C ABI declared in include/stof_abi.h).
+
+Two bindings of the same functions, same names, same positional arguments:
+  * the extension module ``_stof_ext`` (pybind11, built by csrc/build.py next to the library;
+    the counterpart of the reference's pybind11 modules, src/ops/src/block_attn_mask.cpp:52-56):
+    pointers and the stream are ints, None is NULL, a stride triple is a tuple of three ints;
+  * ctypes on the library itself, used when the extension module is absent (no pybind11 at
+    build time) or when ``STOF_BINDING=ctypes`` is set.
+``lib()`` returns whichever is in use; ``i64x3`` builds a stride triple for it.
 
 The library is loaded from this directory.  It is never built implicitly on a machine
 with a GPU: a missing library is an error there, so a silent fallback cannot hide it.
@@ -29,7 +37,6 @@ _SIGNATURES = {
     "stof_attn_plan_rows": (c_int, [c_int, c_int, c_int, c_int]),
     "stof_attn_plan_bytes": (c_int64, [c_int, c_int, c_int]),
     "stof_attn_plan_build": (c_int, [_P, _P, _P, _P, c_int, c_int64, c_int, c_int, _P, c_int64, _P]),
-    "stof_attn_set_launch_form": (c_int, [c_int]),
     "stof_pack_mask_bits": (c_int, [_P, _P, c_int64, c_int64, c_int64, c_int, _P]),
     "stof_rowwise_attn_fwd": (c_int, [_P, _P, _P, _P, c_int, c_int, c_int, _P,
                                       c_int, c_int, c_int, c_int, c_int, c_int, _P]),
@@ -57,7 +64,8 @@ _SIGNATURES = {
     "stof_gemm_bias_res_ln_cluster_dt": (c_int, [_P, _P, _P, _P, _P, _P, _P, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64,
                                                  c_float, _P, c_int64, c_int, _P]),
     "stof_gemm_bias_res_ln_cluster_workspace_bytes": (c_int64, [c_int64, c_int64]),
-    "stof_gemm_bias_res_ln_cluster_set_spin_limit": (c_int, [c_int]),
+    "stof_gemm_bias_res_ln_cluster_bounded": (c_int, [_P, _P, _P, _P, _P, _P, _P, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64,
+                                                      c_float, _P, c_int64, c_int, c_int, _P]),
     "stof_gemm_bias_res_ln_cluster": (c_int, [_P, _P, _P, _P, _P, _P, _P, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64,
                                               c_float, _P, c_int64, _P]),
 }
@@ -67,21 +75,65 @@ class StofError(RuntimeError):
     """A C-ABI call returned a negative status."""
 
 
-def lib():
-    """Load (once) and return the ctypes handle; raise if the library is absent."""
-    global _lib
+_ext_used = False
+
+
+def _load_ctypes():
+    h = ctypes.CDLL(LIB_PATH)
+    for name, (res, args) in _SIGNATURES.items():
+        fn = getattr(h, name)
+        fn.restype = res
+        fn.argtypes = args
+    return h
+
+
+def _load_ext():
+    """The extension module, or None if it is not built or is older than the library."""
+    import importlib.util
+    import sysconfig
+    path = os.path.join(os.path.dirname(LIB_PATH), "_stof_ext" + (sysconfig.get_config_var("EXT_SUFFIX") or ".so"))
+    if not os.path.exists(path) or os.path.getmtime(path) + 1 < os.path.getmtime(LIB_PATH):
+        return None
+    # the module is linked against libstof_hip.so with an $ORIGIN run path; loading the library
+    # first (globally) makes the process use the one at LIB_PATH whatever the loader would find
+    ctypes.CDLL(LIB_PATH, mode=ctypes.RTLD_GLOBAL)
+    spec = importlib.util.spec_from_file_location("_stof_ext", path)
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    if any(not hasattr(mod, name) for name in _SIGNATURES):
+        return None
+    return mod
+
+
+def lib(binding=None):
+    """Load (once) and return the binding in use; raise if the library is absent.
+    ``binding="ctypes"`` / ``"ext"`` returns that binding without changing the one in use."""
+    global _lib, _ext_used
+    if not os.path.exists(LIB_PATH):
+        raise StofError(
+            f"{LIB_PATH} is missing: build it with `python sc25-stof-ad_amd/csrc/build.py` "
+            "(hipcc, gfx950). There is no fallback path.")
+    if binding == "ctypes":
+        return _load_ctypes()
+    if binding == "ext":
+        return _load_ext()
     if _lib is None:
-        if not os.path.exists(LIB_PATH):
-            raise StofError(
-                f"{LIB_PATH} is missing: build it with `python sc25-stof-ad_amd/csrc/build.py` "
-                "(hipcc, gfx950). There is no fallback path.")
-        h = ctypes.CDLL(LIB_PATH)
-        for name, (res, args) in _SIGNATURES.items():
-            fn = getattr(h, name)
-            fn.restype = res
-            fn.argtypes = args
-        _lib = h
+        ext = None if os.environ.get("STOF_BINDING", "") == "ctypes" else _load_ext()
+        _ext_used = ext is not None
+        _lib = ext if ext is not None else _load_ctypes()
     return _lib
+
+
+def binding_name():
+    """"ext" (pybind11 module) or "ctypes": which binding ``lib()`` hands out."""
+    lib()
+    return "ext" if _ext_used else "ctypes"
+
+
+def i64x3(a, b, c):
+    """An int64[3] argument (the stride triples of the attention entry points) for the binding in use."""
+    lib()
+    return (a, b, c) if _ext_used else _I64x3(a, b, c)
 
 
 def check(status, what):
@@ -92,4 +144,4 @@ def check(status, what):
 
 def strides3(t):
     """(batch, head, seq) element strides of a [B,H,S,D] view as an int64[3]."""
-    return _I64x3(t.stride(0), t.stride(1), t.stride(2))
+    return i64x3(t.stride(0), t.stride(1), t.stride(2))

@@ -194,9 +194,25 @@ def _cluster_workspace(dev, stream, nbytes):
     return ws
 
 
+def check_cluster_exchange(dev=None):
+    """Raise ``StofError`` if a bounded wait inside any cluster-form LayerNorm GEMM launched on
+    ``dev`` since the last check ran out (the rows that launch wrote are then invalid), and put
+    the error word back to zero.  The word stays set until it is cleared, so ONE check after a
+    batch of work covers every launch of that batch.  Synchronises the device: call it where the
+    caller synchronises anyway (``EncoderLayer`` / ``EncoderStack`` / ``CapturedForward`` do so
+    with ``check=True``).  The waits only run out when something else keeps compute units
+    occupied for about a tenth of a second while the kernel runs - another stream's or another
+    process's long kernel; on a device of one's own they cannot."""
+    if cluster_exchange_failed(dev):
+        clear_cluster_exchange_error(dev)
+        raise StofError("a LayerNorm GEMM in its cluster form gave up waiting for a partner workgroup (the device was "
+                        "shared with a long-running kernel?): the outputs since the last check are invalid. Use "
+                        "ln_fusion='split' / form='split' where the device is shared.")
+
+
 def cluster_exchange_failed(dev=None):
     """True if a wait inside any cluster-form launch on ``dev`` ran out (its output is then
-    invalid): the first word of the workspace.  Synchronises the device; for tests and debugging."""
+    invalid): the first word of the workspace.  Synchronises the device."""
     dev = torch.device("cuda", torch.cuda.current_device()) if dev is None else torch.device(dev)
     torch.cuda.synchronize(dev)
     return any(bool(ws[:4].view(torch.int32).item()) for (d, _), ws in _cluster_ws.items() if d == dev.index)
@@ -243,8 +259,14 @@ def ln_gemm_form(M, N, K):
     return "split" if K % 64 == 0 else "row"
 
 
-def gemm_bias_residual_layernorm(x, Wt, bias, residual, gamma, beta, eps=1e-5, out=None, form="auto"):
+def gemm_bias_residual_layernorm(x, Wt, bias, residual, gamma, beta, eps=1e-5, out=None, form="auto", spin_limit=0):
     """LN(x @ Wt^T + bias + residual) * gamma + beta.
+
+    The cluster form (what ``"auto"`` takes from 192 output tiles of 128 x 128 on) assumes a
+    device that is not shared with long-running kernels of other streams or processes: its
+    workgroups wait for one another, boundedly; a wait that runs out leaves invalid rows and
+    sets an error word that ``check_cluster_exchange`` reads.  ``spin_limit`` (polls, 0 = the
+    library's 2^18) is for tests of that path.
 
     ``form="row"``: one workgroup owns the whole row of N features (stof_gemm_bias_res_ln).
     ``form="cluster"``: the N / 128 workgroups of a block of 128 token rows each own 128 features
@@ -273,15 +295,17 @@ def gemm_bias_residual_layernorm(x, Wt, bias, residual, gamma, beta, eps=1e-5, o
     if out is None:
         out = torch.empty(x.shape[:-1] + (N,), dtype=x.dtype, device=x.device)
     _require(out.dtype == x.dtype, "out must have x's element format")
+    _require(out.device == x.device and tuple(out.shape) == tuple(x.shape[:-1]) + (N,) and out.is_contiguous(),
+             f"out must be a contiguous {tuple(x.shape[:-1]) + (N,)} tensor on x's device")
     lib = _lib.lib()
     st = _stream(out)
     if form == "cluster":
         _require(cluster_supported(N, K), f"unsupported shape for the cluster form: N {N}, K {K}")
         nbytes = lib.stof_gemm_bias_res_ln_cluster_workspace_bytes(M, N)
         ws = _cluster_workspace(x.device, st, nbytes)
-        check(lib.stof_gemm_bias_res_ln_cluster_dt(x.data_ptr(), Wt.data_ptr(), _p(bias), _p(residual), _p(gamma), _p(beta),
-                                                   out.data_ptr(), M, N, K, K, N, N, float(eps),
-                                                   ws.data_ptr(), ws.numel(), dt, st),
+        check(lib.stof_gemm_bias_res_ln_cluster_bounded(x.data_ptr(), Wt.data_ptr(), _p(bias), _p(residual), _p(gamma), _p(beta),
+                                                        out.data_ptr(), M, N, K, K, N, N, float(eps),
+                                                        ws.data_ptr(), ws.numel(), dt, int(spin_limit), st),
               "stof_gemm_bias_res_ln_cluster")
         return out
     check(lib.stof_gemm_bias_res_ln(x.data_ptr(), Wt.data_ptr(), _p(bias), _p(residual),

@@ -59,9 +59,12 @@ class EncoderLayer:
         return fused.ln_gemm_form(M, self.hidden, K)
 
     def pre_ln_stored(self, M):
-        """True if the products that feed the two LayerNorms are stored as fp16 tensors for M token
-        rows (the split form), False if they stay in registers (fused and cluster forms)."""
-        return self._ln_form(M, self.hidden) == "split"
+        """For M token rows, whether the product that feeds a LayerNorm is stored as a 16-bit tensor
+        first (the split form) or stays in registers (fused and cluster forms): one flag for the
+        attention-output GEMM (K = hidden) and one for the FFN-output GEMM (K = ffn) - the two can
+        take different forms (4096 rows at hidden 768: cluster for K 768, split-K GEMM + LayerNorm
+        kernel for K 3072)."""
+        return (self._ln_form(M, self.hidden) == "split", self._ln_form(M, self.W1.shape[0]) == "split")
 
     def _gemm_ln(self, x, Wt, bias, residual, gamma, beta):
         form = self._ln_form(x.numel() // x.shape[-1], x.shape[-1])
@@ -82,7 +85,10 @@ class EncoderLayer:
         f = fused.gemm_bias_act(h, self.W1, self.b1, self.act)
         return self._gemm_ln(f, self.W2, self.b2, h, self.g2, self.be2)
 
-    def forward(self, x, lut, block=64):
+    def forward(self, x, lut, block=64, check=False):
+        """``check=True`` synchronises the device after the layer and raises if a cluster-form
+        LayerNorm GEMM (this layer's or an earlier one on the device) gave up a wait - see
+        ``fused.check_cluster_exchange``; for callers that share the device with other work."""
         B, S, D = x.shape
         H = self.n_heads
         hd = D // H
@@ -90,7 +96,10 @@ class EncoderLayer:
         q, k, v = (qkv[..., t * D:(t + 1) * D].view(B, S, H, hd).permute(0, 2, 1, 3) for t in range(3))
         attn = block_attn(q, k, v, lut, block, block, out_layout="bshd")      # [B,S,D]
         h = self._gemm_ln(attn, self.Wo, self.bo, x, self.g1, self.be1)
-        return self._ffn(h)
+        y = self._ffn(h)
+        if check:
+            fused.check_cluster_exchange(x.device)
+        return y
 
     __call__ = forward
 
@@ -122,9 +131,12 @@ class EncoderStack:
     def __init__(self, layer_weights, n_heads, eps=1e-12, gelu="erf", ln_fusion="auto", ffn_chain="auto"):
         self.layers = [EncoderLayer(w, n_heads, eps, gelu, ln_fusion, ffn_chain) for w in layer_weights]
 
-    def forward(self, x, lut, block=64):
+    def forward(self, x, lut, block=64, check=False):
+        """``check=True``: one ``fused.check_cluster_exchange`` after the last layer (it covers all)."""
         for layer in self.layers:
             x = layer(x, lut, block)
+        if check:
+            fused.check_cluster_exchange(x.device)
         return x
 
     __call__ = forward
@@ -154,9 +166,13 @@ class CapturedForward:
         with torch.cuda.graph(self.graph):
             self.y = module(self.x, lut, block)
 
-    def __call__(self, x):
+    def __call__(self, x, check=False):
+        """``check=True``: synchronise after the replay and raise if a cluster-form LayerNorm GEMM
+        gave up a wait (``fused.check_cluster_exchange``)."""
         self.x.copy_(x)
         self.graph.replay()
+        if check:
+            fused.check_cluster_exchange(self.x.device)
         return self.y
 
 

@@ -50,20 +50,26 @@ _LAUNCH_FORMS = {None: -1, "default": -1, "auto": -1, "two_rows": 0, "key_split"
 def _form(launch_form):
     _require(launch_form in _LAUNCH_FORMS,
              f"launch form must be one of 'default', 'two_rows', 'key_split', 'pipelined', got {launch_form!r}")
-    return _LAUNCH_FORMS[launch_form]
+    f = _LAUNCH_FORMS[launch_form]
+    return _default_form if f < 0 and launch_form != "auto" else f
+
+
+_default_form = -1
 
 
 def set_attention_launch_form(form="auto"):
-    """Process-wide DEFAULT launch form of the attention kernels, used by calls that do not
-    name one: ``"auto"`` (by grid size), ``"two_rows"`` (two query blocks per workgroup, for
-    large grids) or ``"key_split"`` (one query block per workgroup with the keys of each tile
-    split over two wavefront pairs, for small grids).  The reference selects its kernel per
-    call with ``num_warps`` (src/ops/src/block_attn_mask_cuda.cu:6064-6322); the per-call
-    counterpart here is the ``launch_form`` argument of ``block_attn`` and of the row-wise
-    operators' functional form.  Results agree within rounding in every form."""
+    """DEFAULT launch form of the attention operators of this module, used by calls that do not
+    name one: ``"auto"`` (the library chooses by grid size), ``"two_rows"`` (two query blocks per
+    workgroup, for large grids), ``"key_split"`` (one query block per workgroup with the keys of
+    each tile split over two wavefront pairs, for small grids) or ``"pipelined"``.  The reference
+    selects its kernel per call with ``num_warps`` (src/ops/src/block_attn_mask_cuda.cu:6064-6322);
+    the per-call counterpart here is the ``launch_form`` argument of ``block_attn`` and of the
+    row-wise operators' functional form.  The default lives in this Python module (the library
+    keeps no state: every C-ABI call names its form).  Results agree within rounding in every form."""
+    global _default_form
     _require(form in ("auto", "two_rows", "key_split", "pipelined"),
              f"launch form must be 'auto', 'two_rows', 'key_split' or 'pipelined', got {form!r}")
-    check(_lib.lib().stof_attn_set_launch_form(_LAUNCH_FORMS[form]), "stof_attn_set_launch_form")
+    _default_form = _LAUNCH_FORMS[form]
 
 
 def pack_mask_bits(src, additive):
@@ -251,8 +257,8 @@ def block_attn(q, k, v, lut, block_m=64, block_n=64, out=None, out_layout="bhsd"
     per sample).  Returns ``out``: ``[B,H,S,D]`` (``out_layout='bhsd'``) or ``[B,S,H*D]``
     (``'bshd'``); ``out`` may be ``q`` itself.
 
-    ``launch_form``: ``None`` / ``"default"`` (the process default, automatic by grid size
-    unless ``set_attention_launch_form`` changed it), ``"two_rows"`` or ``"key_split"`` - the
+    ``launch_form``: ``None`` / ``"default"`` (this module's default, automatic by grid size
+    unless ``set_attention_launch_form`` changed it), ``"auto"``, ``"two_rows"`` or ``"key_split"`` - the
     per-call counterpart of the reference's ``num_warps``.  ``use_plan=False`` makes the kernel
     read the LUT itself instead of the walk laid out once per LUT (same result bit for bit; the
     plan saves the dependent LUT reads at the start of every workgroup).  ``revalidate=True`` discards what
@@ -282,7 +288,7 @@ def block_attn(q, k, v, lut, block_m=64, block_n=64, out=None, out_layout="bhsd"
         ostr = strides3(out)
     elif out_layout == "bshd":
         _require(out.shape == (B, S, H * D) and out.stride(2) == 1, "out must be [B,S,H*D] with contiguous last dim")
-        ostr = (_lib.c_int64 * 3)(out.stride(0), D, out.stride(1))
+        ostr = _lib.i64x3(out.stride(0), D, out.stride(1))
     else:
         raise StofError(f"unknown out_layout {out_layout!r}")
     _require(out.dtype == q.dtype and out.device == dev, "out must have q's dtype and device")

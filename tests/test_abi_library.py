@@ -19,11 +19,21 @@ def _declared_symbols():
     return sorted(set(re.findall(r"\b(stof_[a-z0-9_]+)\s*\(", text)))
 
 
-@pytest.fixture(scope="module")
-def lib():
+@pytest.fixture(scope="module", params=["ctypes", "ext"])
+def lib(request):
+    """Every test of this module runs against both bindings of the C ABI: ctypes on the library
+    itself and the pybind11 extension module built beside it."""
+    global _BINDING
     if not os.path.exists(_lib.LIB_PATH):
         pytest.skip("libstof_hip.so not built (python sc25-stof-ad_amd/csrc/build.py)")
-    return _lib.lib()
+    h = _lib.lib(request.param)
+    if h is None:
+        pytest.skip("extension module _stof_ext not built (python sc25-stof-ad_amd/csrc/build.py; needs pybind11)")
+    _BINDING = request.param
+    return h
+
+
+_BINDING = "ctypes"
 
 
 def test_every_declared_symbol_is_exported_and_bound(lib):
@@ -33,7 +43,16 @@ def test_every_declared_symbol_is_exported_and_bound(lib):
     for s in syms:
         assert hasattr(raw, s), f"{s} declared in stof_abi.h but not exported"
         assert s in _lib._SIGNATURES, f"{s} has no ctypes signature"
+        assert hasattr(lib, s), f"{s} missing from the {_BINDING} binding"
     assert sorted(_lib._SIGNATURES) == syms
+
+
+def test_the_binding_in_use_is_the_extension_module_when_it_is_built():
+    if _lib.lib("ext") is None:
+        pytest.skip("extension module not built")
+    if os.environ.get("STOF_BINDING", "") == "ctypes":
+        pytest.skip("ctypes forced by the environment")
+    assert _lib.binding_name() == "ext"
 
 
 def test_version_and_status_strings(lib):
@@ -43,7 +62,7 @@ def test_version_and_status_strings(lib):
 
 
 def _s3(a, b, c):
-    return (ctypes.c_int64 * 3)(a, b, c)
+    return (a, b, c) if _BINDING == "ext" else (ctypes.c_int64 * 3)(a, b, c)
 
 
 def test_block_attn_argument_checks(lib):
@@ -87,8 +106,6 @@ def test_attention_plan_argument_checks(lib):
 
 def test_other_entry_points_argument_checks(lib):
     P = 4096
-    assert lib.stof_attn_set_launch_form(7) == -3
-    assert lib.stof_attn_set_launch_form(-1) == 0
     assert lib.stof_pack_mask_bits(None, P, 64, 64, 64, 1, None) == -1
     assert lib.stof_pack_mask_bits(P, P, 64, 100, 100, 1, None) == -2
     assert lib.stof_bias_res_ln(P, None, None, None, None, P, None, None, 10, 12, 1e-5, None) == -2   # N % 8

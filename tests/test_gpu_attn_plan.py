@@ -144,7 +144,7 @@ def test_planned_entry_point_through_the_c_abi():
     frp, fci, prp, pci, pbm, lrp, lci = lut
     from stof.ops import pack_mask_bits
     bits = pack_mask_bits(pbm, additive=True)
-    st = (ctypes.c_int64 * 3)(H * S * 64, S * 64, 64)
+    st = _lib.i64x3(H * S * 64, S * 64, 64)
     rows = lib.stof_attn_plan_rows(B, H, S, 0)
     assert rows == 2 and lib.stof_attn_plan_rows(B, H, S, 1) == 1 and lib.stof_attn_plan_rows(B, H, S, 2) == 0
     plans = {r: _build_plan(lut, S, r) for r in (1, 2)}

@@ -238,10 +238,26 @@ def test_encoder_layer_c3(fusion, B):
     lut = pm.get_sparse_storage_batched(mask.float().cuda(), 64, 64)[1:]
     layer = EncoderLayer({k: v.cuda() for k, v in w.items()}, H, eps=1e-12, ln_fusion=fusion)
     got = layer(x.cuda(), lut)
-    want16 = oe.bert_layer(x, w, mask.float(), H, eps=1e-12, round_fp16="split" if layer.pre_ln_stored(B * S) else True)
+    want16 = oe.bert_layer(x, w, mask.float(), H, eps=1e-12, round_fp16=layer.pre_ln_stored(B * S))
     want32 = oe.bert_layer(x, w, mask.float(), H, eps=1e-12)
     valid = torch.arange(S)[None, :] < L[:, None]          # rows past the sample length are don't-care
     _layer_checks(got, want16, want32, f"C3 layer B{B} {fusion}", 5e-3, valid)   # observed 2.9e-3 (B4), 3.3e-3 (B16)
+
+
+def test_encoder_layer_mixed_layernorm_forms():
+    """4096 tokens at hidden 768: "auto" runs the attention-output LayerNorm GEMM (K 768) in its
+    cluster form and the FFN-output one (K 3072) as split-K GEMM + LayerNorm kernel; the oracle
+    rounds the pre-LayerNorm product only where the kernels store it."""
+    B, S, D, H, F = 8, 512, 768, 12, 3072
+    w = configs.layer_weights(D, F, seed=3)
+    x = configs.layer_input(configs.LayerConfig("t", B, S, D, H, F, 1), seed=4)
+    mask = configs.mask_c1(S)[None].expand(B, -1, -1)
+    lut = pm.get_sparse_storage(mask[:1].float().cuda(), 64, 64)[1:]
+    layer = EncoderLayer({k: v.cuda() for k, v in w.items()}, H, eps=1e-12)
+    assert layer.pre_ln_stored(B * S) == (False, True)
+    got = layer(x.cuda(), lut, check=True)
+    _layer_checks(got, oe.bert_layer(x, w, mask.float(), H, eps=1e-12, round_fp16=layer.pre_ln_stored(B * S)),
+                  oe.bert_layer(x, w, mask.float(), H, eps=1e-12), "layer with mixed LayerNorm forms", 5e-3)
 
 
 @pytest.mark.parametrize("act", ["tanh", "relu"])
@@ -254,7 +270,7 @@ def test_encoder_layer_gpt_and_t5_activations(act):
     lut = pm.get_sparse_storage(mask[:1].float().cuda(), 64, 64)[1:]
     layer = EncoderLayer({k: v.cuda() for k, v in w.items()}, H, eps=1e-12, gelu=act)
     got = layer(x.cuda(), lut)
-    mode = "split" if layer.pre_ln_stored(B * S) else True
+    mode = layer.pre_ln_stored(B * S)
     _layer_checks(got, oe.bert_layer(x, w, mask.float(), H, eps=1e-12, gelu=act, round_fp16=mode),
                   oe.bert_layer(x, w, mask.float(), H, eps=1e-12, gelu=act), f"layer {act}", 5e-3)   # observed 3.5e-3
     with pytest.raises(ValueError):
@@ -269,7 +285,7 @@ def test_encoder_stack_two_layers_c5_shape_reduced():
     lut = pm.get_sparse_storage(mask.float().cuda(), 64, 64)[1:]
     stack = EncoderStack([{k: v.cuda() for k, v in w.items()} for w in ws], H, eps=1e-12)
     got = stack(x.cuda(), lut)
-    mode = "split" if stack.layers[0].pre_ln_stored(B * S) else True
+    mode = stack.layers[0].pre_ln_stored(B * S)
     want16 = want32 = x
     for w in ws:
         want16 = oe.bert_layer(want16, w, mask.float(), H, eps=1e-12, round_fp16=mode)
@@ -298,7 +314,7 @@ def test_encoder_stack_c5_full_size():
         y = layer(x, lut)
         if i in checked:
             print(f"C5 layer {i + 1}", flush=True)
-            mode = "split" if layer.pre_ln_stored(cfg.batch * cfg.seq) else True
+            mode = layer.pre_ln_stored(cfg.batch * cfg.seq)
             xin = x.cpu()
             want16 = oe.bert_layer(xin, w, mask.float()[None], cfg.heads, eps=cfg.eps, round_fp16=mode)
             want32 = oe.bert_layer(xin, w, mask.float()[None], cfg.heads, eps=cfg.eps)
@@ -326,7 +342,7 @@ def test_captured_stack_replays_match_eager_launches():
         got = run(x).clone()
         torch.cuda.synchronize()
         assert torch.equal(got, want), f"replay {i} differs from the eager result"
-    mode = "split" if stack.layers[0].pre_ln_stored(B * S) else True
+    mode = stack.layers[0].pre_ln_stored(B * S)
     want0 = xs[0].cpu()
     for w in ws:
         want0 = oe.bert_layer(want0, w, mask.float(), H, eps=1e-12, round_fp16=mode)

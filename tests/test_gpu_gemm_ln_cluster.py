@@ -112,24 +112,38 @@ def test_gemm_ln_cluster_bounded_wait_gives_up_and_recovers():
     """The wait for the partners is bounded: with a limit of one poll some waves of a launch give up
     (the kernel still ends normally, the error word is set, the output is not to be used); with the
     default limit restored and the word cleared the same workspace serves the next call."""
-    from stof import _lib
     M, N, K = 8192, 768, 768
     x = _rand(M, K, seed=40); W = _rand(K, N, seed=41, scale=0.05); b = _rand(N, seed=42, scale=0.5)
     r = _rand(M, N, seed=43); gm = (1 + 0.1 * _rand(N, seed=44).float()).half(); bt = _rand(N, seed=45, scale=0.1)
     args = (x.cuda(), fused.pack_weight(W.cuda()), b.cuda(), r.cuda(), gm.cuda(), bt.cuda(), 1e-5)
     want = oe.gemm_bias_residual_layernorm(x, W, b, r, gm, bt, 1e-5)
     _close(fused.gemm_bias_residual_layernorm(*args, form="cluster"), want, "before")
-    lib = _lib.lib()
-    try:
-        assert lib.stof_gemm_bias_res_ln_cluster_set_spin_limit(1) == 0
-        for _ in range(5):                       # (a single launch in which every wave finds its partners at once is conceivable)
-            fused.gemm_bias_residual_layernorm(*args, form="cluster")
-        torch.cuda.synchronize()                 # the launches end although waves gave up
-        assert fused.cluster_exchange_failed()
-    finally:
-        assert lib.stof_gemm_bias_res_ln_cluster_set_spin_limit(0) == 0
-    fused.clear_cluster_exchange_error()
-    assert not fused.cluster_exchange_failed()
+    for _ in range(5):                           # (a single launch in which every wave finds its partners at once is conceivable)
+        fused.gemm_bias_residual_layernorm(*args, form="cluster", spin_limit=1)
+    torch.cuda.synchronize()                     # the launches end although waves gave up
+    assert fused.cluster_exchange_failed()
+    with pytest.raises(fused.StofError):         # what the layer / stack / bench call where they synchronise
+        fused.check_cluster_exchange()
+    assert not fused.cluster_exchange_failed()   # (the check cleared the word)
     _close(fused.gemm_bias_residual_layernorm(*args, form="cluster"), want, "after")
-    assert not fused.cluster_exchange_failed()
-    assert lib.stof_gemm_bias_res_ln_cluster_set_spin_limit(-1) == -2
+    fused.check_cluster_exchange()
+    with pytest.raises(fused.StofError):
+        fused.gemm_bias_residual_layernorm(*args, form="cluster", spin_limit=-1)
+
+
+def test_layer_check_flag_raises_after_a_failed_exchange():
+    """EncoderLayer(check=True) surfaces a failed exchange of any earlier cluster launch on the device."""
+    from stof import configs, masks as pm
+    from stof.layer import EncoderLayer
+    B, S, D, H, F = 8, 512, 768, 12, 3072
+    w = {k: v.cuda() for k, v in configs.layer_weights(D, F, seed=0).items()}
+    x = configs.layer_input(configs.LayerConfig("t", B, S, D, H, F, 1), seed=1, device="cuda")
+    lut = pm.get_sparse_storage(configs.mask_c1(S).float()[None].cuda(), 64, 64)[1:]
+    layer = EncoderLayer(w, H, eps=1e-12, ln_fusion="cluster")
+    layer(x, lut, check=True)                    # a clean run passes
+    xa = _rand(4096, 768, seed=1).cuda(); Wt = fused.pack_weight(_rand(768, 768, seed=2, scale=0.05).cuda())
+    for _ in range(5):
+        fused.gemm_bias_residual_layernorm(xa, Wt, None, None, None, None, form="cluster", spin_limit=1)
+    with pytest.raises(fused.StofError):
+        layer(x, lut, check=True)
+    layer(x, lut, check=True)
