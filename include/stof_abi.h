@@ -27,6 +27,7 @@
  *                                                           rowwise_attn_sliding.cpp:8-12, rowwise_attn_mask.cpp:8-12
  *   stof_build_lut,
  *   stof_lut_additive_blocks   get_sparse_storage            src/util/masks.py:125-184 (the host loop :145-170)
+ *   stof_retile_lut            the launcher's kernel selection by (BLOCK_M, BLOCK_N), block_attn_mask_cuda.cu:6064-6322
  *   stof_bias_res_ln           batched_bias_layer_norm_fused_kernel
  *                                                           src/triton_template/add_layernorm.py:19-107
  *   stof_gemm_bias_act         the first product + bias + GELU of triton_matmul_batch_kernel
@@ -48,7 +49,7 @@
 extern "C" {
 #endif
 
-#define STOF_ABI_VERSION 4   /* 4: attention plan entry points and the cluster form with a wait limit added, the two process-wide setters (attention launch form, cluster spin limit) removed - both are per-call arguments, the library keeps no mutable state; 3: split-K and element-format entry points (nothing removed or changed) */
+#define STOF_ABI_VERSION 4   /* 4: attention plan entry points, stof_retile_lut and the cluster form with a wait limit added, the two process-wide setters (attention launch form, cluster spin limit) removed - both are per-call arguments, the library keeps no mutable state; 3: split-K and element-format entry points (nothing removed or changed) */
 
 enum {
   STOF_OK = 0,
@@ -221,6 +222,28 @@ int stof_build_lut(const void* mask, int elem_bytes, int64_t ld, int seq_len, in
                    uint64_t* part_bitmask, int32_t* counts,
                    int64_t cap_full, int64_t cap_part, int64_t cap_load,
                    void* workspace, int64_t workspace_bytes, void* stream);
+
+/*
+ * A LUT built with block_m x block_n blocks (each in {16, 32, 64, 128}) described again with the
+ * 64 x 64 blocks stof_block_attn_fwd takes: what the reference's launcher does by selecting a kernel
+ * per (BLOCK_M, BLOCK_N) (src/ops/src/block_attn_mask_cuda.cu:6064-6322) is done here by re-tiling
+ * the LUT once.  Input: the FULL and PART lists of the source LUT (row pointers of seq_len/block_m + 1
+ * entries - for one sample of a per-sample LUT, pass that sample's row pointers; their values may be
+ * absolute offsets into concatenated lists) and its additive fp16 blocks part_block_mask
+ * [n_part][block_m][block_n] (0 = allowed, -10000 = masked; may be NULL when there is no partial
+ * block).  Output, workspace and counts as for stof_build_lut at 64 x 64 (part_bitmask required):
+ * the lists are exactly those of get_sparse_storage(mask, 64, 64) on the mask the source LUT
+ * encodes.  Two launches, no synchronisation; seq_len a multiple of 64, block_m and block_n.
+ */
+int stof_retile_lut(const int32_t* full_row_ptr, const int32_t* full_col_idx,
+                    const int32_t* part_row_ptr, const int32_t* part_col_idx, const void* part_block_mask,
+                    int block_m, int block_n, int seq_len,
+                    int32_t* out_full_row_ptr, int32_t* out_full_col_idx,
+                    int32_t* out_part_row_ptr, int32_t* out_part_col_idx,
+                    int32_t* out_load_row_ptr, int32_t* out_load_col_idx,
+                    uint64_t* out_part_bitmask, int32_t* counts,
+                    int64_t cap_full, int64_t cap_part, int64_t cap_load,
+                    void* workspace, int64_t workspace_bytes, void* stream);
 
 /*
  * stof_build_lut without the workspace argument, for callers that cannot allocate device memory

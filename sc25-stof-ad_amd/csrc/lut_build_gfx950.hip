@@ -210,6 +210,59 @@ __global__ __launch_bounds__(256) void lut_additive_blocks_kernel(const void* ma
   }
 }
 
+// A LUT built with another block size (the reference's launcher takes BLOCK_M in {16, 32, 64} and
+// BLOCK_N in {16 .. 128}, block_attn_mask_cuda.cu:6064-6322) described again with 64 x 64 tiles,
+// the one shape the attention kernel has: full source block -> ones, partial source block -> the
+// bits of its additive fp16 values, absent -> zeros.  One wavefront per 64 x 64 target tile, lane l
+// forms the 64-bit row 64 I + l from the (at most four) source blocks it crosses, looked up by
+// binary search in the source row's FULL and PART lists; the tile's class byte and bit rows go to
+// the same scratch lut_compact_kernel reads, so the lists come out exactly as if the dense mask
+// had been classified at 64 x 64.
+struct RetileParams {
+  const int32_t* frp; const int32_t* fci; const int32_t* prp; const int32_t* pci; const half_t* pbm;
+  int bm, bn, n64;                       // source block shape; 64 x 64 tiles per side
+  unsigned char* cls; uint64_t* ws_bits;
+};
+
+__device__ __forceinline__ int find_col(const int32_t* __restrict__ ci, int lo, int hi, int col) {
+  // position of `col` in the ascending list ci[lo, hi), or -1
+  while (lo < hi) { const int mid = (lo + hi) >> 1; const int v = ci[mid]; if (v == col) return mid; if (v < col) lo = mid + 1; else hi = mid; }
+  return -1;
+}
+
+__global__ __launch_bounds__(256) void lut_retile_kernel(const RetileParams p) {
+  const int lane = threadIdx.x & 63;
+  const int64_t tile = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (tile >= (int64_t)p.n64 * p.n64) return;
+  const int I = (int)(tile / p.n64), J = (int)(tile - (int64_t)I * p.n64);
+  const int row = 64 * I + lane;
+  const int ib = row / p.bm, ri = row - ib * p.bm;
+  const int f0 = p.frp[ib], f1 = p.frp[ib + 1], q0 = p.prp[ib], q1 = p.prp[ib + 1];
+  uint64_t word = 0;
+  for (int jb = (64 * J) / p.bn; jb * p.bn < 64 * J + 64; ++jb) {
+    const int c_lo = max(64 * J, jb * p.bn), c_hi = min(64 * J + 64, (jb + 1) * p.bn);
+    const int w = c_hi - c_lo;
+    uint64_t bits = 0;
+    if (find_col(p.fci, f0, f1, jb) >= 0) {
+      bits = w == 64 ? ~0ull : ((1ull << w) - 1);
+    } else {
+      const int slot = find_col(p.pci, q0, q1, jb);
+      if (slot >= 0) {
+        const half_t* src = p.pbm + ((int64_t)slot * p.bm + ri) * p.bn + (c_lo - jb * p.bn);   // (a multiple of 16 elements)
+        for (int e0 = 0; e0 < w; e0 += 8) {
+          const half8_t x = *reinterpret_cast<const half8_t*>(src + e0);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) bits |= (uint64_t)((float)x[e] > -5000.0f) << (e0 + e);
+        }
+      }
+    }
+    word |= bits << (c_lo - 64 * J);
+  }
+  const bool full = __ballot(word != ~0ull) == 0ull, empty = __ballot(word != 0ull) == 0ull;
+  if (lane == 0) p.cls[tile] = (unsigned char)(empty ? kClsEmpty : (full ? kClsFull : kClsPart));
+  if (!full && !empty) p.ws_bits[tile * 64 + lane] = word;
+}
+
 constexpr int kMaxDevices = 64;
 unsigned char* g_scratch_ptr[kMaxDevices] = {nullptr};
 
@@ -294,6 +347,43 @@ extern "C" int stof_build_lut(const void* mask, int elem_bytes, int64_t ld, int 
   uint64_t* bits = reinterpret_cast<uint64_t*>(cls + (tiles + 255) / 256 * 256);
   return build(mask, elem_bytes, ld, seq_len, block_m, block_n, full_row_ptr, full_col_idx, part_row_ptr, part_col_idx,
                load_row_ptr, load_col_idx, part_bitmask, counts, cap_full, cap_part, cap_load, cls, bits, (hipStream_t)stream);
+}
+
+extern "C" int stof_retile_lut(const int32_t* full_row_ptr, const int32_t* full_col_idx,
+                               const int32_t* part_row_ptr, const int32_t* part_col_idx, const void* part_block_mask,
+                               int block_m, int block_n, int seq_len,
+                               int32_t* out_full_row_ptr, int32_t* out_full_col_idx,
+                               int32_t* out_part_row_ptr, int32_t* out_part_col_idx,
+                               int32_t* out_load_row_ptr, int32_t* out_load_col_idx,
+                               uint64_t* out_part_bitmask, int32_t* counts,
+                               int64_t cap_full, int64_t cap_part, int64_t cap_load,
+                               void* workspace, int64_t workspace_bytes, void* stream) {
+  if (!full_row_ptr || !part_row_ptr) return STOF_ERR_NULL_POINTER;
+  if (!block_ok(block_m) || !block_ok(block_n)) return STOF_ERR_UNSUPPORTED;
+  if (seq_len <= 0 || seq_len % 64 != 0 || seq_len % block_m != 0 || seq_len % block_n != 0) return STOF_ERR_BAD_SHAPE;
+  if (part_block_mask && !stof_aligned16(part_block_mask)) return STOF_ERR_MISALIGNED;
+  int rc = check_outputs(out_full_row_ptr, out_full_col_idx, out_part_row_ptr, out_part_col_idx, out_load_row_ptr, out_load_col_idx,
+                         out_part_bitmask, 64, 64, cap_full, cap_part, cap_load);
+  if (rc != STOF_OK) return rc;
+  if (!workspace || !out_part_bitmask) return STOF_ERR_NULL_POINTER;
+  if (workspace_bytes < stof_build_lut_workspace_bytes(seq_len, 64, 64)) return STOF_ERR_BAD_SHAPE;
+  if ((reinterpret_cast<uintptr_t>(workspace) & 7) != 0) return STOF_ERR_MISALIGNED;
+  const int n64 = seq_len / 64;
+  const int64_t tiles = (int64_t)n64 * n64;
+  RetileParams r;
+  r.frp = full_row_ptr; r.fci = full_col_idx; r.prp = part_row_ptr; r.pci = part_col_idx; r.pbm = (const half_t*)part_block_mask;
+  r.bm = block_m; r.bn = block_n; r.n64 = n64;
+  r.cls = static_cast<unsigned char*>(workspace);
+  r.ws_bits = reinterpret_cast<uint64_t*>(r.cls + (tiles + 255) / 256 * 256);
+  hipLaunchKernelGGL(lut_retile_kernel, dim3((unsigned)((tiles + 3) / 4)), dim3(256), 0, (hipStream_t)stream, r);
+  LutParams p;
+  p.mask = nullptr; p.ld = 0; p.S = seq_len; p.bm = 64; p.bn = 64; p.nQ = n64; p.nK = n64;
+  p.cls = r.cls; p.ws_bits = r.ws_bits;
+  p.frp = out_full_row_ptr; p.fci = out_full_col_idx; p.prp = out_part_row_ptr; p.pci = out_part_col_idx;
+  p.lrp = out_load_row_ptr; p.lci = out_load_col_idx; p.pbits = out_part_bitmask; p.counts = counts;
+  p.cap_full = cap_full; p.cap_part = cap_part; p.cap_load = cap_load;
+  hipLaunchKernelGGL(lut_compact_kernel, dim3((unsigned)n64), dim3(256), 0, (hipStream_t)stream, p);
+  return stof_check_launch();
 }
 
 extern "C" int64_t stof_build_lut_static_max_tiles(void) { return kStaticMaxTiles; }

@@ -56,6 +56,7 @@ PYBIND11_MODULE(_stof_ext, m) {
   STOF_BIND(stof_rowwise_attn_fwd);
   STOF_BIND(stof_build_lut_workspace_bytes);
   STOF_BIND(stof_build_lut);
+  STOF_BIND(stof_retile_lut);
   STOF_BIND(stof_build_lut_static_max_tiles);
   STOF_BIND(stof_build_lut_static);
   STOF_BIND(stof_lut_additive_blocks);

@@ -3,6 +3,7 @@ can hand over bit rows it has already built) and the attention operators (which 
 
 BITS_ATTR = "_stof_packed_bits"       # on part_block_mask / row_mask: (content key, packed bit rows)
 LUT_OK_ATTR = "_stof_lut_checked"     # on load_col_idx: content keys of the four index tensors found in order
+DEVICE_BUILT_ATTR = "_stof_device_built"   # on tensors the library's kernels produced: their attached data is not re-derivable
 
 
 def content_key(t):

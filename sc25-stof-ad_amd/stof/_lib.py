@@ -43,6 +43,8 @@ _SIGNATURES = {
     "stof_build_lut_workspace_bytes": (c_int64, [c_int, c_int, c_int]),
     "stof_build_lut": (c_int, [_P, c_int, c_int64, c_int, c_int, c_int, _P, _P, _P, _P, _P, _P, _P, _P,
                                c_int64, c_int64, c_int64, _P, c_int64, _P]),
+    "stof_retile_lut": (c_int, [_P, _P, _P, _P, _P, c_int, c_int, c_int, _P, _P, _P, _P, _P, _P, _P, _P,
+                                c_int64, c_int64, c_int64, _P, c_int64, _P]),
     "stof_build_lut_static_max_tiles": (c_int64, []),
     "stof_build_lut_static": (c_int, [_P, c_int, c_int64, c_int, c_int, c_int, _P, _P, _P, _P, _P, _P, _P, _P,
                                       c_int64, c_int64, c_int64, _P]),
@@ -109,6 +111,8 @@ def lib(binding=None):
     """Load (once) and return the binding in use; raise if the library is absent.
     ``binding="ctypes"`` / ``"ext"`` returns that binding without changing the one in use."""
     global _lib, _ext_used
+    if _lib is not None and binding is None:
+        return _lib
     if not os.path.exists(LIB_PATH):
         raise StofError(
             f"{LIB_PATH} is missing: build it with `python sc25-stof-ad_amd/csrc/build.py` "
@@ -132,7 +136,8 @@ def binding_name():
 
 def i64x3(a, b, c):
     """An int64[3] argument (the stride triples of the attention entry points) for the binding in use."""
-    lib()
+    if _lib is None:
+        lib()
     return (a, b, c) if _ext_used else _I64x3(a, b, c)
 
 
@@ -144,4 +149,5 @@ def check(status, what):
 
 def strides3(t):
     """(batch, head, seq) element strides of a [B,H,S,D] view as an int64[3]."""
-    return i64x3(t.stride(0), t.stride(1), t.stride(2))
+    s = t.stride()
+    return i64x3(s[0], s[1], s[2])

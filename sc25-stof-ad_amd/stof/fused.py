@@ -50,18 +50,21 @@ _DTYPES = {torch.float16: 0, torch.bfloat16: 1}   # STOF_DTYPE_*
 def _f16c(name, t, allow_none=False, like=None):
     """``t`` contiguous; a CUDA float16 tensor, or of ``like``'s 16-bit format if that is given."""
     if t is None:
-        _require(allow_none, f"{name} is required")
+        if not allow_none:
+            raise StofError(f"{name} is required")
         return None
     want = torch.float16 if like is None else like.dtype
     if not (t.is_cuda and t.dtype == want):
         raise StofError(f"{name} must be a CUDA {str(want).replace('torch.', '')} tensor")
-    return t.contiguous()
+    return t if t.is_contiguous() else t.contiguous()
 
 
 def _elem16(name, t):
     """``t`` must be a CUDA tensor in one of the two 16-bit formats; its STOF_DTYPE_* code."""
-    _require(t.is_cuda and t.dtype in _DTYPES, f"{name} must be a CUDA float16 or bfloat16 tensor")
-    return _DTYPES[t.dtype]
+    dt = _DTYPES.get(t.dtype) if t.is_cuda else None
+    if dt is None:
+        raise StofError(f"{name} must be a CUDA float16 or bfloat16 tensor")
+    return dt
 
 
 def _p(t):
@@ -86,15 +89,19 @@ def bias_residual_layernorm(x, bias, residual, gamma, beta, eps=1e-5, return_sta
     """LN(x + bias + residual) * gamma + beta over the last dim; any operand but x may be None.
     float16 or, all operands alike, bfloat16."""
     dt = _elem16("x", x)
-    x = x.contiguous()
+    if not x.is_contiguous():
+        x = x.contiguous()
     N = x.shape[-1]
     M = x.numel() // N
     bias = _f16c("bias", bias, True, x); residual = _f16c("residual", residual, True, x)
     gamma = _f16c("gamma", gamma, True, x); beta = _f16c("beta", beta, True, x)
     for name, t in (("bias", bias), ("gamma", gamma), ("beta", beta)):
-        _require(t is None or t.numel() == N, f"{name} must have {N} elements")
-    _require(residual is None or residual.shape == x.shape, "residual must have x's shape")
-    _require(out is None or (out.shape == x.shape and out.dtype == x.dtype and out.is_contiguous()), "out must be contiguous, with x's shape")
+        if t is not None and t.numel() != N:
+            raise StofError(f"{name} must have {N} elements")
+    if residual is not None and residual.shape != x.shape:
+        raise StofError("residual must have x's shape")
+    if out is not None and not (out.shape == x.shape and out.dtype == x.dtype and out.is_contiguous()):
+        raise StofError("out must be contiguous, with x's shape")
     y = torch.empty_like(x) if out is None else out
     mean = rstd = None
     if return_stats:
@@ -132,23 +139,37 @@ def gemm_bias_act(x, Wt, bias=None, act="none", out=None, splits=None):
     ``splits``: None = the library's rule (stof_gemm_bias_act_splitk_plan: K split over several
     workgroups per tile where the output has few tiles and K is long), 1 = one workgroup per tile
     (stof_gemm_bias_act), 2 .. 8 = that many splits (stof_gemm_bias_act_splitk)."""
-    _require(act in ACT, f"unknown activation {act!r}")
-    _require(splits is None or 1 <= int(splits) <= 8, "splits must be None or 1 .. 8")
+    if act not in ACT:
+        raise StofError(f"unknown activation {act!r}")
+    if splits is not None and not 1 <= int(splits) <= 8:
+        raise StofError("splits must be None or 1 .. 8")
     dt = _elem16("x", x)
     Wt = _f16c("Wt", Wt, like=x); bias = _f16c("bias", bias, True, x)
     K = x.shape[-1]
     N = Wt.shape[0]
-    _require(Wt.dim() == 2 and Wt.shape[1] == K, f"Wt must be [N, {K}]")
-    _require(bias is None or bias.numel() == N, f"bias must have {N} elements")
-    x2 = x.reshape(-1, K)
-    if x2.stride(1) != 1:
-        x2 = x2.contiguous()
-    M = x2.shape[0]
+    if Wt.dim() != 2 or Wt.shape[1] != K:
+        raise StofError(f"Wt must be [N, {K}]")
+    if bias is not None and bias.numel() != N:
+        raise StofError(f"bias must have {N} elements")
+    # rows of x: dense tensors (the usual case) are addressed as they are, others through a 2-D view
+    if x.is_contiguous():
+        x2, lda = x, K
+    else:
+        x2 = x if x.dim() == 2 else x.reshape(-1, K)
+        if x2.stride(1) != 1:
+            x2 = x2.contiguous()
+        lda = x2.stride(0)
+    M = x.numel() // K
     if out is None:
         out = torch.empty(x.shape[:-1] + (N,), dtype=x.dtype, device=x.device)
-    _require(out.dtype == x.dtype, "out must have x's element format")
-    o2 = out.view(-1, N)
-    _require(o2.shape[0] == M and o2.stride(1) == 1, "out must be [..., N] with contiguous rows")
+        o2, ldc = out, N
+    else:
+        if out.dtype != x.dtype:
+            raise StofError("out must have x's element format")
+        o2 = out if out.dim() == 2 else out.view(-1, N)
+        if o2.shape[0] != M or o2.stride(1) != 1:
+            raise StofError("out must be [..., N] with contiguous rows")
+        ldc = o2.stride(0)
     lib = _lib.lib()
     st = _stream(o2)
     if splits is None:
@@ -158,12 +179,12 @@ def gemm_bias_act(x, Wt, bias=None, act="none", out=None, splits=None):
         _require(nbytes > 0, f"shape not supported by the split-K form: M {M}, N {N}")
         ws = _splitk_workspace(x.device, st, nbytes)
         check(lib.stof_gemm_bias_act_splitk_dt(x2.data_ptr(), Wt.data_ptr(), _p(bias), o2.data_ptr(),
-                                               M, N, K, x2.stride(0), o2.stride(0), ACT[act], int(splits),
+                                               M, N, K, lda, ldc, ACT[act], int(splits),
                                                ws.data_ptr(), ws.numel(), dt, st),
               "stof_gemm_bias_act_splitk")
         return out
     check(lib.stof_gemm_bias_act_dt(x2.data_ptr(), Wt.data_ptr(), _p(bias), o2.data_ptr(),
-                                    M, N, K, x2.stride(0), o2.stride(0), ACT[act], dt, st),
+                                    M, N, K, lda, ldc, ACT[act], dt, st),
           "stof_gemm_bias_act")
     return out
 
@@ -274,29 +295,37 @@ def gemm_bias_residual_layernorm(x, Wt, bias, residual, gamma, beta, eps=1e-5, o
     In both the pre-normalisation values stay in registers.
     ``form="split"``: stof_gemm_bias_act, then stof_bias_residual_layernorm.
     ``form="auto"``: ``ln_gemm_form`` chooses."""
-    _require(form in ("auto", "row", "cluster", "split"), f"unknown form {form!r}")
+    if form not in ("auto", "row", "cluster", "split"):
+        raise StofError(f"unknown form {form!r}")
     if form == "auto":
         form = ln_gemm_form(x.numel() // x.shape[-1], Wt.shape[0], x.shape[-1])
     if form == "split":
         y = gemm_bias_act(x, Wt, None, "none")
-        return bias_residual_layernorm(y, bias, None if residual is None else residual.reshape(y.shape), gamma, beta, eps, out=out)
+        if residual is not None and residual.shape != y.shape:
+            residual = residual.reshape(y.shape)
+        return bias_residual_layernorm(y, bias, residual, gamma, beta, eps, out=out)
     dt = _elem16("x", x)
-    _require(dt == 0 or form == "cluster", "the row form takes float16 only")
-    x = x.contiguous(); Wt = _f16c("Wt", Wt, like=x)
+    if dt != 0 and form != "cluster":
+        raise StofError("the row form takes float16 only")
+    if not x.is_contiguous():
+        x = x.contiguous()
+    Wt = _f16c("Wt", Wt, like=x)
     bias = _f16c("bias", bias, True, x); residual = _f16c("residual", residual, True, x)
     gamma = _f16c("gamma", gamma, True, x); beta = _f16c("beta", beta, True, x)
     K = x.shape[-1]
     N = Wt.shape[0]
     M = x.numel() // K
-    _require(Wt.dim() == 2 and Wt.shape[1] == K, f"Wt must be [N, {K}]")
-    _require(residual is None or residual.numel() == M * N, "residual must be [..., N] matching x's rows")
+    if Wt.dim() != 2 or Wt.shape[1] != K:
+        raise StofError(f"Wt must be [N, {K}]")
+    if residual is not None and residual.numel() != M * N:
+        raise StofError("residual must be [..., N] matching x's rows")
     for name, t in (("bias", bias), ("gamma", gamma), ("beta", beta)):
-        _require(t is None or t.numel() == N, f"{name} must have {N} elements")
+        if t is not None and t.numel() != N:
+            raise StofError(f"{name} must have {N} elements")
     if out is None:
         out = torch.empty(x.shape[:-1] + (N,), dtype=x.dtype, device=x.device)
-    _require(out.dtype == x.dtype, "out must have x's element format")
-    _require(out.device == x.device and tuple(out.shape) == tuple(x.shape[:-1]) + (N,) and out.is_contiguous(),
-             f"out must be a contiguous {tuple(x.shape[:-1]) + (N,)} tensor on x's device")
+    elif not (out.dtype == x.dtype and out.device == x.device and tuple(out.shape) == tuple(x.shape[:-1]) + (N,) and out.is_contiguous()):
+        raise StofError(f"out must be a contiguous {tuple(x.shape[:-1]) + (N,)} tensor of x's element format on x's device")
     lib = _lib.lib()
     st = _stream(out)
     if form == "cluster":

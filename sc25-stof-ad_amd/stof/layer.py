@@ -21,7 +21,7 @@ tuner.
 import torch
 
 from . import fused
-from .ops import block_attn
+from .ops import block_attn, block_attn_packed_qkv
 
 
 class EncoderLayer:
@@ -93,8 +93,7 @@ class EncoderLayer:
         H = self.n_heads
         hd = D // H
         qkv = fused.gemm_bias_act(x, self.Wqkv, self.bqkv, "none")           # [B,S,3D]
-        q, k, v = (qkv[..., t * D:(t + 1) * D].view(B, S, H, hd).permute(0, 2, 1, 3) for t in range(3))
-        attn = block_attn(q, k, v, lut, block, block, out_layout="bshd")      # [B,S,D]
+        attn = block_attn_packed_qkv(qkv, H, lut, block, block)               # q, k, v read in place; [B,S,D]
         h = self._gemm_ln(attn, self.Wo, self.bo, x, self.g1, self.be1)
         y = self._ffn(h)
         if check:

@@ -225,13 +225,15 @@ def build_lut_device(Mask, block_size_m=64, block_size_n=64):
     full capacity (entries beyond the last row pointer are unused) and ``part_block_mask`` is a
     one-block placeholder that carries the partial tiles' packed bit rows, which is what the
     attention kernel reads.  64 x 64 blocks only."""
-    from ._cache import BITS_ATTR, LUT_OK_ATTR, content_key
+    from ._cache import BITS_ATTR, DEVICE_BUILT_ATTR, LUT_OK_ATTR, content_key
     if not _device_path(Mask, block_size_m, block_size_n) or (block_size_m, block_size_n) != (64, 64):
         raise ValueError("build_lut_device needs an fp16 / fp32 [B,S,S] mask on the GPU and 64 x 64 blocks")
     _, frp, fci, prp, pci, lrp, lci, bits, _ = _build_on_device(Mask[0], 64, 64, want_bits=True)
     pbm = torch.ones(1, 64, 64, dtype=torch.float16, device=Mask.device)
     setattr(pbm, BITS_ATTR, (content_key(pbm), bits))
     setattr(lci, LUT_OK_ATTR, tuple(content_key(t) for t in (lci, pci, lrp, prp)))   # in order by construction
+    # (block_attn(..., revalidate=True) leaves these two attachments in place: there is nothing to derive them from again)
+    setattr(pbm, DEVICE_BUILT_ATTR, True); setattr(lci, DEVICE_BUILT_ATTR, True)
     return frp, fci, prp, pci, pbm, lrp, lci
 
 

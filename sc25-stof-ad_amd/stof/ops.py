@@ -17,10 +17,11 @@ import torch
 from torch.autograd import Function
 
 from . import _lib
-from ._cache import BITS_ATTR as _BITS_ATTR, LUT_OK_ATTR as _LUT_OK_ATTR, content_key as _content_key
+from ._cache import (BITS_ATTR as _BITS_ATTR, DEVICE_BUILT_ATTR as _DEVICE_BUILT_ATTR, LUT_OK_ATTR as _LUT_OK_ATTR,
+                     content_key as _content_key)
 from ._lib import StofError, check, strides3
 
-__all__ = ["block_attn", "rowwise_attn", "block_attn_mask_op", "rowwise_attn_full_op", "rowwise_attn_sliding_op",
+__all__ = ["block_attn", "block_attn_packed_qkv", "rowwise_attn", "block_attn_mask_op", "rowwise_attn_full_op", "rowwise_attn_sliding_op",
            "rowwise_attn_mask_op", "pack_mask_bits", "set_attention_launch_form", "StofError"]
 
 
@@ -88,8 +89,15 @@ def pack_mask_bits(src, additive):
 
 
 def _drop_caches(lut):
+    """Forget what was derived from a LUT's tensors (``revalidate=True``).  Tensors the library
+    itself produced on the device (masks.build_lut_device, a re-tiled LUT) keep their bit rows
+    and their "in order" mark: those ARE the LUT's content there - the placeholder block mask
+    they hang on holds nothing to derive them from again."""
     for t in lut:
+        keep = (_BITS_ATTR, _LUT_OK_ATTR) if getattr(t, _DEVICE_BUILT_ATTR, False) else ()
         for attr in (_BITS_ATTR, _LUT_OK_ATTR, _LUT64_ATTR, _LUT_READY_ATTR):
+            if attr in keep:
+                continue
             if hasattr(t, attr):
                 try:
                     delattr(t, attr)
@@ -129,6 +137,11 @@ def _check_lut_order(lrp, lci, prp, pci, n_cols):
         if ci.numel() == 0:
             continue
         flat = rp.reshape(-1, rp.shape[-1]).long()
+        used = int(flat.max())
+        _require(0 <= used <= ci.numel(), f"{name}_row_ptr points past the end of {name}_col_idx")
+        ci = ci[:used]                       # (lists kept at full capacity: the tail is unused)
+        if used == 0:
+            continue
         ok = bool((ci >= 0).all()) and bool((ci < n_cols).all())
         if ci.numel() > 1:
             inc = ci[1:] > ci[:-1]
@@ -153,20 +166,64 @@ def _lut_at_64(lut, S, block_m, block_n):
     """The same mask described with 64 x 64 blocks, for a LUT built with another block size
     (the reference's kernels cover BLOCK_M / BLOCK_N of 16..128,
     src/ops/src/block_attn_mask_cuda.cu:6064-6322; the kernel here has one tile shape).  The
-    LUT is expanded to the dense 0/1 mask it encodes and classified again; the attention
-    result depends on the mask only, so this changes nothing but the tiling.  Done once per
+    library re-tiles the LUT on the device (stof_retile_lut: full source block -> ones, partial
+    -> the bits of its additive values, absent -> zeros, classified again at 64 x 64); the
+    attention result depends on the mask only, so this changes nothing but the tiling.  Shared
+    and per-sample LUTs alike (a per-sample LUT is re-tiled sample by sample).  Done once per
     LUT (kept on the LOAD column tensor, keyed by the tensors' content versions)."""
-    from . import masks as pm
     frp, fci, prp, pci, pbm, lrp, lci = lut
     key = tuple(_content_key(t) for t in lut) + (block_m, block_n)
     cached = getattr(lci, _LUT64_ATTR, None)
     if cached is not None and cached[0] == key:
         return cached[1]
-    _require(lrp.dim() == 1, "per-sample LUTs are supported with 64 x 64 blocks only")
-    _require(tuple(pbm.shape[-2:]) == (block_m, block_n) or int(prp.reshape(-1)[-1]) == 0,
-             f"part_block_mask must hold {block_m} x {block_n} blocks")
-    dense = pm.expand_sparse_storage((None, frp, fci, prp, pci, pbm, lrp, lci), S, block_m, block_n)
-    lut64 = tuple(pm.get_sparse_storage(dense[None], 64, 64)[1:])
+    _require(block_m in (16, 32, 64, 128) and block_n in (16, 32, 64, 128),
+             f"LUT block sizes must be 16, 32, 64 or 128, got {block_m} x {block_n}")
+    n_part = int(prp.reshape(-1)[-1])
+    _require(n_part == 0 or (pbm.dim() == 3 and tuple(pbm.shape[-2:]) == (block_m, block_n) and pbm.shape[0] >= n_part),
+             f"part_block_mask must hold {n_part} blocks of {block_m} x {block_n}")
+    dev = lrp.device
+    lib = _lib.lib()
+    n64 = S // 64
+    tiles = n64 * n64
+    pbm_c = pbm.contiguous() if n_part else None
+    ws = torch.empty(lib.stof_build_lut_workspace_bytes(S, 64, 64), dtype=torch.uint8, device=dev)
+    frp2, prp2 = frp.reshape(-1, frp.shape[-1]), prp.reshape(-1, prp.shape[-1])
+    per_sample = []
+    for b in range(frp2.shape[0]):
+        i32 = lambda k: torch.empty(k, dtype=torch.int32, device=dev)
+        o_frp, o_prp, o_lrp = i32(n64 + 1), i32(n64 + 1), i32(n64 + 1)
+        o_fci, o_pci, o_lci, counts = i32(tiles), i32(tiles), i32(tiles), i32(4)
+        o_bits = torch.empty((tiles, 64), dtype=torch.int64, device=dev)
+        check(lib.stof_retile_lut(frp2[b].data_ptr(), _ptr(fci), prp2[b].data_ptr(), _ptr(pci), _ptr(pbm_c), block_m, block_n, S,
+                                  o_frp.data_ptr(), o_fci.data_ptr(), o_prp.data_ptr(), o_pci.data_ptr(),
+                                  o_lrp.data_ptr(), o_lci.data_ptr(), o_bits.data_ptr(), counts.data_ptr(),
+                                  tiles, tiles, tiles, ws.data_ptr(), ws.numel(), _stream(dev)), "stof_retile_lut")
+        per_sample.append((o_frp, o_fci, o_prp, o_pci, o_lrp, o_lci, o_bits, counts))
+    if lrp.dim() == 1:
+        # one shared LUT: the lists stay at full capacity (entries past the last row pointer unused), nothing is read back
+        o_frp, o_fci, o_prp, o_pci, o_lrp, o_lci, o_bits, _ = per_sample[0]
+    else:
+        # per-sample: exact lengths are needed to concatenate (one read of the counts per sample), row pointers become absolute
+        fo = po = lo = 0
+        parts = {k: [] for k in ("frp", "fci", "prp", "pci", "lrp", "lci", "bits")}
+        for (a, bq, c, d, e, f, g, counts) in per_sample:
+            n_full, n_part64, n_load, overflow = counts.tolist()
+            assert not overflow
+            parts["frp"].append(a + fo); parts["fci"].append(bq[:n_full])
+            parts["prp"].append(c + po); parts["pci"].append(d[:n_part64])
+            parts["lrp"].append(e + lo); parts["lci"].append(f[:n_load]); parts["bits"].append(g[:n_part64])
+            fo += n_full; po += n_part64; lo += n_load
+        st = lambda k: torch.stack(parts[k], 0).contiguous()
+        ct = lambda k: torch.cat(parts[k], 0).contiguous()
+        o_frp, o_fci, o_prp, o_pci, o_lrp, o_lci, o_bits = st("frp"), ct("fci"), st("prp"), ct("pci"), st("lrp"), ct("lci"), ct("bits")
+    # The attention kernel reads bit rows, not additive blocks: a one-block placeholder carries them
+    # (as masks.build_lut_device does), and the lists are in order by construction.
+    o_pbm = torch.ones(1, 64, 64, dtype=torch.float16, device=dev)
+    setattr(o_pbm, _BITS_ATTR, (_content_key(o_pbm), o_bits))
+    setattr(o_pbm, _DEVICE_BUILT_ATTR, True)
+    setattr(o_lci, _LUT_OK_ATTR, tuple(_content_key(t) for t in (o_lci, o_pci, o_lrp, o_prp)))
+    setattr(o_lci, _DEVICE_BUILT_ATTR, True)
+    lut64 = (o_frp, o_fci, o_prp, o_pci, o_pbm, o_lrp, o_lci)
     try:
         setattr(lci, _LUT64_ATTR, (key, lut64))
     except AttributeError:
@@ -183,8 +240,12 @@ def _prepared_lut(lut, B, S, block_m, block_n, dev):
     packing of the partial blocks, re-tiling to 64 x 64) is done once per LUT: the result is
     kept on the LOAD column tensor, keyed by the identity and content version of all seven
     tensors, the problem size and the device, and it holds the tensors it points into."""
-    lci = lut[6]
-    key = (B, S, block_m, block_n, dev) + tuple((id(t),) + _content_key(t) for t in lut)
+    a, b, c, d, e, f, lci = lut
+    # (identity, storage address and content version of the seven tensors, spelled out: this runs on every call)
+    key = (B, S, block_m, block_n, dev,
+           id(a), a.data_ptr(), a._version, id(b), b.data_ptr(), b._version, id(c), c.data_ptr(), c._version,
+           id(d), d.data_ptr(), d._version, id(e), e.data_ptr(), e._version, id(f), f.data_ptr(), f._version,
+           id(lci), lci.data_ptr(), lci._version)
     cached = getattr(lci, _LUT_READY_ATTR, None)
     if cached is not None and cached[0] == key:
         return cached[1], cached[2], cached[5]
@@ -207,6 +268,7 @@ def _prepared_lut(lut, B, S, block_m, block_n, dev):
     if (block_m, block_n) != (64, 64):
         _require(S % 64 == 0, f"seq_len {S} must be a multiple of 64")
         frp, fci, prp, pci, pbm, lrp, lci_c = _lut_at_64((frp, fci, prp, pci, pbm, lrp, lci_c), S, block_m, block_n)
+        lut_bs = S // 64 + 1 if lrp.dim() == 2 else 0
     bits = _packed_partial_bits(pbm)
     keep = (frp, fci, prp, pci, bits, lrp, lci_c)
     ptrs = tuple(_ptr(t) for t in keep)
@@ -222,24 +284,27 @@ def _plan(plans, lut_ptrs, lut_bs, B, H, S, form, dev):
     """The precomputed walk of this LUT for the launch form the library will take (built by one
     small launch the first time a LUT meets that form, then kept with the LUT's other prepared
     data).  Returns (pointer, bytes, rows per workgroup) or (None, 0, 0) where no plan applies."""
+    hit = plans.get((B, H, S, form))
+    if hit is not None:
+        return hit
     lib = _lib.lib()
     rows = lib.stof_attn_plan_rows(B, H, S, form)
-    if rows <= 0:
-        return None, 0, 0
-    plan = plans.get(rows)
-    if plan is None:
-        batches = B if lut_bs else 1
-        nbytes = lib.stof_attn_plan_bytes(S, rows, batches)
-        if nbytes <= 0:
-            plans[rows] = False
-            return None, 0, 0
-        plan = torch.empty(nbytes // 8, dtype=torch.int64, device=dev)
-        check(lib.stof_attn_plan_build(lut_ptrs[2], lut_ptrs[3], lut_ptrs[5], lut_ptrs[6], S, lut_bs, batches, rows,
-                                       plan.data_ptr(), nbytes, _stream(dev)), "stof_attn_plan_build")
-        plans[rows] = plan
-    if plan is False:
-        return None, 0, 0
-    return plan.data_ptr(), plan.numel() * 8, rows
+    triple = (None, 0, 0)
+    if rows > 0:
+        plan = plans.get(rows)
+        if plan is None:
+            batches = B if lut_bs else 1
+            nbytes = lib.stof_attn_plan_bytes(S, rows, batches)
+            plan = False
+            if nbytes > 0:
+                plan = torch.empty(nbytes // 8, dtype=torch.int64, device=dev)
+                check(lib.stof_attn_plan_build(lut_ptrs[2], lut_ptrs[3], lut_ptrs[5], lut_ptrs[6], S, lut_bs, batches, rows,
+                                               plan.data_ptr(), nbytes, _stream(dev)), "stof_attn_plan_build")
+            plans[rows] = plan
+        if plan is not False:
+            triple = (plan.data_ptr(), plan.numel() * 8, rows)
+    plans[(B, H, S, form)] = triple
+    return triple
 
 
 def _check_i32(name, t, device):
@@ -265,41 +330,87 @@ def block_attn(q, k, v, lut, block_m=64, block_n=64, out=None, out_layout="bhsd"
     is cached for this LUT (validation, packed bit rows, re-tiling) and prepares it again: for
     LUT buffers rewritten behind PyTorch's back, which the caches cannot see.
     """
-    _require(q.is_cuda, "q must be a CUDA tensor (this path has no CPU implementation)")
+    if not q.is_cuda:
+        raise StofError("q must be a CUDA tensor (this path has no CPU implementation)")
     dev = q.device
-    _require(q.dtype in _DTYPES, f"q must be float16 or bfloat16, got {q.dtype}")
-    for name, t in (("q", q), ("k", k), ("v", v)):
-        _require(t.dtype == q.dtype, f"{name} must be {q.dtype} like q, got {t.dtype}")
-        _require(t.dim() == 4 and t.stride(3) == 1, f"{name} must be [B,H,S,D] with contiguous D")
-        _require(t is q or t.device == dev, f"{name} is on a different device than q")
-    _require(k.shape == q.shape and v.shape == q.shape, "q, k, v must have the same shape")
-    B, H, S, D = q.shape
+    dt = _DTYPES.get(q.dtype)
+    if dt is None:
+        raise StofError(f"q must be float16 or bfloat16, got {q.dtype}")
+    qs, ks, vs = q.stride(), k.stride(), v.stride()
+    for name, t, st in (("q", q, qs), ("k", k, ks), ("v", v, vs)):
+        if t.dtype != q.dtype:
+            raise StofError(f"{name} must be {q.dtype} like q, got {t.dtype}")
+        if len(st) != 4 or st[3] != 1:
+            raise StofError(f"{name} must be [B,H,S,D] with contiguous D")
+        if t is not q and t.device != dev:
+            raise StofError(f"{name} is on a different device than q")
+    shape = q.shape
+    if k.shape != shape or v.shape != shape:
+        raise StofError("q, k, v must have the same shape")
+    B, H, S, D = shape
+    if out is None:
+        out = torch.empty((B, H, S, D) if out_layout == "bhsd" else (B, S, H * D), dtype=q.dtype, device=dev)
+    os_ = out.stride()
+    if out_layout == "bhsd":
+        if out.shape != shape or os_[3] != 1:
+            raise StofError("out must be [B,H,S,D] with contiguous D")
+        ostr = _lib.i64x3(os_[0], os_[1], os_[2])
+    elif out_layout == "bshd":
+        if out.shape != (B, S, H * D) or os_[2] != 1:
+            raise StofError("out must be [B,S,H*D] with contiguous last dim")
+        ostr = _lib.i64x3(os_[0], D, os_[1])
+    else:
+        raise StofError(f"unknown out_layout {out_layout!r}")
+    if out.dtype != q.dtype or out.device != dev:
+        raise StofError("out must have q's dtype and device")
+    return _attn_launch(q.data_ptr(), k.data_ptr(), v.data_ptr(), out, _lib.i64x3(qs[0], qs[1], qs[2]),
+                        _lib.i64x3(ks[0], ks[1], ks[2]), _lib.i64x3(vs[0], vs[1], vs[2]), ostr, B, H, S, D, dt, dev,
+                        lut, block_m, block_n, softmax_scale, launch_form, revalidate, use_plan)
+
+
+def _attn_launch(qp, kp, vp, out, qstr, kstr, vstr, ostr, B, H, S, D, dt, dev, lut, block_m, block_n,
+                 softmax_scale, launch_form, revalidate, use_plan):
+    """The LUT side of an attention call (prepared data, plan) and the launch; q, k, v arrive as
+    validated device addresses with their (batch, head, row) element strides."""
     form = _form(launch_form)
     if revalidate:
         _drop_caches(lut)
     lut_ptrs, lut_bs, plans = _prepared_lut(lut, B, S, block_m, block_n, dev)
-    if out is None:
-        if out_layout == "bhsd":
-            out = torch.empty((B, H, S, D), dtype=q.dtype, device=dev)
-        else:
-            out = torch.empty((B, S, H * D), dtype=q.dtype, device=dev)
-    if out_layout == "bhsd":
-        _require(out.shape == (B, H, S, D) and out.stride(3) == 1, "out must be [B,H,S,D] with contiguous D")
-        ostr = strides3(out)
-    elif out_layout == "bshd":
-        _require(out.shape == (B, S, H * D) and out.stride(2) == 1, "out must be [B,S,H*D] with contiguous last dim")
-        ostr = _lib.i64x3(out.stride(0), D, out.stride(1))
-    else:
-        raise StofError(f"unknown out_layout {out_layout!r}")
-    _require(out.dtype == q.dtype and out.device == dev, "out must have q's dtype and device")
     scale = softmax_scale if softmax_scale is not None else 1.0 / math.sqrt(D)
     plan_ptr, plan_bytes, plan_rows = _plan(plans, lut_ptrs, lut_bs, B, H, S, form, dev) if use_plan else (None, 0, 0)
     check(_lib.lib().stof_block_attn_fwd_planned(
-        q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(),
-        *lut_ptrs, 64, 64, scale,
-        strides3(q), strides3(k), strides3(v), ostr,
-        B, S, H, D, _DTYPES[q.dtype], lut_bs, form, plan_ptr, plan_bytes, plan_rows, _stream(dev)), "stof_block_attn_fwd")
+        qp, kp, vp, out.data_ptr(), *lut_ptrs, 64, 64, scale, qstr, kstr, vstr, ostr,
+        B, S, H, D, dt, lut_bs, form, plan_ptr, plan_bytes, plan_rows, _stream(dev)), "stof_block_attn_fwd")
     return out
+
+
+def block_attn_packed_qkv(qkv, n_heads, lut, block_m=64, block_n=64, out=None, softmax_scale=None,
+                          launch_form=None, use_plan=True):
+    """``block_attn`` on the packed projection ``qkv`` [B, S, 3*H*D] (q, k, v side by side in the
+    last dim, each as H heads of D channels - what one QKV GEMM writes), result ``[B, S, H*D]``.
+    The same launch as ``block_attn`` on the three strided views; this entry spares the nine
+    view / permute operations that forming them costs on the host."""
+    if not qkv.is_cuda:
+        raise StofError("qkv must be a CUDA tensor (this path has no CPU implementation)")
+    dt = _DTYPES.get(qkv.dtype)
+    if dt is None:
+        raise StofError(f"qkv must be float16 or bfloat16, got {qkv.dtype}")
+    if qkv.dim() != 3 or qkv.stride(2) != 1 or qkv.shape[2] % (3 * n_heads) != 0:
+        raise StofError("qkv must be [B, S, 3*H*D] with a contiguous last dim")
+    B, S, D3 = qkv.shape
+    Dm = D3 // 3
+    D = Dm // n_heads
+    dev = qkv.device
+    if out is None:
+        out = torch.empty((B, S, Dm), dtype=qkv.dtype, device=dev)
+    elif out.shape != (B, S, Dm) or out.stride(2) != 1 or out.dtype != qkv.dtype or out.device != dev:
+        raise StofError("out must be [B,S,H*D] with contiguous last dim, of qkv's dtype and device")
+    sb, ss, _ = qkv.stride()
+    st = _lib.i64x3(sb, D, ss)
+    base = qkv.data_ptr()
+    esz = 2
+    return _attn_launch(base, base + Dm * esz, base + 2 * Dm * esz, out, st, st, st, _lib.i64x3(out.stride(0), D, out.stride(1)),
+                        B, n_heads, S, D, dt, dev, lut, block_m, block_n, softmax_scale, launch_form, False, use_plan)
 
 
 class Block_Attn_Mask(Function):

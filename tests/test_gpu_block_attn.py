@@ -224,21 +224,6 @@ def test_long_sequence_walks_several_column_windows():
     _close(got, _oracle(q, k, v, mask.float()), "S 8192, 8 heads")
 
 
-@pytest.mark.parametrize("bm,bn", [(16, 16), (32, 32), (128, 128), (32, 64), (64, 16), (128, 32)])
-def test_other_lut_block_sizes(bm, bn):
-    """LUTs built with the reference's other BLOCK_M / BLOCK_N values describe the same mask and
-    give the same result (they are re-tiled to 64 x 64 on the host)."""
-    S = 512
-    g = torch.Generator().manual_seed(bm * 1000 + bn)
-    mask = configs.mask_c1(S).float()
-    mask[200:330, 350:480] = (torch.rand(130, 130, generator=g) < 0.5).float()   # ragged patch of partial tiles
-    q, k, v = _inputs(2, 3, S, seed=11)
-    want = _oracle(q, k, v, mask)
-    lut = pm.get_sparse_storage(mask[None].cuda(), bm, bn)
-    _close(block_attn(q, k, v, lut[1:], bm, bn), want, f"block {bm}x{bn}")
-    _close(block_attn_mask_op(q.clone(), k, v, *lut[1:], bm, bn, 4), want, f"op, block {bm}x{bn}")
-
-
 def test_large_logits_no_overflow():
     """|score| of several hundred: the max-subtracted softmax must stay finite."""
     q, k, v = _inputs(1, 2, 256, seed=6, scale=6.0)
