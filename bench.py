@@ -67,6 +67,31 @@ def attn_setup(cfg, mask_fn, device):
 
 
 SETTLE_MS = 80.0   # the GPU's clocks take tens of ms of load to settle (first launches run ~25 % slower)
+FLOP_PER_CLK_PER_CU = 4096    # dense fp16 MFMA: 4 SIMDs x 1024 FLOP per clock (32x32x16 in 32 clocks)
+
+
+class ClockProbe:
+    """Shader clock under load, measured in the run: the library's one-wave probe kernel
+    (stof_probe_clock: shader cycle counter against the constant 100 MHz counter) launched on a
+    second stream while the timed kernels run on the first."""
+
+    def __init__(self):
+        from stof import _lib
+        self.lib = _lib.lib()
+        self.out = torch.zeros(3, dtype=torch.int64, device="cuda")
+        self.side = torch.cuda.Stream()
+        self.samples = []
+
+    def sample(self, iters=2000):
+        self.lib.stof_probe_clock(self.out.data_ptr(), iters, self.side.cuda_stream)
+        self.side.synchronize()
+        cycles, ticks, _ = self.out.tolist()
+        if ticks > 0:
+            self.samples.append(cycles / ticks * 0.1)
+
+    def ghz(self):
+        s = sorted(self.samples)
+        return s[len(s) // 2] if s else None
 
 
 def time_region(fn, steps, warmup, settle_ms=SETTLE_MS):
@@ -94,16 +119,46 @@ def time_region(fn, steps, warmup, settle_ms=SETTLE_MS):
     return (t1 - t0) * 1e3 / steps, e0.elapsed_time(e1) / steps
 
 
-def bench_attn(cfg, mask_fn, steps, warmup, settle_ms=SETTLE_MS, launch_form=None, dtype=torch.float16):
+def bench_attn(cfg, mask_fn, steps, warmup, settle_ms=SETTLE_MS, launch_form=None, dtype=torch.float16, probe=None):
     from stof.ops import block_attn
     q, k, v, lut, n_active, _ = attn_setup(cfg, mask_fn, "cuda")
     q, k, v = (t.to(dtype) for t in (q, k, v))
     out = torch.empty_like(q)
-    block_attn(q, k, v, lut, out=out, launch_form=launch_form)          # packs the partial-block bit masks once
+    block_attn(q, k, v, lut, out=out, launch_form=launch_form)          # packs the partial-block bit masks and lays out the walk once
     wall_ms, ev_ms = time_region(lambda: block_attn(q, k, v, lut, out=out, launch_form=launch_form), steps, warmup, settle_ms)
     flop = FLOP_PER_BLOCK * cfg.batch * cfg.heads * n_active
-    return {"wall_ms": wall_ms, "kernel_ms": ev_ms, "flop": flop, "active_blocks": n_active,
-            "tflops_wall": flop / wall_ms / 1e9, "tflops_kernel": flop / ev_ms / 1e9}
+    r = {"wall_ms": wall_ms, "kernel_ms": ev_ms, "flop": flop, "active_blocks": n_active,
+         "tflops_wall": flop / wall_ms / 1e9, "tflops_kernel": flop / ev_ms / 1e9}
+    if probe is not None:
+        # the clock the chip holds under this very load: right after the timed region, with the same
+        # launches still queued on the first stream, the probe runs on the second
+        for _ in range(8):
+            for _ in range(200):
+                block_attn(q, k, v, lut, out=out, launch_form=launch_form)
+            probe.sample()
+        torch.cuda.synchronize()
+    return r
+
+
+def host_cost_us(n=2000):
+    """Host time of one block_attn call (Python operator + binding + hipLaunchKernel): a loop of
+    launches of the small C1 problem with the clock stopped BEFORE the device is waited for."""
+    from stof import _lib, configs
+    from stof.ops import block_attn
+    q, k, v, lut, _, _ = attn_setup(configs.AttnConfig("C1", 1, 12, 512), configs.mask_c1, "cuda")
+    out = torch.empty_like(q)
+    for _ in range(200):
+        block_attn(q, k, v, lut, out=out)
+    torch.cuda.synchronize()
+    best = None
+    for _ in range(3):
+        t0 = time.perf_counter()
+        for _ in range(n):
+            block_attn(q, k, v, lut, out=out)
+        dt = (time.perf_counter() - t0) / n * 1e6
+        torch.cuda.synchronize()
+        best = dt if best is None else min(best, dt)
+    return {"block_attn_host_us_per_call": best, "binding": _lib.binding_name()}
 
 
 def cpu_baseline_attn(cfg, mask_fn, n_active, budget_s=12.0, max_iters=20, min_iters=3):
@@ -298,7 +353,8 @@ def bench_hbm_kernels(steps, warmup):
         b = torch.randn(N, generator=g).half().cuda()
         _, ev = time_region(lambda: fused.bias_residual_layernorm(x, b, r, b, b, 1e-12), steps, warmup)
         nbytes = 3 * M * N * 2
-        out[tag] = {"ms": ev, "GBs": nbytes / ev / 1e6, "frac_hbm": nbytes / ev / 1e6 / PEAK_HBM_GBS, "shape": [M, N]}
+        out[tag] = {"ms": ev, "GBs": nbytes / ev / 1e6, "frac_hbm": nbytes / ev / 1e6 / PEAK_HBM_GBS, "shape": [M, N],
+                    "copy_same_bytes": same_size_copy(nbytes)}
         del x, r
     # what a plain device copy reaches on this machine (read + write of 256 MiB each way)
     src = torch.empty(256 << 20, dtype=torch.uint8, device="cuda").fill_(1)
@@ -312,8 +368,18 @@ def bench_hbm_kernels(steps, warmup):
     _, ev2 = time_region(lambda: pack_mask_bits(m, additive=False), steps, warmup)
     pk_bytes = S * S * 2 + S * S // 8
     out["pack_mask_bits"] = {"ms": ev2, "GBs": pk_bytes / ev2 / 1e6, "frac_hbm": pk_bytes / ev2 / 1e6 / PEAK_HBM_GBS,
-                             "shape": [S, S]}
+                             "shape": [S, S], "copy_same_bytes": same_size_copy(pk_bytes)}
     return out
+
+
+def same_size_copy(nbytes):
+    """A plain device copy moving the same number of bytes (half read, half written) as an
+    HBM-bound kernel: what the machine gives at that size, launch ramp included."""
+    half = max(int(nbytes) // 2, 16)
+    src = torch.empty(half, dtype=torch.uint8, device="cuda").fill_(1)
+    dst = torch.empty_like(src)
+    _, ev = time_region(lambda: dst.copy_(src), 200, 20)
+    return {"ms": ev, "GBs": 2 * half / ev / 1e6, "frac_hbm": 2 * half / ev / 1e6 / PEAK_HBM_GBS, "bytes": 2 * half}
 
 
 def bench_lut_build(with_cpu, steps=200):
@@ -351,6 +417,7 @@ def bench_lut_build(with_cpu, steps=200):
         out[f"kernels_ms_S4096_{tag}"] = ev
         out[f"kernels_GBs_{tag}"] = nbytes / ev / 1e6
         out[f"kernels_frac_hbm_{tag}"] = nbytes / ev / 1e6 / PEAK_HBM_GBS
+        out[f"copy_same_bytes_{tag}"] = same_size_copy(nbytes)
     out["gpu_ms_S4096"] = out["kernels_ms_S4096_fp16"]
     if with_cpu:
         from oracle import masks as om
@@ -368,7 +435,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=2000,
                     help="untimed steps before the timed ones; the default (about 70 ms of load) lets the clocks settle")
     ap.add_argument("--no-extras", action="store_true", help="skip everything but the C4 attention step")
-    ap.add_argument("--extras", default="c1,c2,c4big,forms,dense,c3,c3small,c5,hbm,lut",
+    ap.add_argument("--extras", default="c1,c2,c5attn,c4big,forms,dense,c3,c3small,c5,hbm,lut",
                     help="comma-separated subset of the extra workloads to run (for profiling one kind of kernel)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--copy-probe", action="store_true",
@@ -390,7 +457,11 @@ def main():
         dst = torch.empty_like(src)
         dst.copy_(src)
         torch.cuda.synchronize()
-    c4 = bench_attn(configs.C4, configs.mask_c4, args.steps, args.warmup, settle_ms=0)   # exactly W warm-up steps, then K timed
+    from stof import _lib
+    probe = ClockProbe()
+    cus = _lib.lib().stof_device_compute_units()
+    c4 = bench_attn(configs.C4, configs.mask_c4, args.steps, args.warmup, settle_ms=0, probe=probe)   # exactly W warm-up steps, then K timed
+    clock = probe.ghz()
     traffic, traffic_source = measured_traffic()
     line = {
         "metric": "masked-MHA TFLOP/s (active blocks) + encoder-layer ms, fp16, 1xMI355X",
@@ -404,17 +475,28 @@ def main():
         "roofline": {"bound": "mfma", "achieved": c4["tflops_kernel"], "peak": PEAK_FP16_TFLOPS, "unit": "TFLOP/s",
                      "frac": c4["tflops_kernel"] / PEAK_FP16_TFLOPS, "traffic": traffic, "traffic_source": traffic_source,
                      "algorithmic_bytes": 4 * configs.C4.batch * configs.C4.heads * configs.C4.seq * 64 * 2,
-                     "kernel": "block_attn_fwd_kernel", "kernel_ms": c4["kernel_ms"]},
+                     "kernel": "block_attn_fwd_kernel", "kernel_ms": c4["kernel_ms"],
+                     # what was measured on this box in this run, next to the published peak the fraction divides by:
+                     # compute units (hipDeviceGetAttribute) and the shader clock under the timed load (the library's
+                     # probe kernel on a second stream: shader cycle counter against the 100 MHz counter, median of 8)
+                     "cu_count": cus, "clock_ghz_under_load": clock,
+                     "peak_at_measured_clock": (cus * FLOP_PER_CLK_PER_CU * clock / 1e3) if clock else None,
+                     "frac_at_measured_clock": (c4["tflops_kernel"] / (cus * FLOP_PER_CLK_PER_CU * clock / 1e3)) if clock else None},
     }
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline_attn(configs.C4, configs.mask_c4, c4["active_blocks"])
     if not args.no_extras:
         also = {}
         want = set(args.extras.split(","))
+        also["host"] = host_cost_us()
         if "c2" in want:
             c2 = bench_attn(configs.C2, configs.mask_c2, args.steps, args.warmup)
             also["C2_mha_S1024"] = {"tflops": c2["tflops_kernel"], "frac_mfma_peak": c2["tflops_kernel"] / PEAK_FP16_TFLOPS,
                                     "kernel_ms": c2["kernel_ms"], "active_blocks": c2["active_blocks"]}
+        if "c5attn" in want:
+            c5a = bench_attn(configs.AttnConfig("C5-attention", 4, 16, 2048), configs.mask_c5, args.steps, args.warmup)
+            also["C5_attention_B4_H16_S2048"] = {"tflops": c5a["tflops_kernel"], "frac_mfma_peak": c5a["tflops_kernel"] / PEAK_FP16_TFLOPS,
+                                                 "kernel_ms": c5a["kernel_ms"], "active_blocks": c5a["active_blocks"]}
         if "c4big" in want:
             big = configs.AttnConfig("C4x8", 16, 16, 4096)
             c4b = bench_attn(big, configs.mask_c4, max(args.steps // 4, 10), 5)

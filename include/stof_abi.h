@@ -210,11 +210,16 @@ int stof_rowwise_attn_fwd(
  *   counts[4] (optional): {entries in FULL, PART, LOAD; 1 if a capacity was too small (the lists are
  *   then truncated, the row pointers still exact)}.
  * workspace: stof_build_lut_workspace_bytes() bytes of device memory, 8-byte aligned, used as
- * scratch for the duration of the call (one class byte per tile, 512 B of bit rows per tile).
+ * scratch for the duration of the call (one class byte per tile, 512 B of bit rows per 64 x 64 tile, a
+ * 2-byte count per tile and, in its last 16 bytes, the mask's non-zero count: stof_build_lut_nnz_offset).
  * block_m, block_n in {16, 32, 64, 128} dividing seq_len; mask 16-byte aligned, ld * elem_bytes
  * a multiple of 16.  HBM-bound: seq_len^2 * elem_bytes bytes read once.
  */
 int64_t stof_build_lut_workspace_bytes(int seq_len, int block_m, int block_n);
+/* Byte offset inside that workspace at which a call of stof_build_lut leaves the number of non-zero
+ * mask elements as an int64 (the reference's nnz figure, src/util/masks.py:137, counted in the same
+ * pass as the classification); the last 16 bytes of the workspace. */
+int64_t stof_build_lut_nnz_offset(int seq_len, int block_m, int block_n);
 int stof_build_lut(const void* mask, int elem_bytes, int64_t ld, int seq_len, int block_m, int block_n,
                    int32_t* full_row_ptr, int32_t* full_col_idx,
                    int32_t* part_row_ptr, int32_t* part_col_idx,
@@ -408,6 +413,18 @@ int stof_gemm_bias_res_ln_cluster_dt(const void* A, const void* Wt, const void* 
                                      const void* gamma, const void* beta, void* C,
                                      int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldr, int64_t ldc,
                                      float eps, void* workspace, int64_t workspace_bytes, int dtype, void* stream);
+
+/*
+ * Measurement probes (no counterpart in the reference; used by bench.py, not by any operator).
+ * stof_device_compute_units: compute units of the current device (hipDeviceAttributeMultiprocessorCount),
+ * or a negative status.  stof_probe_clock: one wavefront spins for `iters` x 16 dependent adds between
+ * two readings of the shader cycle counter and of the constant 100 MHz counter and writes
+ * {shader cycles, 10 ns ticks, scratch} to out3 (device memory, three 8-byte words): shader clock =
+ * out3[0] / out3[1] * 100 MHz.  Launched on a second stream while other kernels run, it reads the
+ * clock the chip holds under that load.
+ */
+int stof_device_compute_units(void);
+int stof_probe_clock(unsigned long long* out3, int iters, void* stream);
 
 #ifdef __cplusplus
 }

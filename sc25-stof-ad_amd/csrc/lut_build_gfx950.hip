@@ -28,7 +28,8 @@
 constexpr int64_t kStaticMaxTiles = 16384;   // S = 8192 at 64 x 64 blocks
 constexpr int64_t kClsBytesStatic = kStaticMaxTiles;
 constexpr int64_t kBitsBytesStatic = kStaticMaxTiles * 64 * 8;
-static __device__ __align__(256) unsigned char scratch[kClsBytesStatic + kBitsBytesStatic];
+constexpr int64_t kCntBytesStatic = kStaticMaxTiles * 2 + 16;   // non-zero count per tile, then the total (see LutParams)
+static __device__ __align__(256) unsigned char scratch[kClsBytesStatic + kBitsBytesStatic + kCntBytesStatic];
 
 namespace {
 
@@ -38,6 +39,7 @@ struct LutParams {
   const void* mask; int64_t ld;           // row pitch in elements
   int S, bm, bn, nQ, nK;
   unsigned char* cls; uint64_t* ws_bits;  // scratch: class byte per tile; 64 bit rows per tile (64 x 64 only, else null)
+  unsigned short* cnt; long long* nnz;    // scratch: non-zero elements per tile (or null); their sum, written by the last row's workgroup
   int32_t* frp; int32_t* fci; int32_t* prp; int32_t* pci; int32_t* lrp; int32_t* lci;
   uint64_t* pbits;                        // [cap_part][64] or null
   int32_t* counts;                        // {n_full, n_part, n_load, overflow} or null
@@ -49,44 +51,53 @@ __device__ __forceinline__ half_t additive_of(half_t x) {
   return (half_t)-10000.0f * ((half_t)1.0f - x);
 }
 
-// One 16-byte chunk of a tile row: updates the two "every element is ..." votes and returns the
-// chunk's keep bits (bit e = element e allowed, by the rule the bit rows are packed with
-// elsewhere: additive value above -5000).
+// Eight consecutive elements of a tile row (one 16-byte load of fp16, two of fp32, both requested
+// before the first compare): updates the two "every element is ..." votes and returns the keep
+// bits (bit e = element e allowed, by the rule the bit rows are packed with elsewhere: additive
+// value above -5000).
 template <typename T>
-__device__ __forceinline__ uint32_t chunk_bits(const T* src, bool& not_one, bool& not_zero) {
-  constexpr int E = 16 / (int)sizeof(T);
+__device__ __forceinline__ uint32_t chunk_bits(const T* src, bool& not_one, bool& not_zero, int& nonzero) {
+  constexpr int E = 16 / (int)sizeof(T);      // elements per 16-byte load
+  constexpr int L = 8 / E;                    // loads per eight elements
   typedef T vec_t __attribute__((ext_vector_type(E)));
-  const vec_t x = *reinterpret_cast<const vec_t*>(src);
+  vec_t x[L];
+#pragma unroll
+  for (int l = 0; l < L; ++l) x[l] = *reinterpret_cast<const vec_t*>(src + l * E);
   uint32_t cb = 0;
 #pragma unroll
-  for (int e = 0; e < E; ++e) {
-    const float f = (float)x[e];
-    not_one |= f != 1.0f;
-    not_zero |= f != 0.0f;
-    cb |= (uint32_t)((float)additive_of((half_t)x[e]) > -5000.0f) << e;
-  }
+  for (int l = 0; l < L; ++l)
+#pragma unroll
+    for (int e = 0; e < E; ++e) {
+      const float f = (float)x[l][e];
+      not_one |= f != 1.0f;
+      not_zero |= f != 0.0f;
+      nonzero += f != 0.0f;
+      cb |= (uint32_t)((float)additive_of((half_t)x[l][e]) > -5000.0f) << (l * E + e);
+    }
   return cb;
 }
 
-// T = half_t or float; E elements per 16-byte chunk.  One wavefront per tile.
+// T = half_t or float.  One wavefront per tile; a lane takes eight elements (one byte of a bit row) at a time.
 template <typename T>
 __global__ __launch_bounds__(256) void lut_classify_kernel(const LutParams p) {
-  constexpr int E = 16 / (int)sizeof(T);
   const int lane = threadIdx.x & 63;
   const int64_t tile = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
   if (tile >= (int64_t)p.nQ * p.nK) return;
   const int r = (int)(tile / p.nK), c = (int)(tile - (int64_t)r * p.nK);
   const T* base = reinterpret_cast<const T*>(p.mask) + (int64_t)r * p.bm * p.ld + (int64_t)c * p.bn;
   bool not_one = false, not_zero = false;
+  int nonzero = 0;   // this lane's share of the tile's non-zero elements (summed over the wave at the end)
   if (p.ws_bits) {
-    // 64 x 64 tile: CPR lanes hold one row of 64 keys, a pass covers 64 / CPR rows, 64 / E passes
-    constexpr int CPR = 64 / E, PASSES = 64 / E, ROWS = 64 / CPR;
+    // 64 x 64 tile: 8 lanes hold one row of 64 keys, a pass covers 8 rows, 8 passes.  (fp32 read
+    // four elements per lane at first: twice the passes and lane exchanges for the same bytes,
+    // and a larger mask ran slower per byte than the fp16 one.)
+    constexpr int CPR = 8, PASSES = 8, ROWS = 8;
     const int ch = lane & (CPR - 1), row_in_pass = lane / CPR;
     uint64_t words[PASSES];   // lanes with chunk 0: the bit row of (pass, row_in_pass)
 #pragma unroll
     for (int ps = 0; ps < PASSES; ++ps) {
-      const uint32_t cb = chunk_bits<T>(base + (int64_t)(ps * ROWS + row_in_pass) * p.ld + ch * E, not_one, not_zero);
-      const int sh = ch * E;
+      const uint32_t cb = chunk_bits<T>(base + (int64_t)(ps * ROWS + row_in_pass) * p.ld + ch * 8, not_one, not_zero, nonzero);
+      const int sh = ch * 8;
       uint32_t lo = sh < 32 ? cb << sh : 0u, hi = sh >= 32 ? cb << (sh - 32) : 0u;
 #pragma unroll
       for (int m = 1; m < CPR; m <<= 1) {
@@ -102,14 +113,18 @@ __global__ __launch_bounds__(256) void lut_classify_kernel(const LutParams p) {
       for (int ps = 0; ps < PASSES; ++ps) p.ws_bits[tile * 64 + ps * ROWS + row_in_pass] = words[ps];
     }
   } else {
-    const int cpr = p.bn / E;                 // 16-byte chunks per tile row
+    const int cpr = p.bn / 8;                 // eight-element chunks per tile row
     const int total = p.bm * cpr;
     for (int idx = lane; idx < total; idx += 64) {
       const int row = idx / cpr, ch = idx - row * cpr;
-      chunk_bits<T>(base + (int64_t)row * p.ld + ch * E, not_one, not_zero);
+      chunk_bits<T>(base + (int64_t)row * p.ld + ch * 8, not_one, not_zero, nonzero);
     }
     const bool full = __ballot(not_one) == 0ull, empty = __ballot(not_zero) == 0ull;
     if (lane == 0) p.cls[tile] = (unsigned char)(empty ? kClsEmpty : (full ? kClsFull : kClsPart));
+  }
+  if (p.cnt) {   // (at most 128 x 128 = 16384 per tile)
+    for (int o = 32; o > 0; o >>= 1) nonzero += __shfl_xor(nonzero, o, 64);
+    if (lane == 0) p.cnt[tile] = (unsigned short)nonzero;
   }
 }
 
@@ -177,6 +192,26 @@ __global__ __launch_bounds__(256) void lut_compact_kernel(const LutParams p) {
     }
     fbase += f_all; pbase += p_all;
     __syncthreads();
+  }
+  if (r == p.nQ - 1 && p.cnt && p.nnz) {
+    // the mask's non-zero elements: the per-tile counts of the classify pass, summed by this one workgroup
+    long long total = 0;
+    const int64_t tiles = (int64_t)p.nQ * p.nK;
+    // eight counts per 16-byte load (the count array starts 16-byte aligned), all of a thread's loads independent
+    typedef unsigned short ushort8v __attribute__((ext_vector_type(8)));
+    const int64_t vecs = tiles >> 3;
+    for (int64_t i = tid; i < vecs; i += 256) {
+      const ushort8v c8 = *reinterpret_cast<const ushort8v*>(p.cnt + 8 * i);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) total += c8[e];
+    }
+    for (int64_t i = 8 * vecs + tid; i < tiles; i += 256) total += p.cnt[i];
+    for (int o = 32; o > 0; o >>= 1) total += __shfl_xor(total, o, 64);
+    __shared__ long long part_sum[4];
+    __syncthreads();
+    if (lane == 0) part_sum[wave] = total;
+    __syncthreads();
+    if (tid == 0) *p.nnz = part_sum[0] + part_sum[1] + part_sum[2] + part_sum[3];
   }
   if (tid == 0) {
     if (r == 0) { p.frp[0] = 0; p.prp[0] = 0; p.lrp[0] = 0; }
@@ -280,6 +315,11 @@ int static_scratch(unsigned char** out) {
 
 bool block_ok(int b) { return b == 16 || b == 32 || b == 64 || b == 128; }
 
+// Workspace layout: class bytes | bit rows (64 x 64 blocks only) | non-zero count per tile (2 bytes) | total (8 bytes + 8 spare)
+int64_t ws_cnt_offset(int64_t tiles, int block_m, int block_n) {
+  return (tiles + 255) / 256 * 256 + ((block_m == 64 && block_n == 64) ? tiles * 64 * 8 : 0);
+}
+
 int check_common(const void* mask, int elem_bytes, int64_t ld, int seq_len, int block_m, int block_n) {
   if (!mask) return STOF_ERR_NULL_POINTER;
   if (elem_bytes != 2 && elem_bytes != 4) return STOF_ERR_UNSUPPORTED;
@@ -292,8 +332,9 @@ int check_common(const void* mask, int elem_bytes, int64_t ld, int seq_len, int 
 int build(const void* mask, int elem_bytes, int64_t ld, int seq_len, int block_m, int block_n,
           int32_t* frp, int32_t* fci, int32_t* prp, int32_t* pci, int32_t* lrp, int32_t* lci,
           uint64_t* part_bitmask, int32_t* counts, int64_t cap_full, int64_t cap_part, int64_t cap_load,
-          unsigned char* cls, uint64_t* ws_bits, hipStream_t stream) {
+          unsigned char* cls, uint64_t* ws_bits, unsigned short* cnt, long long* nnz, hipStream_t stream) {
   LutParams p;
+  p.cnt = cnt; p.nnz = nnz;
   p.mask = mask; p.ld = ld; p.S = seq_len; p.bm = block_m; p.bn = block_n;
   p.nQ = seq_len / block_m; p.nK = seq_len / block_n;
   p.cls = cls; p.ws_bits = (block_m == 64 && block_n == 64 && part_bitmask) ? ws_bits : nullptr;
@@ -323,8 +364,12 @@ int check_outputs(const int32_t* frp, const int32_t* fci, const int32_t* prp, co
 extern "C" int64_t stof_build_lut_workspace_bytes(int seq_len, int block_m, int block_n) {
   if (seq_len <= 0 || !block_ok(block_m) || !block_ok(block_n) || seq_len % block_m || seq_len % block_n) return STOF_ERR_BAD_SHAPE;
   const int64_t tiles = (int64_t)(seq_len / block_m) * (seq_len / block_n);
-  const int64_t cls = (tiles + 255) / 256 * 256;
-  return cls + ((block_m == 64 && block_n == 64) ? tiles * 64 * 8 : 0);
+  return ws_cnt_offset(tiles, block_m, block_n) + (tiles * 2 + 15) / 16 * 16 + 16;
+}
+
+extern "C" int64_t stof_build_lut_nnz_offset(int seq_len, int block_m, int block_n) {
+  const int64_t total = stof_build_lut_workspace_bytes(seq_len, block_m, block_n);
+  return total < 0 ? total : total - 16;
 }
 
 extern "C" int stof_build_lut(const void* mask, int elem_bytes, int64_t ld, int seq_len, int block_m, int block_n,
@@ -345,8 +390,10 @@ extern "C" int stof_build_lut(const void* mask, int elem_bytes, int64_t ld, int 
   const int64_t tiles = (int64_t)(seq_len / block_m) * (seq_len / block_n);
   unsigned char* cls = static_cast<unsigned char*>(workspace);
   uint64_t* bits = reinterpret_cast<uint64_t*>(cls + (tiles + 255) / 256 * 256);
+  unsigned short* cnt = reinterpret_cast<unsigned short*>(cls + ws_cnt_offset(tiles, block_m, block_n));
+  long long* nnz = reinterpret_cast<long long*>(cls + stof_build_lut_nnz_offset(seq_len, block_m, block_n));
   return build(mask, elem_bytes, ld, seq_len, block_m, block_n, full_row_ptr, full_col_idx, part_row_ptr, part_col_idx,
-               load_row_ptr, load_col_idx, part_bitmask, counts, cap_full, cap_part, cap_load, cls, bits, (hipStream_t)stream);
+               load_row_ptr, load_col_idx, part_bitmask, counts, cap_full, cap_part, cap_load, cls, bits, cnt, nnz, (hipStream_t)stream);
 }
 
 extern "C" int stof_retile_lut(const int32_t* full_row_ptr, const int32_t* full_col_idx,
@@ -378,7 +425,7 @@ extern "C" int stof_retile_lut(const int32_t* full_row_ptr, const int32_t* full_
   hipLaunchKernelGGL(lut_retile_kernel, dim3((unsigned)((tiles + 3) / 4)), dim3(256), 0, (hipStream_t)stream, r);
   LutParams p;
   p.mask = nullptr; p.ld = 0; p.S = seq_len; p.bm = 64; p.bn = 64; p.nQ = n64; p.nK = n64;
-  p.cls = r.cls; p.ws_bits = r.ws_bits;
+  p.cls = r.cls; p.ws_bits = r.ws_bits; p.cnt = nullptr; p.nnz = nullptr;
   p.frp = out_full_row_ptr; p.fci = out_full_col_idx; p.prp = out_part_row_ptr; p.pci = out_part_col_idx;
   p.lrp = out_load_row_ptr; p.lci = out_load_col_idx; p.pbits = out_part_bitmask; p.counts = counts;
   p.cap_full = cap_full; p.cap_part = cap_part; p.cap_load = cap_load;
@@ -406,7 +453,9 @@ extern "C" int stof_build_lut_static(const void* mask, int elem_bytes, int64_t l
   if (rc != STOF_OK) return rc;
   return build(mask, elem_bytes, ld, seq_len, block_m, block_n, full_row_ptr, full_col_idx, part_row_ptr, part_col_idx,
                load_row_ptr, load_col_idx, part_bitmask, counts, cap_full, cap_part, cap_load,
-               ptr, reinterpret_cast<uint64_t*>(ptr + kClsBytesStatic), (hipStream_t)stream);
+               ptr, reinterpret_cast<uint64_t*>(ptr + kClsBytesStatic),
+               reinterpret_cast<unsigned short*>(ptr + kClsBytesStatic + kBitsBytesStatic),
+               reinterpret_cast<long long*>(ptr + kClsBytesStatic + kBitsBytesStatic + kStaticMaxTiles * 2), (hipStream_t)stream);
 }
 
 extern "C" int stof_lut_additive_blocks(const void* mask, int elem_bytes, int64_t ld, int seq_len, int block_m, int block_n,

@@ -46,6 +46,8 @@ auto wrap(R (*f)(A...)) {
 PYBIND11_MODULE(_stof_ext, m) {
   m.doc() = "pybind11 binding of libstof_hip.so (C ABI of include/stof_abi.h); pointers and streams are ints";
   STOF_BIND(stof_abi_version);
+  STOF_BIND(stof_device_compute_units);
+  STOF_BIND(stof_probe_clock);
   m.def("stof_status_string", [](int status) { return py::bytes(stof_status_string(status)); });
   STOF_BIND(stof_block_attn_fwd);
   STOF_BIND(stof_block_attn_fwd_planned);
@@ -55,6 +57,7 @@ PYBIND11_MODULE(_stof_ext, m) {
   STOF_BIND(stof_pack_mask_bits);
   STOF_BIND(stof_rowwise_attn_fwd);
   STOF_BIND(stof_build_lut_workspace_bytes);
+  STOF_BIND(stof_build_lut_nnz_offset);
   STOF_BIND(stof_build_lut);
   STOF_BIND(stof_retile_lut);
   STOF_BIND(stof_build_lut_static_max_tiles);

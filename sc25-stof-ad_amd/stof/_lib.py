@@ -24,6 +24,8 @@ _P = c_void_p
 _I64x3 = c_int64 * 3
 
 _SIGNATURES = {
+    "stof_device_compute_units": (c_int, []),
+    "stof_probe_clock": (c_int, [_P, c_int, _P]),
     "stof_abi_version": (c_int, []),
     "stof_status_string": (c_char_p, [c_int]),
     "stof_block_attn_fwd": (c_int, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P,
@@ -41,6 +43,7 @@ _SIGNATURES = {
     "stof_rowwise_attn_fwd": (c_int, [_P, _P, _P, _P, c_int, c_int, c_int, _P,
                                       c_int, c_int, c_int, c_int, c_int, c_int, _P]),
     "stof_build_lut_workspace_bytes": (c_int64, [c_int, c_int, c_int]),
+    "stof_build_lut_nnz_offset": (c_int64, [c_int, c_int, c_int]),
     "stof_build_lut": (c_int, [_P, c_int, c_int64, c_int, c_int, c_int, _P, _P, _P, _P, _P, _P, _P, _P,
                                c_int64, c_int64, c_int64, _P, c_int64, _P]),
     "stof_retile_lut": (c_int, [_P, _P, _P, _P, _P, c_int, c_int, c_int, _P, _P, _P, _P, _P, _P, _P, _P,

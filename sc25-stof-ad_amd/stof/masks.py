@@ -152,18 +152,29 @@ def _build_on_device(m2d, bm, bn, want_bits):
     nq, nk = n // bm, n // bn
     tiles = nq * nk
     dev = m2d.device
-    i32 = lambda k: torch.empty(k, dtype=torch.int32, device=dev)
-    frp, prp, lrp = i32(nq + 1), i32(nq + 1), i32(nq + 1)
-    fci, pci, lci = i32(tiles), i32(tiles), i32(tiles)
-    counts = i32(4)
+    # one allocation for the six index arrays (each part 16-byte aligned)
+    rp = (nq + 1 + 3) & ~3
+    idx = torch.empty(3 * rp + 3 * tiles, dtype=torch.int32, device=dev)
+    frp, prp, lrp = idx[0:nq + 1], idx[rp:rp + nq + 1], idx[2 * rp:2 * rp + nq + 1]
+    fci, pci, lci = (idx[3 * rp + i * tiles:3 * rp + (i + 1) * tiles] for i in range(3))
     bits = torch.empty((tiles, 64), dtype=torch.int64, device=dev) if (want_bits and bm == 64 and bn == 64) else None
     lib = _lib.lib()
-    ws = torch.empty(lib.stof_build_lut_workspace_bytes(n, bm, bn), dtype=torch.uint8, device=dev)
+    # The workspace ends with the mask's non-zero count (8 bytes + 8 spare); the four list counts are
+    # placed right behind it, so that one device -> host read of 32 bytes brings all of them.
+    wbytes = lib.stof_build_lut_workspace_bytes(n, bm, bn)
+    ws = torch.empty(wbytes + 16, dtype=torch.uint8, device=dev)
+    counts = ws[wbytes - 16:].view(torch.int64)          # [nnz, spare, n_full | n_part << 32, n_load | overflow << 32]
     _lib.check(lib.stof_build_lut(m2d.data_ptr(), m2d.element_size(), m2d.stride(0), n, bm, bn,
                                   frp.data_ptr(), fci.data_ptr(), prp.data_ptr(), pci.data_ptr(), lrp.data_ptr(), lci.data_ptr(),
-                                  bits.data_ptr() if bits is not None else None, counts.data_ptr(),
-                                  tiles, tiles, tiles, ws.data_ptr(), ws.numel(), _stream(dev)), "stof_build_lut")
+                                  bits.data_ptr() if bits is not None else None, ws.data_ptr() + wbytes,
+                                  tiles, tiles, tiles, ws.data_ptr(), wbytes, _stream(dev)), "stof_build_lut")
     return m2d, frp, fci, prp, pci, lrp, lci, bits, counts
+
+
+def _read_counts(counts):
+    """(non-zero elements, n_full, n_part, n_load, overflow) from the 32 bytes behind the workspace: one read."""
+    nnz, _, a, b = counts.tolist()
+    return nnz, a & 0xFFFFFFFF, (a >> 32) & 0xFFFFFFFF, b & 0xFFFFFFFF, (b >> 32) & 0xFFFFFFFF
 
 
 def _get_sparse_storage_device(m2d, bm, bn):
@@ -173,7 +184,7 @@ def _get_sparse_storage_device(m2d, bm, bn):
     from ._cache import BITS_ATTR, content_key
     from .ops import _stream
     m2d, frp, fci, prp, pci, lrp, lci, bits, counts = _build_on_device(m2d, bm, bn, want_bits=True)
-    n_full, n_part, n_load, overflow = counts.tolist()
+    nonzero, n_full, n_part, n_load, overflow = _read_counts(counts)
     assert not overflow
     n = m2d.shape[-1]
     fci, pci, lci = fci[:n_full], pci[:n_part], lci[:n_load]
@@ -186,7 +197,7 @@ def _get_sparse_storage_device(m2d, bm, bn):
                                                        _stream(m2d.device)), "stof_lut_additive_blocks")
         if bits is not None:   # the attention operator finds the bit rows of these blocks already packed
             setattr(pbm, BITS_ATTR, (content_key(pbm), bits[:n_part]))
-    return frp, fci, prp, pci, pbm, lrp, lci
+    return nonzero, (frp, fci, prp, pci, pbm, lrp, lci)
 
 
 def get_sparse_storage(Mask, block_size_m, block_size_n):
@@ -203,9 +214,17 @@ def get_sparse_storage(Mask, block_size_m, block_size_n):
     Both give the same tensors bit for bit.
     """
     n = Mask.shape[-1]
-    nnz = torch.count_nonzero(Mask) / (n * n) * 100
     if _device_path(Mask, block_size_m, block_size_n):
-        return (nnz,) + _get_sparse_storage_device(Mask[0], block_size_m, block_size_n)
+        # the non-zero count of batch 0 comes out of the classification pass; further batches (which the
+        # LUT ignores, but the reference's figure counts) are counted by torch
+        nonzero, lut = _get_sparse_storage_device(Mask[0], block_size_m, block_size_n)
+        if Mask.shape[0] > 1:
+            nonzero += int(torch.count_nonzero(Mask[1:]))
+        import numpy as np
+        # (the reference's arithmetic: an int64 count / int * int in float32, src/util/masks.py:137)
+        nnz = torch.tensor(float(np.float32(nonzero) / np.float32(n * n) * np.float32(100)), device=Mask.device)
+        return (nnz,) + lut
+    nnz = torch.count_nonzero(Mask) / (n * n) * 100
     blocks, full, part = _classify(Mask[0], block_size_m, block_size_n)
     full_row_ptr, full_col_idx = _csr(full)
     part_row_ptr, part_col_idx = _csr(part)
@@ -251,7 +270,7 @@ def get_sparse_storage_batched(Mask, block_size_m, block_size_n):
     on_device = _device_path(Mask, block_size_m, block_size_n)
     for b in range(B):
         if on_device:
-            frp, fci, prp, pci, pbm_b, lrp, lci = _get_sparse_storage_device(Mask[b], block_size_m, block_size_n)
+            _, (frp, fci, prp, pci, pbm_b, lrp, lci) = _get_sparse_storage_device(Mask[b], block_size_m, block_size_n)
         else:
             blocks, full, part = _classify(Mask[b], block_size_m, block_size_n)
             frp, fci = _csr(full); prp, pci = _csr(part); lrp, lci = _csr(full | part)

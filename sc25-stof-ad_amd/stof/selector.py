@@ -60,6 +60,9 @@ class Selection:
     rho: float             # active tiles / tiles of the square
     groups_per_cu: float   # two-row workgroups per compute unit
     reason: str
+    row_kind: str = "full"   # row-wise only: which of the reference's three row-wise operators
+                             # (src/ops/package_op.py:11-48): "full" (dense / causal), "sliding", "mask"
+    bandwidth: int = 0       # row_kind "sliding": the window (keys j > i - bandwidth)
 
     def __str__(self):
         if self.operator == "row-wise":
@@ -123,31 +126,76 @@ def phase2_selection(gpu, seq_len, batch_size, head_num):
     return ("two_rows", per_cu, why)
 
 
-def select_operator(gpu_params, load_row_ptr, batch_size, seq_len, head_num, is_causal=False, lut=None):
+def _sliding_rows(nq, bandwidth, is_causal):
+    """Key blocks per query block that the row-wise sliding operator visits: keys j > i - bandwidth,
+    up to the diagonal block when causal, else to the end of the sequence."""
+    rows = []
+    for r in range(nq):
+        first_key = BLOCK * r - bandwidth + 1
+        lo = first_key // BLOCK if first_key > 0 else 0
+        rows.append((r if is_causal else nq - 1) - lo + 1)
+    return rows
+
+
+def select_operator(gpu_params, load_row_ptr, batch_size, seq_len, head_num, is_causal=False, lut=None,
+                    mask_kind=None, bandwidth=0):
     """Reference: select_operator(gpu_params, load_row_ptr, batch_size, seq_len, head_num),
     benchmk_attn_unified.py:157-163, which returns ``"block-wise warp{w}m{m}n{n}"`` or
     ``"row-wise"``; ``str()`` of the result here has the same two shapes.  Pass the whole
     ``lut`` as well to have "row-wise" returned only when the dense / causal row-wise operator
-    computes exactly the LUT's mask (see ``phase1_decision``)."""
+    computes exactly the LUT's mask (see ``phase1_decision``).
+
+    ``mask_kind`` / ``bandwidth``: what the caller knows about the mask, as the reference's
+    benchmark does by the mask's name: "sliding" with its bandwidth selects the row-wise
+    sliding-window operator when the LUT lists exactly the tiles that window touches;
+    ``load_row_ptr=None`` (no LUT at hand) selects the row-wise operator of the stated kind -
+    "dense" / "causal" (full), "sliding", or "element" (the row-wise mask operator on ``row_mask``).
+    The software-pipelined launch form is never selected: measured level with "two_rows" on grids
+    of many rounds and behind it on single-round grids."""
     if seq_len % BLOCK:
         raise ValueError(f"seq_len ({seq_len}) must be a multiple of {BLOCK}")
+    if mask_kind not in (None, "dense", "causal", "sliding", "element"):
+        raise ValueError(f"mask_kind must be None, 'dense', 'causal', 'sliding' or 'element', got {mask_kind!r}")
     nq = seq_len // BLOCK
-    rho = _active_blocks(load_row_ptr) / float(nq * nq)
     form, per_cu, why = phase2_selection(gpu_params, seq_len, batch_size, head_num)
+    # What the caller knows about the mask (the reference's benchmark knows its mask by name and
+    # calls the matching row-wise operator, src/benchmk_attn_unified.py:396-407).  Every operator runs
+    # on one tile engine here, so a row-wise operator is never faster per tile; it is the choice
+    # where no LUT exists to drive the block-wise one, and where the LUT would list exactly the
+    # tiles the operator's index predicate visits anyway (then it saves building LUT and plan).
+    if load_row_ptr is None:
+        if mask_kind is None:
+            raise ValueError("without a LUT the mask kind must be given ('dense', 'causal', 'sliding' or 'element')")
+        kind = {"dense": "full", "causal": "full", "sliding": "sliding", "element": "mask"}[mask_kind]
+        if kind == "sliding" and bandwidth <= 0:
+            raise ValueError("mask_kind='sliding' needs the bandwidth")
+        return Selection("row-wise", form, BLOCK, BLOCK, float("nan"), per_cu, "no LUT given: row-wise by the stated mask kind; " + why,
+                         row_kind=kind, bandwidth=int(bandwidth))
+    rho = _active_blocks(load_row_ptr) / float(nq * nq)
+    if mask_kind == "sliding" and bandwidth > 0:
+        lrp = load_row_ptr if load_row_ptr.dim() == 1 else (load_row_ptr[0] if load_row_ptr.shape[0] == 1 else None)
+        if lrp is not None and (lrp[1:] - lrp[:-1]).tolist() == _sliding_rows(nq, int(bandwidth), is_causal):
+            return Selection("row-wise", form, BLOCK, BLOCK, rho, per_cu,
+                             "the LUT lists exactly the tiles of the stated sliding window; " + why,
+                             row_kind="sliding", bandwidth=int(bandwidth))
     if phase1_decision(load_row_ptr, seq_len, is_causal, lut=lut):
         return Selection("block-wise", form, BLOCK, BLOCK, rho, per_cu, why)
     return Selection("row-wise", form, BLOCK, BLOCK, rho, per_cu,
                      "the LUT lists nearly every tile the index predicate visits; " + why)
 
 
-def apply(selection, q, k, v, lut=None, is_causal=False, out_layout="bshd"):
+def apply(selection, q, k, v, lut=None, is_causal=False, out_layout="bshd", row_mask=None):
     """Run the selected operator in the selected launch form (passed per call, no process
     state involved) and return its result: ``[B,S,H*D]`` (``out_layout="bshd"``, the layout
     of the reference's row-wise operators) or ``[B,H,S,D]`` (``"bhsd"``, block-wise only).
-    ``lut``: the seven LUT tensors, needed for "block-wise"."""
+    ``lut``: the seven LUT tensors, needed for "block-wise"; ``row_mask`` [S,S] of 0/1 for the
+    row-wise element-mask operator."""
     from .ops import block_attn, rowwise_attn
     if selection.operator == "row-wise":
-        return rowwise_attn("full", q, k, v, is_causal, launch_form=selection.launch_form)
+        if selection.row_kind == "mask" and row_mask is None:
+            raise ValueError("the row-wise mask operator needs row_mask [S,S]")
+        return rowwise_attn(selection.row_kind, q, k, v, is_causal, bandwidth=selection.bandwidth, row_mask=row_mask,
+                            launch_form=selection.launch_form)
     if lut is None:
         raise ValueError("the block-wise operator needs the LUT")
     return block_attn(q, k, v, lut, selection.block_m, selection.block_n, out_layout=out_layout,

@@ -192,7 +192,9 @@ def test_lut_build_argument_checks(lib):
     assert i(bits=P, bm=32, bn=32) == -3       # bit rows exist for 64 x 64 only
     assert i(ws=None) == -1
     assert i(wsb=100) == -2                    # workspace too small
-    assert lib.stof_build_lut_workspace_bytes(4096, 64, 64) == 4096 + 4096 * 512
-    assert lib.stof_build_lut_workspace_bytes(256, 16, 16) == 256
+    # class bytes (a multiple of 256) + 512 B of bit rows per 64 x 64 tile + 2 B of count per tile (a multiple of 16) + 16
+    assert lib.stof_build_lut_workspace_bytes(4096, 64, 64) == 4096 + 4096 * 512 + 4096 * 2 + 16
+    assert lib.stof_build_lut_workspace_bytes(256, 16, 16) == 256 + 256 * 2 + 16
+    assert lib.stof_build_lut_nnz_offset(256, 16, 16) == 256 + 256 * 2
     assert lib.stof_lut_additive_blocks(P, 2, 256, 256, 64, 64, None, None, 0, None, None) == 0
     assert lib.stof_lut_additive_blocks(P, 2, 256, 256, 64, 64, None, None, 3, None, None) == -1

@@ -101,3 +101,25 @@ def test_per_call_form_overrides_module_default():
     _close(a, want, "key_split per call"); _close(b, want, "default")
     with pytest.raises(Exception):
         block_attn(q, k, v, lut, launch_form="three_rows")
+
+
+def test_row_wise_variants_selected_by_mask_kind():
+    """select -> apply for the sliding-window and element-mask row-wise operators, result vs the oracle."""
+    B, H, S, bw = 2, 4, 1024, 200
+    q, k, v = configs.qkv(configs.AttnConfig("rw", B, H, S), seed=4, device="cuda")
+    i = torch.arange(S)
+    win = (i[:, None] - i[None, :] < bw) & (i[None, :] <= i[:, None])
+    lut = pm.get_sparse_storage(win.float()[None].cuda(), 64, 64)[1:]
+    sel = selector.select_operator(selector.GPUParams(), lut[5], B, S, H, is_causal=True, lut=lut, mask_kind="sliding", bandwidth=bw)
+    assert (sel.operator, sel.row_kind) == ("row-wise", "sliding")
+    got = selector.apply(sel, q, k, v, is_causal=True).view(B, S, H, 64).permute(0, 2, 1, 3)
+    _close(got, oa.dense_masked_attention(q.cpu().float(), k.cpu().float(), v.cpu().float(), win), "row-wise sliding")
+    blk = selector.apply(selector.select_operator(selector.GPUParams(), lut[5], B, S, H, is_causal=True, lut=lut), q, k, v, lut, is_causal=True)
+    _close(blk.view(B, S, H, 64).permute(0, 2, 1, 3), oa.dense_masked_attention(q.cpu().float(), k.cpu().float(), v.cpu().float(), win), "block-wise on the same mask")
+    g = torch.Generator().manual_seed(8)
+    em = torch.rand(S, S, generator=g) < 0.7
+    em[:, 0] = True
+    sel = selector.select_operator(selector.GPUParams(), None, B, S, H, mask_kind="element")
+    assert (sel.operator, sel.row_kind) == ("row-wise", "mask")
+    got = selector.apply(sel, q, k, v, row_mask=em.half().cuda()).view(B, S, H, 64).permute(0, 2, 1, 3)
+    _close(got, oa.dense_masked_attention(q.cpu().float(), k.cpu().float(), v.cpu().float(), em), "row-wise element mask")

@@ -77,3 +77,28 @@ def test_per_sample_row_pointers_and_errors():
         selector.select_operator(selector.GPUParams(), lut[6], 4, 500, 12)
     with pytest.raises(ValueError):
         selector.GPUParams("A100")
+
+
+def test_stated_mask_kinds_select_the_row_wise_variants():
+    """The caller's knowledge of the mask (the reference's benchmark selects its row-wise operator
+    by the mask's name, src/benchmk_attn_unified.py:396-407)."""
+    gpu = selector.GPUParams()
+    s, bw = 1024, 200
+    i = torch.arange(s)
+    win = ((i[:, None] - i[None, :] < bw) & (i[None, :] <= i[:, None])).float()      # causal sliding window
+    lut = _lut(win)
+    sel = selector.select_operator(gpu, lut[6], 2, s, 12, is_causal=True, mask_kind="sliding", bandwidth=bw)
+    assert (sel.operator, sel.row_kind, sel.bandwidth) == ("row-wise", "sliding", bw)
+    # a LUT that lists other tiles than the stated window stays block-wise
+    assert selector.select_operator(gpu, _lut(configs.mask_c5(s))[6], 2, s, 12, is_causal=True,
+                                    mask_kind="sliding", bandwidth=bw).operator == "block-wise"
+    # no LUT at hand: row-wise by the stated kind
+    for kind, want in (("dense", "full"), ("causal", "full"), ("sliding", "sliding"), ("element", "mask")):
+        sel = selector.select_operator(gpu, None, 2, s, 12, mask_kind=kind, bandwidth=bw)
+        assert sel.operator == "row-wise" and sel.row_kind == want and str(sel) == "row-wise"
+    with pytest.raises(ValueError):
+        selector.select_operator(gpu, None, 2, s, 12)
+    with pytest.raises(ValueError):
+        selector.select_operator(gpu, None, 2, s, 12, mask_kind="sliding")
+    with pytest.raises(ValueError):
+        selector.select_operator(gpu, lut[6], 2, s, 12, mask_kind="banded")
