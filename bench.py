@@ -140,6 +140,37 @@ def bench_attn(cfg, mask_fn, steps, warmup, settle_ms=SETTLE_MS, launch_form=Non
     return r
 
 
+def probe_issue_mix(steps=4000):
+    """The arithmetic of the attention loop alone (library probe stof_probe_issue_mix): ns per
+    wave-step and SIMD for the MFMAs only, the vector arithmetic only and both, at 1 .. 4 wavefronts
+    per SIMD, with the shader clock read inside each launch; and what that ceiling is in TFLOP/s."""
+    from stof import _lib
+    lib = _lib.lib()
+    cus = lib.stof_device_compute_units()
+    out = torch.zeros(3, dtype=torch.int64, device="cuda")
+    sink = torch.zeros(256, dtype=torch.float32, device="cuda")
+    stream = torch.cuda.current_stream().cuda_stream
+    rows = []
+    for waves in (1, 2, 3, 4):
+        row = {"waves_per_simd": waves}
+        for parts, name in ((1, "mfma_only"), (2, "valu_only"), (3, "both")):
+            fn = lambda: lib.stof_probe_issue_mix(parts, waves, steps, out.data_ptr(), sink.data_ptr(), stream)
+            _, ev_ms = time_region(fn, 20, 5, settle_ms=60.0)
+            cyc, ticks, _ = out.tolist()
+            ns = ev_ms * 1e6 / (steps * waves)
+            row[name] = {"ns_per_wave_step": ns, "clock_ghz": cyc / ticks * 0.1 if ticks else None,
+                         "cycles_per_wave_step": ns * (cyc / ticks * 0.1) if ticks else None}
+        b = row["both"]["ns_per_wave_step"]
+        # a wave-step is 32 queries x 64 keys x 64 channels x 4 FLOP; 4 SIMDs per compute unit
+        row["ceiling_tflops"] = 4 * cus * (32 * 64 * 64 * 4) / b / 1e3
+        row["overlap"] = (row["mfma_only"]["ns_per_wave_step"] + row["valu_only"]["ns_per_wave_step"] - b) / min(
+            row["mfma_only"]["ns_per_wave_step"], row["valu_only"]["ns_per_wave_step"])
+        rows.append(row)
+    return {"cu_count": cus, "steps": steps,
+            "mix_per_wave_step": "16 v_mfma_f32_32x32x16_f16, 32 v_fma_f32, 32 v_exp_f32, 16 v_cvt_pk_f16_f32, 16 v_pk_add_f16, "
+                                 "16 v_max3_f32 + lazy-max test; no memory, LDS or barrier", "rows": rows}
+
+
 def host_cost_us(n=2000):
     """Host time of one block_attn call (Python operator + binding + hipLaunchKernel): a loop of
     launches of the small C1 problem with the clock stopped BEFORE the device is waited for."""
@@ -438,6 +469,8 @@ def main():
     ap.add_argument("--extras", default="c1,c2,c5attn,c4big,forms,dense,c3,c3small,c5,hbm,lut",
                     help="comma-separated subset of the extra workloads to run (for profiling one kind of kernel)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--probe-mix", action="store_true",
+                    help="run only the instruction-mix probe of the attention loop and print its table as JSON")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run one plain device copy of 256 MiB, so that a counter run of this "
                          "command holds a kernel of known traffic to scale FETCH_SIZE / WRITE_SIZE by")
@@ -452,6 +485,9 @@ def main():
 
     from stof import configs
     torch.cuda.set_device(0)
+    if args.probe_mix:
+        print(json.dumps(probe_issue_mix()))
+        return
     if args.copy_probe:
         src = torch.empty(256 << 20, dtype=torch.uint8, device="cuda").fill_(1)
         dst = torch.empty_like(src)

@@ -425,6 +425,17 @@ int stof_gemm_bias_res_ln_cluster_dt(const void* A, const void* Wt, const void* 
  */
 int stof_device_compute_units(void);
 int stof_probe_clock(unsigned long long* out3, int iters, void* stream);
+/*
+ * The arithmetic of one step of the attention loop (per wavefront 32 queries x 64 keys at head size
+ * 64: 16 MFMA 32x32x16, 32 multiply-adds, 32 exp2, 16 converts, 16 packed adds, 16 max3) with no
+ * memory access, LDS access or barrier, run for `steps` steps by waves_per_simd (1 .. 4) wavefronts
+ * on every SIMD of the device.  parts: 1 = the MFMAs only, 2 = the vector arithmetic only, 3 = both.
+ * The launch's duration / (steps * waves_per_simd) is the time one SIMD needs per wave-step of this
+ * mix: the ceiling of the loop before loads, LDS reads, barriers, masks and the walk.  out3 as for
+ * stof_probe_clock (first wavefront of the launch; out3[2] = steps); sink256: 256 floats of device
+ * memory, never written in practice.
+ */
+int stof_probe_issue_mix(int parts, int waves_per_simd, int steps, unsigned long long* out3, float* sink256, void* stream);
 
 #ifdef __cplusplus
 }

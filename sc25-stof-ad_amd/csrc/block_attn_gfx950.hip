@@ -42,7 +42,14 @@ constexpr int kBM = 64;       // query rows per block
 constexpr int kBN = 64;       // keys per block
 constexpr int kTile = kBN * kD * 2;   // bytes of one K or V tile in LDS (8 KB, unpadded)
 constexpr float kLazy = 8.0f;         // log2 slack before the running max is raised
-constexpr int kPrioStep = 6;          // key blocks of remaining chain per issue-priority level
+// Key blocks of remaining chain per issue-priority level (levels 0 .. 3: 6 and more left, 4-5, 2-3,
+// under 2).  A compute unit's four workgroups arrive longest first, and among waves of equal
+// priority a SIMD issues from the oldest: above the top threshold that order IS longest first.
+// What the step sets is the endgame: all waves below the last threshold are equal again, the
+// youngest workgroup starves and then finishes alone - about one step's worth of chain per unit
+// of kPrioStep.  Measured (step 6 -> 2): B2 H16 S4096 sparse 40.4 -> 38.8 us, B4 H16 S2048 20.8 ->
+// 19.0, B8 H12 S1024 21.7 -> 20.5, B16 H12 S512 14.0 -> 13.0, dense unchanged; step 1 gives back 1-5 %.
+constexpr int kPrioStep = 2;
 
 typedef __attribute__((address_space(3))) unsigned char lds_byte;
 typedef short short4_t __attribute__((ext_vector_type(4)));

@@ -48,6 +48,7 @@ PYBIND11_MODULE(_stof_ext, m) {
   STOF_BIND(stof_abi_version);
   STOF_BIND(stof_device_compute_units);
   STOF_BIND(stof_probe_clock);
+  STOF_BIND(stof_probe_issue_mix);
   m.def("stof_status_string", [](int status) { return py::bytes(stof_status_string(status)); });
   STOF_BIND(stof_block_attn_fwd);
   STOF_BIND(stof_block_attn_fwd_planned);

@@ -26,6 +26,7 @@ _I64x3 = c_int64 * 3
 _SIGNATURES = {
     "stof_device_compute_units": (c_int, []),
     "stof_probe_clock": (c_int, [_P, c_int, _P]),
+    "stof_probe_issue_mix": (c_int, [c_int, c_int, c_int, _P, _P, _P]),
     "stof_abi_version": (c_int, []),
     "stof_status_string": (c_char_p, [c_int]),
     "stof_block_attn_fwd": (c_int, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P,
