@@ -254,7 +254,7 @@ int stof_retile_lut(const int32_t* full_row_ptr, const int32_t* full_col_idx,
  * stof_build_lut without the workspace argument, for callers that cannot allocate device memory
  * (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has
  * no counterpart in the reference.  The scratch is a fixed array in device memory that the
- * library holds per GPU until the process ends (8.02 MB: class bytes and bit rows for up to
+ * library holds per GPU until the process ends (8.05 MiB: class bytes, bit rows and per-tile counts for up to
  * stof_build_lut_static_max_tiles() = 16384 tiles, i.e. seq_len 8192 at 64 x 64 blocks); a
  * larger problem returns STOF_ERR_TOO_LARGE.  No hipMalloc / hipFree or allocating routine is
  * called.  Every call on a GPU uses that GPU's one array: calls that overlap on one GPU (two

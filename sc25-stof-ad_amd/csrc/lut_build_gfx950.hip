@@ -22,7 +22,7 @@
 #include "stof_common.h"
 
 // Scratch of stof_build_lut_static, the entry point that allocates nothing: class bytes and bit
-// rows for at most kStaticMaxTiles tiles (8.02 MB per GPU, held until the process ends).  In
+// rows for at most kStaticMaxTiles tiles (8.05 MiB per GPU with the per-tile counts, held until the process ends).  In
 // host code the array's name is a stand-in, not a device address: the address of each device's
 // copy is taken once per device with hipGetSymbolAddress and only that pointer is used.
 constexpr int64_t kStaticMaxTiles = 16384;   // S = 8192 at 64 x 64 blocks
