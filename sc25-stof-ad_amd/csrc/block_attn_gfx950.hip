@@ -1256,15 +1256,19 @@ enum { kFormAuto = -1, kFormTwoRows = 0, kFormKeySplit = 1, kFormPipelined = 2 }
 constexpr int kKeySplitMaxGroupsPerCu = 2;
 constexpr int kKeySplitMinQueryBlocks = 4;
 
+// Compute units of the current device, asked once per device (relaxed atomics: two threads that
+// both find the slot empty store the same number).
 int compute_units() {
-  static int cus = 0;
-  if (cus == 0) {
-    int dev = 0, n = 0;
-    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
-      n = 256;
-    cus = n;
+  constexpr int kMaxDevices = 64;
+  static int cached[kMaxDevices] = {};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return 256;
+  int n = __atomic_load_n(&cached[dev], __ATOMIC_RELAXED);
+  if (n == 0) {
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    __atomic_store_n(&cached[dev], n, __ATOMIC_RELAXED);
   }
-  return cus;
+  return n;
 }
 
 int pick_form(int requested, int64_t two_row_groups, int nQ) {

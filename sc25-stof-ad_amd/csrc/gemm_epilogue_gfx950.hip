@@ -1175,15 +1175,17 @@ int64_t cluster_resident_groups() {
   static int cached[kMaxDevices] = {};   // 0 = not asked yet, -1 = the query failed
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return 0;
-  if (cached[dev] == 0) {
+  int groups = __atomic_load_n(&cached[dev], __ATOMIC_RELAXED);   // (two threads that both find 0 store the same number)
+  if (groups == 0) {
     int cus = 0, per_cu = 0;
     if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0 ||
         hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, gemm_bias_res_ln_cluster_kernel<NT, BF>, 256, 0) != hipSuccess || per_cu <= 0)
-      cached[dev] = -1;
+      groups = -1;
     else
-      cached[dev] = (per_cu < kClusterGroupsPerCu ? per_cu : kClusterGroupsPerCu) * cus;
+      groups = (per_cu < kClusterGroupsPerCu ? per_cu : kClusterGroupsPerCu) * cus;
+    __atomic_store_n(&cached[dev], groups, __ATOMIC_RELAXED);
   }
-  return cached[dev] < 0 ? 0 : cached[dev] / 8 * 8;
+  return groups < 0 ? 0 : groups / 8 * 8;
 }
 }  // namespace
 

@@ -304,12 +304,14 @@ unsigned char* g_scratch_ptr[kMaxDevices] = {nullptr};
 int static_scratch(unsigned char** out) {
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return STOF_ERR_LAUNCH;
-  if (!g_scratch_ptr[dev]) {
+  unsigned char* cached = __atomic_load_n(&g_scratch_ptr[dev], __ATOMIC_RELAXED);
+  if (!cached) {   // (two threads that both find the slot empty store the same address)
     void* ptr = nullptr;
     if (hipGetSymbolAddress((void**)&ptr, HIP_SYMBOL(scratch)) != hipSuccess || !ptr) return STOF_ERR_LAUNCH;
-    g_scratch_ptr[dev] = static_cast<unsigned char*>(ptr);
+    cached = static_cast<unsigned char*>(ptr);
+    __atomic_store_n(&g_scratch_ptr[dev], cached, __ATOMIC_RELAXED);
   }
-  *out = g_scratch_ptr[dev];
+  *out = cached;
   return STOF_OK;
 }
 

@@ -141,9 +141,13 @@ def test_layer_check_flag_raises_after_a_failed_exchange():
     lut = pm.get_sparse_storage(configs.mask_c1(S).float()[None].cuda(), 64, 64)[1:]
     layer = EncoderLayer(w, H, eps=1e-12, ln_fusion="cluster")
     layer(x, lut, check=True)                    # a clean run passes
-    xa = _rand(4096, 768, seed=1).cuda(); Wt = fused.pack_weight(_rand(768, 768, seed=2, scale=0.05).cuda())
-    for _ in range(5):
-        fused.gemm_bias_residual_layernorm(xa, Wt, None, None, None, None, form="cluster", spin_limit=1)
+    # the condition is forced from the host: the error word of the workspace the layer's launches use is
+    # set as a wave that gave up would set it (the kernel's own give-up path is the test above)
+    torch.cuda.synchronize()
+    words = [ws for (d, _), ws in fused._cluster_ws.items() if d == x.device.index]
+    assert words, "the layer ran no cluster-form launch"
+    for ws in words:
+        ws[:4].view(torch.int32).fill_(1)
     with pytest.raises(fused.StofError):
         layer(x, lut, check=True)
-    layer(x, lut, check=True)
+    layer(x, lut, check=True)                    # the check cleared the word
