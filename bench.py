@@ -94,11 +94,18 @@ class ClockProbe:
         return s[len(s) // 2] if s else None
 
 
-def time_region(fn, steps, warmup, settle_ms=SETTLE_MS):
+def time_region(fn, steps, warmup, settle_ms=SETTLE_MS, preheat_ms=0.0):
     """(wall ms per step, event ms per step) for `steps` calls after `warmup` untimed ones.
     After the warm-up calls, further untimed calls keep the GPU busy until `settle_ms` of wall
     time have passed, so that every region - ours, PyTorch's, the copies - is timed at settled
-    clocks.  The headline region passes settle_ms=0 and relies on its warm-up count alone."""
+    clocks.  The headline region passes settle_ms=0: it runs exactly `warmup` untimed steps right
+    before the timed ones, and keeps the GPU under the same load for `preheat_ms` BEFORE those
+    (the clocks of an idle GPU need tens of ms of load, however many warm-up steps are asked for)."""
+    t_heat = time.perf_counter()
+    while preheat_ms > 0 and (time.perf_counter() - t_heat) * 1e3 < preheat_ms:
+        for _ in range(50):
+            fn()
+        torch.cuda.synchronize()
     for _ in range(warmup):
         fn()
     torch.cuda.synchronize()
@@ -119,13 +126,13 @@ def time_region(fn, steps, warmup, settle_ms=SETTLE_MS):
     return (t1 - t0) * 1e3 / steps, e0.elapsed_time(e1) / steps
 
 
-def bench_attn(cfg, mask_fn, steps, warmup, settle_ms=SETTLE_MS, launch_form=None, dtype=torch.float16, probe=None):
+def bench_attn(cfg, mask_fn, steps, warmup, settle_ms=SETTLE_MS, launch_form=None, dtype=torch.float16, probe=None, preheat_ms=0.0):
     from stof.ops import block_attn
     q, k, v, lut, n_active, _ = attn_setup(cfg, mask_fn, "cuda")
     q, k, v = (t.to(dtype) for t in (q, k, v))
     out = torch.empty_like(q)
     block_attn(q, k, v, lut, out=out, launch_form=launch_form)          # packs the partial-block bit masks and lays out the walk once
-    wall_ms, ev_ms = time_region(lambda: block_attn(q, k, v, lut, out=out, launch_form=launch_form), steps, warmup, settle_ms)
+    wall_ms, ev_ms = time_region(lambda: block_attn(q, k, v, lut, out=out, launch_form=launch_form), steps, warmup, settle_ms, preheat_ms)
     flop = FLOP_PER_BLOCK * cfg.batch * cfg.heads * n_active
     r = {"wall_ms": wall_ms, "kernel_ms": ev_ms, "flop": flop, "active_blocks": n_active,
          "tflops_wall": flop / wall_ms / 1e9, "tflops_kernel": flop / ev_ms / 1e9}
@@ -465,6 +472,9 @@ def main():
     ap.add_argument("--steps", type=int, default=2000)
     ap.add_argument("--warmup", type=int, default=2000,
                     help="untimed steps before the timed ones; the default (about 70 ms of load) lets the clocks settle")
+    ap.add_argument("--settle-ms", type=float, default=SETTLE_MS,
+                    help="ms of the same load run BEFORE the warm-up steps of the headline, so that a small --warmup is not "
+                         "timed on the clock ramp of an idle GPU (0 = none); reported as config.clock_settle_ms")
     ap.add_argument("--no-extras", action="store_true", help="skip everything but the C4 attention step")
     ap.add_argument("--extras", default="c1,c2,c5attn,c4big,forms,dense,c3,c3small,c5,hbm,lut",
                     help="comma-separated subset of the extra workloads to run (for profiling one kind of kernel)")
@@ -496,7 +506,8 @@ def main():
     from stof import _lib
     probe = ClockProbe()
     cus = _lib.lib().stof_device_compute_units()
-    c4 = bench_attn(configs.C4, configs.mask_c4, args.steps, args.warmup, settle_ms=0, probe=probe)   # exactly W warm-up steps, then K timed
+    # the GPU is kept under this load for --settle-ms first (clock ramp of an idle device), then exactly W warm-up steps, then K timed
+    c4 = bench_attn(configs.C4, configs.mask_c4, args.steps, args.warmup, settle_ms=0, probe=probe, preheat_ms=args.settle_ms)
     clock = probe.ghz()
     traffic, traffic_source = measured_traffic()
     line = {
@@ -507,7 +518,8 @@ def main():
         "dtype": "f16", "data": "synthetic",
         "config": {"workload": "C4: long-sequence block-masked MHA, B2 H16 S4096 D64, causal sliding window of 512 + "
                                "every 4th key block, 64 x 64 blocks", "active_blocks": c4["active_blocks"],
-                   "blocks_total": (configs.C4.seq // 64) ** 2, "block": 64, "flop_per_step": c4["flop"]},
+                   "blocks_total": (configs.C4.seq // 64) ** 2, "block": 64, "flop_per_step": c4["flop"],
+                   "clock_settle_ms": args.settle_ms},
         "roofline": {"bound": "mfma", "achieved": c4["tflops_kernel"], "peak": PEAK_FP16_TFLOPS, "unit": "TFLOP/s",
                      "frac": c4["tflops_kernel"] / PEAK_FP16_TFLOPS, "traffic": traffic, "traffic_source": traffic_source,
                      "algorithmic_bytes": 4 * configs.C4.batch * configs.C4.heads * configs.C4.seq * 64 * 2,
