@@ -171,3 +171,47 @@ def test_planned_entry_point_through_the_c_abi():
     want = oa.dense_masked_attention(q.cpu().float(), k.cpu().float(), v.cpu().float(), mask)
     err = (base.float().cpu() - want).abs()
     assert not bool((err > ATOL + RTOL * want.abs()).any())
+
+
+def _hand_lut(S, device="cuda"):
+    """A LUT written down directly (no dense S x S mask, which at these lengths would not fit): query
+    block r lists key block 0 (full; for r = 0 it is the diagonal), r - 1 (full) and r (partial: causal
+    inside the block)."""
+    nq = S // 64
+    lci, fci, pci, lrp, frp, prp = [], [], [], [0], [0], [0]
+    for r in range(nq):
+        full = sorted({0, r - 1} - {r, -1})
+        fci += full; pci.append(r); lci += sorted(full + [r])
+        frp.append(len(fci)); prp.append(len(pci)); lrp.append(len(lci))
+    t = lambda a: torch.tensor(a, dtype=torch.int32, device=device)
+    tri = torch.tril(torch.ones(64, 64))
+    pbm = (-10000.0 * (1 - tri)).half().to(device).expand(nq, 64, 64).contiguous()
+    return (t(frp), t(fci), t(prp), t(pci), pbm, t(lrp), t(lci))
+
+
+@pytest.mark.parametrize("S,planned", [(65536, True), (65600, False)])
+def test_longest_sequence_with_a_plan_and_the_first_without(S, planned):
+    """1024 key blocks is the longest walk a plan holds; beyond it the operator runs the in-kernel
+    walk.  Both against dense attention on a few query blocks (first, second, one in the middle,
+    the last), and at the limit the two paths bit for bit."""
+    print(f"plan limit S{S}", flush=True)
+    lib = _lib.lib()
+    assert (lib.stof_attn_plan_bytes(S, 2, 1) > 0) == planned
+    g = torch.Generator(device="cuda").manual_seed(S)
+    q, k, v = (torch.randn(1, 1, S, 64, device="cuda", generator=g).half() for _ in range(3))
+    lut = _hand_lut(S)
+    got = block_attn(q, k, v, lut)
+    if planned:
+        assert torch.equal(got, block_attn(q, k, v, lut, use_plan=False))
+    nq = S // 64
+    for r in (0, 1, nq // 2 + 1, nq - 1):
+        cols = sorted({0, r - 1, r} - {-1})
+        keys = torch.cat([torch.arange(64 * c, 64 * c + 64) for c in cols]).cuda()
+        qi = torch.arange(64 * r, 64 * r + 64).cuda()
+        allow = torch.ones(64, len(keys), dtype=torch.bool, device="cuda")
+        allow[:, -64:] = torch.tril(torch.ones(64, 64, dtype=torch.bool, device="cuda"))      # the diagonal block comes last
+        s = (q[0, 0, qi].float() @ k[0, 0, keys].float().t()) * 0.125
+        s = s.masked_fill(~allow, float("-inf"))
+        want = torch.softmax(s, -1) @ v[0, 0, keys].float()
+        err = (got[0, 0, qi].float() - want).abs()
+        assert bool((err <= ATOL + RTOL * want.abs()).all()), f"S{S} query block {r}: max err {float(err.max()):.2e}"
