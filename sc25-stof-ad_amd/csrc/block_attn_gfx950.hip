@@ -130,6 +130,7 @@ __device__ __forceinline__ void attn_group(const AttnParams& p, const int bh, co
   // instructions between the start of the workgroup and its first K/V tile.
   int pair = pair_or_slot;
   uint32_t plan_lo = 0, plan_hi = 0;     // the current window of 64 plan words, one per lane
+  uint64_t plan_sw[4] = {0, 0, 0, 0};    // words 0-3 of the block in scalar registers (a block has at least 8 words)
   const uint64_t* plan_blk = nullptr;
   if constexpr (PLAN) {
     const int sample = p.lut_bs ? bh / p.H : 0;
@@ -137,6 +138,10 @@ __device__ __forceinline__ void attn_group(const AttnParams& p, const int bh, co
     const int l = threadIdx.x & 63;
     const uint64_t w = l < p.plan_stride ? plan_blk[l] : 0ull;
     plan_lo = (uint32_t)w; plan_hi = (uint32_t)(w >> 32);
+    // the header and the first two steps also through the scalar cache: a wave-uniform address, and the
+    // answer does not queue behind the vector-memory traffic of the sixteen waves that start together
+#pragma unroll
+    for (int i = 0; i < 4; ++i) plan_sw[i] = plan_blk[i];
   }
   constexpr int kDma = 4 / (ROWS * KS);   // direct-to-LDS instructions per wave and operand tile (8 per tile)
   constexpr int kMT = 2 / KS;             // 32-key sub-tiles of a key block handled by one wave
@@ -155,10 +160,10 @@ __device__ __forceinline__ void attn_group(const AttnParams& p, const int bh, co
 
   int plan_n = 0, plan_p0 = 0, plan_i = 0;   // PLAN: steps of the group, first PART slot of this wave's row, next step
   if constexpr (PLAN) {
-    const uint32_t h0 = __builtin_amdgcn_readlane(plan_lo, 0);
+    const uint32_t h0 = (uint32_t)plan_sw[0];
     pair = h0 & 0xffff;
     plan_n = h0 >> 16;
-    plan_p0 = rsel == 0 ? __builtin_amdgcn_readlane(plan_lo, 1) : __builtin_amdgcn_readlane(plan_hi, 1);
+    plan_p0 = rsel == 0 ? (int)(uint32_t)plan_sw[1] : (int)(uint32_t)(plan_sw[1] >> 32);
   }
   const int b = bh / p.H;
   const int h = bh - b * p.H;
@@ -348,8 +353,14 @@ __device__ __forceinline__ void attn_group(const AttnParams& p, const int bh, co
       if (plan_i >= plan_n) return s;
       const int word = plan_i + 2;
       if ((word & 63) == 0) { plan_lo = plan_nlo; plan_hi = plan_nhi; }
-      const uint32_t lo = __builtin_amdgcn_readlane(plan_lo, word & 63);
-      const uint32_t hi = __builtin_amdgcn_readlane(plan_hi, word & 63);
+      uint32_t lo, hi;
+      if (word < 4) {   // the first two steps: from the scalar copy, without waiting for the window
+        const uint64_t w = word == 2 ? plan_sw[2] : plan_sw[3];
+        lo = (uint32_t)w; hi = (uint32_t)(w >> 32);
+      } else {
+        lo = __builtin_amdgcn_readlane(plan_lo, word & 63);
+        hi = __builtin_amdgcn_readlane(plan_hi, word & 63);
+      }
       if ((word & 63) == 48 && (word | 63) + 1 < plan_n + 2) {
         const int at = (word | 63) + 1 + lane;
         const uint64_t w = at < p.plan_stride ? plan_blk[at] : 0ull;
