@@ -713,7 +713,8 @@ __global__ __launch_bounds__(256, kClusterGroupsPerCu) void gemm_bias_res_ln_clu
   __shared__ __attribute__((aligned(1024))) unsigned char a_lds1[kGTile];
   __shared__ __attribute__((aligned(1024))) unsigned char w_lds0[kGTile];
   __shared__ __attribute__((aligned(1024))) unsigned char w_lds1[kGTile];
-  constexpr int kParts = 2 * NT;
+  constexpr int kParts = NT;           // published words per row: one per workgroup of the row block (its 128 features)
+  constexpr int kLeavers = 2 * NT;     // waves that read the words of a half row block (two feature halves per workgroup)
 
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int lane = threadIdx.x & 63;
@@ -877,13 +878,30 @@ __global__ __launch_bounds__(256, kClusterGroupsPerCu) void gemm_bias_res_ln_clu
     wm2[mi] = pair_sum(d2);
   }
 
-  // ---- publish; lane (j32, g) speaks for row 64 wm + 32 g + j32 of the row block
+  // ---- the two waves of a row half (feature halves wn = 0, 1) first merge their statistics through
+  // LDS (the W buffer of the last tile's stage is free since the barrier above): the workgroup then
+  // publishes ONE word per row for its 128 features, a wave's own workgroup never costs it a trip
+  // through memory, and a poll reads half as many words.  Lane (j32, g) speaks for row
+  // 64 wm + 32 g + j32 of the row block.
   const int row_l = 64 * wm + 32 * g + j32;
-  unsigned long long* my_stats = p.stats + ((int64_t)tm * kParts) * kGT + row_l;
+  unsigned long long* my_stats = p.stats + ((int64_t)tm * (2 * NT)) * kGT + row_l;   // (the workspace keeps room for 2 NT words per row)
+  float own_mean, own_m2;   // of this workgroup's 128 features
   {
+    __attribute__((address_space(3))) float* xs = (__attribute__((address_space(3))) float*)(last_in_0 ? (lds_byte*)w_lds0 : (lds_byte*)w_lds1);
     const float pm = g ? wmean[1] : wmean[0], pq = g ? wm2[1] : wm2[0];
-    const unsigned long long word = ((unsigned long long)__builtin_bit_cast(unsigned, pq) << 32) | __builtin_bit_cast(unsigned, pm);
-    __hip_atomic_store(my_stats + (int64_t)(2 * tn + wn) * kGT, word | kStatsValid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    xs[(2 * wn) * kGT + row_l] = pm;
+    xs[(2 * wn + 1) * kGT + row_l] = pq;
+    __syncthreads();
+    const float om = xs[(2 * (1 - wn)) * kGT + row_l], oq = xs[(2 * (1 - wn) + 1) * kGT + row_l];
+    const float ma = wn ? om : pm, mb = wn ? pm : om;   // (feature half 0, feature half 1: the same order in both waves)
+    const float qa = wn ? oq : pq, qb = wn ? pq : oq;
+    own_mean = 0.5f * (ma + mb);
+    const float da = ma - own_mean, db = mb - own_mean;
+    own_m2 = (qa + qb) + 64.0f * (da * da + db * db);
+    if (wn == 0) {
+      const unsigned long long word = ((unsigned long long)__builtin_bit_cast(unsigned, own_m2) << 32) | __builtin_bit_cast(unsigned, own_mean);
+      __hip_atomic_store(my_stats + (int64_t)tn * kGT, word | kStatsValid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
   }
   // gamma and beta are requested here: they arrive while the wave waits for the other parts
   half4_t gv[2][4], tv[2][4];
@@ -898,15 +916,17 @@ __global__ __launch_bounds__(256, kClusterGroupsPerCu) void gemm_bias_res_ln_clu
       if (p.beta) tv[ni][q4] = *reinterpret_cast<const half4_t*>(p.beta + n);
     }
 
-  // ---- collect the parts of this lane's row: read all of them until all are valid
+  // ---- collect the parts of this lane's row: read those of the other workgroups until all are valid
   unsigned long long word[kParts];
   {
+    const unsigned long long own_word = (((unsigned long long)__builtin_bit_cast(unsigned, own_m2) << 32) | __builtin_bit_cast(unsigned, own_mean)) | kStatsValid;
     int polls = 0;
     for (;;) {
       bool ok = true;
 #pragma unroll
       for (int pt = 0; pt < kParts; ++pt) {
-        word[pt] = __hip_atomic_load(my_stats + (int64_t)pt * kGT, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        word[pt] = own_word;
+        if (pt != tn) word[pt] = __hip_atomic_load(my_stats + (int64_t)pt * kGT, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         ok = ok && (word[pt] & kStatsValid) != 0;
       }
       if (!__any(!ok)) break;
@@ -930,7 +950,7 @@ __global__ __launch_bounds__(256, kClusterGroupsPerCu) void gemm_bias_res_ln_clu
     const float d = __builtin_bit_cast(float, (unsigned)(word[pt] & 0xffffffffull)) - mean_own;
     spread += d * d;
   }
-  m2 += 64.0f * spread;
+  m2 += 128.0f * spread;   // (every part speaks for 128 features)
   const float rstd_own = 1.0f / sqrtf(m2 * p.inv_n + p.eps);
   const float mean_other = xchg32(mean_own), rstd_other = xchg32(rstd_own);
   float mean[2], rstd[2];
@@ -969,7 +989,7 @@ __global__ __launch_bounds__(256, kClusterGroupsPerCu) void gemm_bias_res_ln_clu
   int prev = 0;
   if (lane == 0) prev = __hip_atomic_fetch_add(dep, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   prev = __builtin_amdgcn_readfirstlane(prev);
-  if (prev == kParts - 1) {
+  if (prev == kLeavers - 1) {
 #pragma unroll
     for (int pt = 0; pt < kParts; ++pt)
       __hip_atomic_store(my_stats + (int64_t)pt * kGT, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
