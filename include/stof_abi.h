@@ -217,8 +217,9 @@ int stof_rowwise_attn_fwd(
  */
 int64_t stof_build_lut_workspace_bytes(int seq_len, int block_m, int block_n);
 /* Byte offset inside that workspace at which a call of stof_build_lut leaves the number of non-zero
- * mask elements as an int64 (the reference's nnz figure, src/util/masks.py:137, counted in the same
- * pass as the classification); the last 16 bytes of the workspace. */
+ * mask elements as an int64 (counted in the same pass as the classification) and, in the 4 bytes
+ * behind it, the reference's nnz figure (src/util/masks.py:137) as a float32: count / seq_len^2 * 100
+ * in fp32 arithmetic; the last 16 bytes of the workspace. */
 int64_t stof_build_lut_nnz_offset(int seq_len, int block_m, int block_n);
 int stof_build_lut(const void* mask, int elem_bytes, int64_t ld, int seq_len, int block_m, int block_n,
                    int32_t* full_row_ptr, int32_t* full_col_idx,

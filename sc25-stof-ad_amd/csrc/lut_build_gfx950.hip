@@ -211,7 +211,12 @@ __global__ __launch_bounds__(256) void lut_compact_kernel(const LutParams p) {
     __syncthreads();
     if (lane == 0) part_sum[wave] = total;
     __syncthreads();
-    if (tid == 0) *p.nnz = part_sum[0] + part_sum[1] + part_sum[2] + part_sum[3];
+    if (tid == 0) {
+      const long long all = part_sum[0] + part_sum[1] + part_sum[2] + part_sum[3];
+      *p.nnz = all;
+      // the reference's figure (src/util/masks.py:137) in its own arithmetic: count / (S * S) * 100 in fp32
+      reinterpret_cast<float*>(p.nnz + 1)[0] = (float)all / (float)((long long)p.S * p.S) * 100.0f;
+    }
   }
   if (tid == 0) {
     if (r == 0) { p.frp[0] = 0; p.prp[0] = 0; p.lrp[0] = 0; }

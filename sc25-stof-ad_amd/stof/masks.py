@@ -152,18 +152,17 @@ def _build_on_device(m2d, bm, bn, want_bits):
     nq, nk = n // bm, n // bn
     tiles = nq * nk
     dev = m2d.device
-    # one allocation for the six index arrays (each part 16-byte aligned)
-    rp = (nq + 1 + 3) & ~3
-    idx = torch.empty(3 * rp + 3 * tiles, dtype=torch.int32, device=dev)
-    frp, prp, lrp = idx[0:nq + 1], idx[rp:rp + nq + 1], idx[2 * rp:2 * rp + nq + 1]
-    fci, pci, lci = (idx[3 * rp + i * tiles:3 * rp + (i + 1) * tiles] for i in range(3))
+    # one allocation for the six index arrays, cut up by one call
+    idx = torch.empty(3 * (nq + 1) + 3 * tiles, dtype=torch.int32, device=dev)
+    frp, prp, lrp, fci, pci, lci = idx.split((nq + 1, nq + 1, nq + 1, tiles, tiles, tiles))
     bits = torch.empty((tiles, 64), dtype=torch.int64, device=dev) if (want_bits and bm == 64 and bn == 64) else None
     lib = _lib.lib()
-    # The workspace ends with the mask's non-zero count (8 bytes + 8 spare); the four list counts are
-    # placed right behind it, so that one device -> host read of 32 bytes brings all of them.
+    # The workspace ends with the mask's non-zero count (int64), that count as the reference's percentage
+    # (float32) and 4 spare bytes; the four list counts are placed right behind it, so that one device ->
+    # host read of 32 bytes brings all of them.
     wbytes = lib.stof_build_lut_workspace_bytes(n, bm, bn)
     ws = torch.empty(wbytes + 16, dtype=torch.uint8, device=dev)
-    counts = ws[wbytes - 16:].view(torch.int64)          # [nnz, spare, n_full | n_part << 32, n_load | overflow << 32]
+    counts = ws[wbytes - 16:].view(torch.int64)          # [nnz, nnz % as float32 | spare, n_full | n_part << 32, n_load | overflow << 32]
     _lib.check(lib.stof_build_lut(m2d.data_ptr(), m2d.element_size(), m2d.stride(0), n, bm, bn,
                                   frp.data_ptr(), fci.data_ptr(), prp.data_ptr(), pci.data_ptr(), lrp.data_ptr(), lci.data_ptr(),
                                   bits.data_ptr() if bits is not None else None, ws.data_ptr() + wbytes,
@@ -197,7 +196,7 @@ def _get_sparse_storage_device(m2d, bm, bn):
                                                        _stream(m2d.device)), "stof_lut_additive_blocks")
         if bits is not None:   # the attention operator finds the bit rows of these blocks already packed
             setattr(pbm, BITS_ATTR, (content_key(pbm), bits[:n_part]))
-    return nonzero, (frp, fci, prp, pci, pbm, lrp, lci)
+    return nonzero, counts, (frp, fci, prp, pci, pbm, lrp, lci)
 
 
 def get_sparse_storage(Mask, block_size_m, block_size_n):
@@ -217,9 +216,12 @@ def get_sparse_storage(Mask, block_size_m, block_size_n):
     if _device_path(Mask, block_size_m, block_size_n):
         # the non-zero count of batch 0 comes out of the classification pass; further batches (which the
         # LUT ignores, but the reference's figure counts) are counted by torch
-        nonzero, lut = _get_sparse_storage_device(Mask[0], block_size_m, block_size_n)
-        if Mask.shape[0] > 1:
-            nonzero += int(torch.count_nonzero(Mask[1:]))
+        nonzero, counts, lut = _get_sparse_storage_device(Mask[0], block_size_m, block_size_n)
+        if Mask.shape[0] == 1:
+            # the kernel has left the figure on the device in the reference's own arithmetic (a view of the
+            # 32-byte counts block at the workspace's end: no host -> device copy for one number)
+            return (counts.view(torch.float32)[2],) + lut
+        nonzero += int(torch.count_nonzero(Mask[1:]))
         import numpy as np
         # (the reference's arithmetic: an int64 count / int * int in float32, src/util/masks.py:137)
         nnz = torch.tensor(float(np.float32(nonzero) / np.float32(n * n) * np.float32(100)), device=Mask.device)
@@ -270,7 +272,7 @@ def get_sparse_storage_batched(Mask, block_size_m, block_size_n):
     on_device = _device_path(Mask, block_size_m, block_size_n)
     for b in range(B):
         if on_device:
-            _, (frp, fci, prp, pci, pbm_b, lrp, lci) = _get_sparse_storage_device(Mask[b], block_size_m, block_size_n)
+            _, _, (frp, fci, prp, pci, pbm_b, lrp, lci) = _get_sparse_storage_device(Mask[b], block_size_m, block_size_n)
         else:
             blocks, full, part = _classify(Mask[b], block_size_m, block_size_n)
             frp, fci = _csr(full); prp, pci = _csr(part); lrp, lci = _csr(full | part)
