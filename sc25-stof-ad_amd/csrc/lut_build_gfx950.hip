@@ -55,25 +55,50 @@ __device__ __forceinline__ half_t additive_of(half_t x) {
 // before the first compare): updates the two "every element is ..." votes and returns the keep
 // bits (bit e = element e allowed, by the rule the bit rows are packed with elsewhere: additive
 // value above -5000).
+// Flag words of a lane over the elements it has looked at, kept as integers (a test per element on
+// the bit patterns costs half the instructions of float compares and per-lane booleans):
+//   nz   OR of the patterns without their sign bits  -> non-zero iff some element is not +-0
+//   ne1  OR of (pattern XOR pattern of 1.0)          -> non-zero iff some element is not 1.0
+//   cnt  non-zero elements (fp16: two 16-bit counters side by side, at most 64 x 2 per lane and call site)
+struct ChunkFlags { uint32_t nz, ne1, cnt; };
+
 template <typename T>
-__device__ __forceinline__ uint32_t chunk_bits(const T* src, bool& not_one, bool& not_zero, int& nonzero) {
+__device__ __forceinline__ uint32_t chunk_bits(const T* src, ChunkFlags& fl) {
   constexpr int E = 16 / (int)sizeof(T);      // elements per 16-byte load
   constexpr int L = 8 / E;                    // loads per eight elements
   typedef T vec_t __attribute__((ext_vector_type(E)));
+  typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+  typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
   vec_t x[L];
 #pragma unroll
   for (int l = 0; l < L; ++l) x[l] = *reinterpret_cast<const vec_t*>(src + l * E);
   uint32_t cb = 0;
 #pragma unroll
-  for (int l = 0; l < L; ++l)
+  for (int l = 0; l < L; ++l) {
+    const u32x4 d = __builtin_bit_cast(u32x4, x[l]);
 #pragma unroll
-    for (int e = 0; e < E; ++e) {
-      const float f = (float)x[l][e];
-      not_one |= f != 1.0f;
-      not_zero |= f != 0.0f;
-      nonzero += f != 0.0f;
-      cb |= (uint32_t)((float)additive_of((half_t)x[l][e]) > -5000.0f) << (l * E + e);
+    for (int w = 0; w < 4; ++w) {
+      if constexpr (sizeof(T) == 2) {
+        const uint32_t a = d[w] & 0x7FFF7FFFu;            // two halves without their signs
+        fl.nz |= a;
+        fl.ne1 |= d[w] ^ 0x3C003C00u;
+        const u16x2 one = {1, 1};
+        const u16x2 a2 = __builtin_bit_cast(u16x2, a);
+        const u16x2 m = __builtin_elementwise_min(a2, one);   // 1 per non-zero half
+        fl.cnt = __builtin_bit_cast(uint32_t, (u16x2)(__builtin_bit_cast(u16x2, fl.cnt) + m));
+      } else {
+        const uint32_t a = d[w] << 1;                     // the pattern without its sign
+        fl.nz |= a;
+        fl.ne1 |= d[w] ^ 0x3F800000u;
+        fl.cnt += a != 0u;
+      }
     }
+#pragma unroll
+    for (int e = 0; e < E; ++e)
+      // (allowed = the additive value -10000 * (1 - x), formed in fp16, is above -5000: for every fp16 x
+      // that is the same as x > 0.5, checked over all 65536 patterns; NaN is not allowed either way)
+      cb |= (uint32_t)((half_t)x[l][e] > (half_t)0.5f) << (l * E + e);
+  }
   return cb;
 }
 
@@ -85,8 +110,7 @@ __global__ __launch_bounds__(256) void lut_classify_kernel(const LutParams p) {
   if (tile >= (int64_t)p.nQ * p.nK) return;
   const int r = (int)(tile / p.nK), c = (int)(tile - (int64_t)r * p.nK);
   const T* base = reinterpret_cast<const T*>(p.mask) + (int64_t)r * p.bm * p.ld + (int64_t)c * p.bn;
-  bool not_one = false, not_zero = false;
-  int nonzero = 0;   // this lane's share of the tile's non-zero elements (summed over the wave at the end)
+  ChunkFlags fl = {0u, 0u, 0u};   // this lane's share of the tile (merged over the wave at the end)
   if (p.ws_bits) {
     // 64 x 64 tile: 8 lanes hold one row of 64 keys, a pass covers 8 rows, 8 passes.  (fp32 read
     // four elements per lane at first: twice the passes and lane exchanges for the same bytes,
@@ -96,7 +120,7 @@ __global__ __launch_bounds__(256) void lut_classify_kernel(const LutParams p) {
     uint64_t words[PASSES];   // lanes with chunk 0: the bit row of (pass, row_in_pass)
 #pragma unroll
     for (int ps = 0; ps < PASSES; ++ps) {
-      const uint32_t cb = chunk_bits<T>(base + (int64_t)(ps * ROWS + row_in_pass) * p.ld + ch * 8, not_one, not_zero, nonzero);
+      const uint32_t cb = chunk_bits<T>(base + (int64_t)(ps * ROWS + row_in_pass) * p.ld + ch * 8, fl);
       const int sh = ch * 8;
       uint32_t lo = sh < 32 ? cb << sh : 0u, hi = sh >= 32 ? cb << (sh - 32) : 0u;
 #pragma unroll
@@ -106,7 +130,7 @@ __global__ __launch_bounds__(256) void lut_classify_kernel(const LutParams p) {
       }
       words[ps] = ((uint64_t)hi << 32) | lo;
     }
-    const bool full = __ballot(not_one) == 0ull, empty = __ballot(not_zero) == 0ull;
+    const bool full = __ballot(fl.ne1 != 0u) == 0ull, empty = __ballot(fl.nz != 0u) == 0ull;
     if (lane == 0) p.cls[tile] = (unsigned char)(empty ? kClsEmpty : (full ? kClsFull : kClsPart));
     if (!full && !empty && ch == 0) {
 #pragma unroll
@@ -117,12 +141,13 @@ __global__ __launch_bounds__(256) void lut_classify_kernel(const LutParams p) {
     const int total = p.bm * cpr;
     for (int idx = lane; idx < total; idx += 64) {
       const int row = idx / cpr, ch = idx - row * cpr;
-      chunk_bits<T>(base + (int64_t)row * p.ld + ch * 8, not_one, not_zero, nonzero);
+      chunk_bits<T>(base + (int64_t)row * p.ld + ch * 8, fl);
     }
-    const bool full = __ballot(not_one) == 0ull, empty = __ballot(not_zero) == 0ull;
+    const bool full = __ballot(fl.ne1 != 0u) == 0ull, empty = __ballot(fl.nz != 0u) == 0ull;
     if (lane == 0) p.cls[tile] = (unsigned char)(empty ? kClsEmpty : (full ? kClsFull : kClsPart));
   }
   if (p.cnt) {   // (at most 128 x 128 = 16384 per tile)
+    int nonzero = sizeof(T) == 2 ? (int)((fl.cnt & 0xFFFFu) + (fl.cnt >> 16)) : (int)fl.cnt;
     for (int o = 32; o > 0; o >>= 1) nonzero += __shfl_xor(nonzero, o, 64);
     if (lane == 0) p.cnt[tile] = (unsigned short)nonzero;
   }

@@ -136,3 +136,34 @@ def test_nnz_counts_every_batch_and_any_non_zero_value():
         want = om.get_sparse_storage(m.numpy(), 32, 64)
         assert np.float32(float(got[0])) == np.float32(float(want[0])), (float(got[0]), float(want[0]))
         assert got[0].device.type == "cuda"
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
+def test_values_other_than_zero_and_one(dtype):
+    """The classification is by value (a tile is FULL iff every element == 1, absent iff every element == 0)
+    and the bit rows follow the additive rule (-10000 * (1 - x) in fp16 above -5000): -0.0, values around
+    0.5 and 1, large, negative, infinite and NaN entries must come out as the oracle and the packed additive
+    blocks have them; the non-zero count takes every value that is not +-0."""
+    S = 256
+    g = torch.Generator().manual_seed(17)
+    m = (torch.rand(S, S, generator=g) < 0.5).float()
+    m[:64, :64] = 1.0; m[:64, 64:128] = 0.0; m[64:128, :64] = -0.0        # a full, an empty and a minus-zero tile
+    m[64:128, 64:128] = 1.0; m[70, 70] = 1.0 + 2.0 ** -10                   # all ones but one element just above
+    m[128:192, 0:64] = 0.0; m[130, 3] = 2.0 ** -20                          # all zeros but one tiny element
+    odd = [0.5, 0.5 + 2.0 ** -11, 0.5 - 2.0 ** -12, 0.25, 0.75, 2.0, -1.0, 60000.0, float("inf"), float("-inf"), float("nan"), -0.0, 1e-7]
+    for i, val in enumerate(odd):
+        m[200 + i, 130 + 3 * i] = val
+    dev_mask = m.to(dtype)[None].cuda()
+    got = pm.get_sparse_storage(dev_mask, 64, 64)
+    with np.errstate(over="ignore"):   # (60000 and inf overflow the additive form on purpose)
+        want = om.get_sparse_storage(m.to(dtype).float()[None].numpy(), 64, 64)     # (the oracle sees the values the device holds)
+    for i in (1, 2, 3, 4, 6, 7):
+        assert np.array_equal(got[i].cpu().numpy(), want[i]), f"list {i} differs"
+    assert np.float32(float(got[0])) == np.float32(float(want[0]))
+    pbm = got[5].cpu().numpy()
+    both_nan = np.isnan(pbm) & np.isnan(want[5])          # (a NaN's sign and payload are not part of the contract)
+    differ = (pbm.view(np.uint16) != want[5].view(np.uint16)) & ~both_nan
+    assert not differ.any(), f"additive blocks differ at {np.argwhere(differ)[:5].tolist()}: {pbm[differ][:5]} vs {want[5][differ][:5]}"
+    bits = getattr(got[5], BITS_ATTR, None)
+    assert bits is not None
+    assert np.array_equal(bits[1].cpu().numpy().view(np.uint64), _bit_rows(pbm)), "bit rows differ from the additive rule"
