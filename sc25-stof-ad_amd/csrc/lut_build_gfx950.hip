@@ -39,7 +39,7 @@ struct LutParams {
   const void* mask; int64_t ld;           // row pitch in elements
   int S, bm, bn, nQ, nK;
   unsigned char* cls; uint64_t* ws_bits;  // scratch: class byte per tile; 64 bit rows per tile (64 x 64 only, else null)
-  unsigned short* cnt; long long* nnz;    // scratch: non-zero elements per tile (or null); their sum, written by the last row's workgroup
+  unsigned short* cnt; long long* nnz;    // scratch: non-zero elements per tile (or null); their sum, written by the first row's workgroup
   int32_t* frp; int32_t* fci; int32_t* prp; int32_t* pci; int32_t* lrp; int32_t* lci;
   uint64_t* pbits;                        // [cap_part][64] or null
   int32_t* counts;                        // {n_full, n_part, n_load, overflow} or null
@@ -218,8 +218,9 @@ __global__ __launch_bounds__(256) void lut_compact_kernel(const LutParams p) {
     fbase += f_all; pbase += p_all;
     __syncthreads();
   }
-  if (r == p.nQ - 1 && p.cnt && p.nnz) {
+  if (r == 0 && p.cnt && p.nnz) {
     // the mask's non-zero elements: the per-tile counts of the classify pass, summed by this one workgroup
+    // (that of the first row of tiles, which has no rows above it to count: the last row's has the most)
     long long total = 0;
     const int64_t tiles = (int64_t)p.nQ * p.nK;
     // eight counts per 16-byte load (the count array starts 16-byte aligned), all of a thread's loads independent
