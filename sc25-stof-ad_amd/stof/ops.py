@@ -21,7 +21,7 @@ from ._cache import (BITS_ATTR as _BITS_ATTR, DEVICE_BUILT_ATTR as _DEVICE_BUILT
                      content_key as _content_key)
 from ._lib import StofError, check, strides3
 
-__all__ = ["block_attn", "block_attn_packed_qkv", "rowwise_attn", "block_attn_mask_op", "rowwise_attn_full_op", "rowwise_attn_sliding_op",
+__all__ = ["block_attn", "BoundAttention", "block_attn_packed_qkv", "rowwise_attn", "block_attn_mask_op", "rowwise_attn_full_op", "rowwise_attn_sliding_op",
            "rowwise_attn_mask_op", "pack_mask_bits", "set_attention_launch_form", "StofError"]
 
 
@@ -314,7 +314,7 @@ def _check_i32(name, t, device):
 
 
 def block_attn(q, k, v, lut, block_m=64, block_n=64, out=None, out_layout="bhsd", softmax_scale=None,
-               launch_form=None, revalidate=False, use_plan=True):
+               launch_form=None, revalidate=False, use_plan=True, _bind=None):
     """Block-masked attention.  q, k, v: fp16 (or, all three, bfloat16) views ``[B,H,S,D]`` with
     unit stride in D (any other strides).  ``lut`` = (full_row_ptr, full_col_idx, part_row_ptr, part_col_idx,
     part_block_mask, load_row_ptr, load_col_idx) as returned by ``get_sparse_storage`` (the
@@ -363,15 +363,37 @@ def block_attn(q, k, v, lut, block_m=64, block_n=64, out=None, out_layout="bhsd"
         raise StofError(f"unknown out_layout {out_layout!r}")
     if out.dtype != q.dtype or out.device != dev:
         raise StofError("out must have q's dtype and device")
-    return _attn_launch(q.data_ptr(), k.data_ptr(), v.data_ptr(), out, _lib.i64x3(qs[0], qs[1], qs[2]),
-                        _lib.i64x3(ks[0], ks[1], ks[2]), _lib.i64x3(vs[0], vs[1], vs[2]), ostr, B, H, S, D, dt, dev,
-                        lut, block_m, block_n, softmax_scale, launch_form, revalidate, use_plan)
+    if _bind is None:
+        return _attn_launch(q.data_ptr(), k.data_ptr(), v.data_ptr(), out, _lib.i64x3(qs[0], qs[1], qs[2]),
+                            _lib.i64x3(ks[0], ks[1], ks[2]), _lib.i64x3(vs[0], vs[1], vs[2]), ostr, B, H, S, D, dt, dev,
+                            lut, block_m, block_n, softmax_scale, launch_form, revalidate, use_plan)
+    # BoundAttention: the arguments are kept, and the first launch happens with them
+    _bind._args = _attn_args(q.data_ptr(), k.data_ptr(), v.data_ptr(), out, _lib.i64x3(qs[0], qs[1], qs[2]),
+                             _lib.i64x3(ks[0], ks[1], ks[2]), _lib.i64x3(vs[0], vs[1], vs[2]), ostr, B, H, S, D, dt, dev,
+                             lut, block_m, block_n, softmax_scale, launch_form, revalidate, use_plan)
+    check(_lib.lib().stof_block_attn_fwd_planned(*_bind._args, _stream(dev)), "stof_block_attn_fwd")
+    return out
+
+
+def _attn_args(qp, kp, vp, out, qstr, kstr, vstr, ostr, B, H, S, D, dt, dev, lut, block_m, block_n,
+               softmax_scale, launch_form, revalidate, use_plan):
+    """The LUT side of an attention call (prepared data, plan): every argument of
+    stof_block_attn_fwd_planned but the stream.  q, k, v arrive as validated device addresses with
+    their (batch, head, row) element strides."""
+    form = _form(launch_form)
+    if revalidate:
+        _drop_caches(lut)
+    lut_ptrs, lut_bs, plans = _prepared_lut(lut, B, S, block_m, block_n, dev)
+    scale = softmax_scale if softmax_scale is not None else 1.0 / math.sqrt(D)
+    plan_ptr, plan_bytes, plan_rows = _plan(plans, lut_ptrs, lut_bs, B, H, S, form, dev) if use_plan else (None, 0, 0)
+    return (qp, kp, vp, out.data_ptr(), *lut_ptrs, 64, 64, scale, qstr, kstr, vstr, ostr,
+            B, S, H, D, dt, lut_bs, form, plan_ptr, plan_bytes, plan_rows)
 
 
 def _attn_launch(qp, kp, vp, out, qstr, kstr, vstr, ostr, B, H, S, D, dt, dev, lut, block_m, block_n,
                  softmax_scale, launch_form, revalidate, use_plan):
-    """The LUT side of an attention call (prepared data, plan) and the launch; q, k, v arrive as
-    validated device addresses with their (batch, head, row) element strides."""
+    """The LUT side of an attention call and the launch (as _attn_args, spelled out once more: this
+    is the per-call path and a tuple built and taken apart again shows in its cost)."""
     form = _form(launch_form)
     if revalidate:
         _drop_caches(lut)
@@ -382,6 +404,34 @@ def _attn_launch(qp, kp, vp, out, qstr, kstr, vstr, ostr, B, H, S, D, dt, dev, l
         qp, kp, vp, out.data_ptr(), *lut_ptrs, 64, 64, scale, qstr, kstr, vstr, ostr,
         B, S, H, D, dt, lut_bs, form, plan_ptr, plan_bytes, plan_rows, _stream(dev)), "stof_block_attn_fwd")
     return out
+
+
+class BoundAttention:
+    """``block_attn`` on fixed buffers with everything that does not change between calls resolved
+    once: a serving loop that keeps q, k, v and the output in place (the way a captured graph does,
+    for callers that cannot capture one) then pays the binding and the launch per call and none of
+    the per-call validation, stride extraction and LUT look-up.
+
+        run = BoundAttention(q, k, v, lut, out=out)      # validates, prepares the LUT, lays out the walk
+        ...                                              # new contents written INTO q, k, v
+        run()                                            # one launch on the current stream; returns out
+
+    The addresses, shapes and strides of the four tensors and the LUT's prepared form are taken at
+    construction and kept alive by this object.  Writing new values into the tensors is what it is
+    for; re-allocating or resizing them, or changing the LUT, needs a new BoundAttention."""
+
+    def __init__(self, q, k, v, lut, block_m=64, block_n=64, out=None, out_layout="bhsd", softmax_scale=None,
+                 launch_form=None, use_plan=True):
+        self._args = None
+        self.out = block_attn(q, k, v, lut, block_m, block_n, out, out_layout, softmax_scale, launch_form,
+                              use_plan=use_plan, _bind=self)
+        self._keep = (q, k, v, lut, getattr(lut[6], _LUT_READY_ATTR, None))   # what the addresses point into
+        self._dev = q.device
+        self._fn = _lib.lib().stof_block_attn_fwd_planned
+
+    def __call__(self):
+        check(self._fn(*self._args, _stream(self._dev)), "stof_block_attn_fwd")
+        return self.out
 
 
 def block_attn_packed_qkv(qkv, n_heads, lut, block_m=64, block_n=64, out=None, softmax_scale=None,

@@ -320,3 +320,24 @@ def test_example_script_runs(mask):
     assert r.returncode == 0, r.stdout + r.stderr
     line = [l for l in r.stdout.splitlines() if l.startswith("max abs difference")][0]
     assert float(line.split(":")[1]) < 5e-3, r.stdout
+
+
+def test_bound_attention_on_fixed_buffers():
+    """BoundAttention: arguments resolved once, then launches on new contents of the same tensors give
+    what block_attn gives (bit for bit: the same kernel on the same arguments), in both output layouts."""
+    from stof.ops import BoundAttention
+    B, H, S = 2, 3, 512
+    mask = configs.mask_c1(S)
+    lut = pm.get_sparse_storage(mask.float()[None].cuda(), 64, 64)[1:]
+    q, k, v = _inputs(B, H, S, seed=21)
+    for layout in ("bhsd", "bshd"):
+        out = torch.empty((B, H, S, 64) if layout == "bhsd" else (B, S, H * 64), dtype=torch.float16, device="cuda")
+        run = BoundAttention(q, k, v, lut, out=out, out_layout=layout)
+        assert run.out is out
+        assert torch.equal(out, block_attn(q, k, v, lut, out_layout=layout))           # the constructor's launch
+        q2, k2, v2 = _inputs(B, H, S, seed=22)
+        q.copy_(q2); k.copy_(k2); v.copy_(v2)                                           # new contents, same buffers
+        got = run()
+        assert got is out
+        assert torch.equal(out, block_attn(q2, k2, v2, lut, out_layout=layout))
+    _close(block_attn(q, k, v, lut), _oracle(q, k, v, mask), "bound attention inputs")
