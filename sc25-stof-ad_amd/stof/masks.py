@@ -18,6 +18,10 @@ import random
 
 import torch
 
+from . import _lib
+from ._cache import BITS_ATTR, DEVICE_BUILT_ATTR, LUT_OK_ATTR, content_key
+from .ops import _stream
+
 NEG_MASK = -10000.0
 
 
@@ -144,8 +148,6 @@ def _device_path(Mask, bm, bn):
 def _build_on_device(m2d, bm, bn, want_bits):
     """One sample's mask [S,S] on the GPU -> (row pointers x3, column lists x3 at full capacity,
     bit rows or None, counts tensor).  No synchronisation: everything stays on the device."""
-    from . import _lib
-    from .ops import _stream
     if m2d.stride(1) != 1 or (m2d.stride(0) * m2d.element_size()) % 16 or m2d.data_ptr() % 16:
         m2d = m2d.contiguous()
     n = m2d.shape[-1]
@@ -179,9 +181,6 @@ def _read_counts(counts):
 def _get_sparse_storage_device(m2d, bm, bn):
     """The seven LUT tensors of one sample, exactly shaped, built by the GPU kernels (one
     device -> host read of the three list lengths)."""
-    from . import _lib
-    from ._cache import BITS_ATTR, content_key
-    from .ops import _stream
     m2d, frp, fci, prp, pci, lrp, lci, bits, counts = _build_on_device(m2d, bm, bn, want_bits=True)
     nonzero, n_full, n_part, n_load, overflow = _read_counts(counts)
     assert not overflow
@@ -246,7 +245,6 @@ def build_lut_device(Mask, block_size_m=64, block_size_n=64):
     full capacity (entries beyond the last row pointer are unused) and ``part_block_mask`` is a
     one-block placeholder that carries the partial tiles' packed bit rows, which is what the
     attention kernel reads.  64 x 64 blocks only."""
-    from ._cache import BITS_ATTR, DEVICE_BUILT_ATTR, LUT_OK_ATTR, content_key
     if not _device_path(Mask, block_size_m, block_size_n) or (block_size_m, block_size_n) != (64, 64):
         raise ValueError("build_lut_device needs an fp16 / fp32 [B,S,S] mask on the GPU and 64 x 64 blocks")
     _, frp, fci, prp, pci, lrp, lci, bits, _ = _build_on_device(Mask[0], 64, 64, want_bits=True)
